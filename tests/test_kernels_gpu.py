@@ -1,0 +1,273 @@
+"""Each HIP kernel alone against a plain float64/float32 torch formula of the same
+operation, at sizes other than the tiny engines' (odd widths, many heads, long rows)."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _tol(dtype):
+    # float32 kernels: a few ulp of accumulated 32-bit rounding; bfloat16: one bf16 rounding
+    # of the result (2^-8 relative) plus accumulated input rounding.
+    return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=2e-3)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from torchlet_amd.kernels import ops
+    return ops
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,H,T", [(300, 96, 7), (1031, 3584, 33)])
+def test_embedding(ops, dtype, V, H, T):
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(V, H, generator=g).to(dtype).cuda()
+    ids = torch.randint(0, V, (T,), generator=g, dtype=torch.int32).cuda()
+    out = torch.empty(T, H, dtype=torch.float32, device="cuda")
+    ops.embedding(ids, table, out)
+    assert torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("wdtype", DTYPES)
+@pytest.mark.parametrize("T,H,eps", [(5, 96, 1e-5), (19, 1000, 1e-6), (3, 5120, 1e-6)])
+def test_add_rmsnorm(ops, dtype, wdtype, T, H, eps):
+    if dtype == torch.float32 and wdtype == torch.bfloat16:
+        pytest.skip("a 32-bit engine widens its vectors")
+    g = torch.Generator().manual_seed(1)
+    res = (torch.randn(T, H, generator=g) * 3).cuda()
+    pend = torch.randn(T, H, generator=g).to(dtype).cuda()
+    w = (1 + 0.1 * torch.randn(H, generator=g)).to(wdtype).cuda()
+    ref_r = res.double() + pend.double()
+    ref = ref_r * torch.rsqrt(ref_r.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    # with pending: residual updated
+    r1 = res.clone()
+    out = torch.empty(T, H, dtype=dtype, device="cuda")
+    ops.add_rmsnorm(r1, pend, w, eps, out)
+    torch.testing.assert_close(r1.double(), ref_r, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(out.double(), ref, **_tol(dtype))
+    # without pending: residual untouched
+    r2 = res.clone()
+    ops.add_rmsnorm(r2, None, w, eps, out)
+    assert torch.equal(r2, res)
+    ref2 = res.double() * torch.rsqrt(res.double().pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    torch.testing.assert_close(out.double(), ref2, **_tol(dtype))
+    # selected rows: nothing written back
+    rows = torch.tensor([T - 1, 0, T - 1], dtype=torch.int32, device="cuda")
+    r3 = res.clone()
+    out3 = torch.empty(3, H, dtype=dtype, device="cuda")
+    ops.add_rmsnorm(r3, pend, w, eps, out3, rows)
+    assert torch.equal(r3, res)
+    torch.testing.assert_close(out3.double(), ref[rows.long()], **_tol(dtype))
+
+
+def test_rmsnorm_zero_row_is_zero_not_nan(ops):
+    res = torch.zeros(2, 64, device="cuda")
+    w = torch.ones(64, device="cuda")
+    out = torch.full((2, 64), 7.0, device="cuda")
+    ops.add_rmsnorm(res, None, w, 1e-6, out)
+    assert torch.equal(out, torch.zeros_like(out))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K,bias", [(1, 300, 96, True), (7, 129, 200, False), (65, 64, 17, True), (130, 513, 1000, True)])
+def test_linear(ops, dtype, M, N, K, bias):
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(M, K, generator=g).to(dtype).cuda()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype).cuda()
+    b = torch.randn(N, generator=g).to(dtype).cuda() if bias else None
+    ref = x.double() @ w.double().T + (b.double() if bias else 0)
+    # A 32-bit sum of K products of size ~rms/sqrt(K) carries a rounding error of about
+    # eps * sqrt(K) * rms (random walk); 8 of those bound the largest of ~1e5 elements.
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    out = torch.empty(M, N, dtype=dtype, device="cuda")
+    ops.linear(x, w, b, out)
+    torch.testing.assert_close(out.double(), ref, **(tol32 if dtype == torch.float32 else _tol(dtype)))
+    out32 = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    ops.linear(x, w, b, out32)
+    torch.testing.assert_close(out32.double(), ref, **tol32)
+    # a strided input view (columns of a wider buffer)
+    wide = torch.zeros(M, K + 24, dtype=dtype, device="cuda")
+    wide[:, 8:8 + K] = x
+    ops.linear(wide[:, 8:8 + K], w, b, out32)
+    torch.testing.assert_close(out32.double(), ref, **tol32)
+
+
+def _rope_ref(x, pos, theta):
+    """x [T, heads, hd] float64; split-half pairing."""
+    hd = x.shape[-1]
+    j = torch.arange(0, hd, 2, dtype=torch.float32)
+    inv = 1.0 / (theta ** (j / hd))
+    ang = torch.outer(pos.float(), inv).double()
+    c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+    x1, x2 = x[..., : hd // 2], x[..., hd // 2:]
+    return torch.cat((x1 * c - x2 * s, x2 * c + x1 * s), dim=-1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,page,theta", [(4, 2, 16, 16, 1e4), (3, 1, 32, 8, 1e6), (28, 4, 128, 16, 1e6), (5, 5, 48, 4, 5e5)])
+def test_rope_cache_write(ops, dtype, nh, nkv, hd, page, theta):
+    g = torch.Generator().manual_seed(3)
+    lens, ctxs = [5, 1, 11], [0, 37, 6]           # three requests: new tokens, cached before
+    T = sum(lens)
+    max_blocks = (max(a + b for a, b in zip(lens, ctxs)) + page - 1) // page
+    pages = 3 * max_blocks + 2
+    qkv = torch.randn(T, (nh + 2 * nkv) * hd, generator=g).to(dtype)
+    positions = torch.cat([torch.arange(c, c + n) for n, c in zip(lens, ctxs)]).int()
+    token_req = torch.cat([torch.full((n,), r) for r, n in enumerate(lens)]).int()
+    perm = torch.randperm(pages - 1, generator=g)[: 3 * max_blocks] + 1
+    bt = perm.view(3, max_blocks).int()
+    j = torch.arange(0, hd, 2, dtype=torch.float32)
+    inv_freq = (1.0 / (theta ** (j / hd)))
+    kp = torch.zeros(pages, nkv, page, hd, dtype=dtype)
+    vp = torch.zeros_like(kp)
+    d_qkv, d_kp, d_vp = qkv.cuda(), kp.cuda(), vp.cuda()
+    ops.rope_cache_write(d_qkv, nh, nkv, hd, nh + nkv, positions.cuda(), inv_freq.cuda(), token_req.cuda(), bt.cuda(), d_kp, d_vp, page)
+    x = qkv.double().view(T, nh + 2 * nkv, hd)
+    ref_qk = _rope_ref(x[:, : nh + nkv], positions, theta)
+    got = d_qkv.cpu().double().view(T, nh + 2 * nkv, hd)
+    torch.testing.assert_close(got[:, : nh + nkv], ref_qk, **_tol(dtype))
+    assert torch.equal(got[:, nh + nkv:], x[:, nh + nkv:])
+    kref = torch.zeros(pages, nkv, page, hd, dtype=torch.float64)
+    vref = torch.zeros_like(kref)
+    for t in range(T):
+        p = int(positions[t]); pg = int(bt[token_req[t], p // page])
+        kref[pg, :, p % page] = got[t, nh: nh + nkv]       # the rotated k as stored in place
+        vref[pg, :, p % page] = x[t, nh + nkv:]
+    assert torch.equal(d_kp.cpu().double(), kref)
+    assert torch.equal(d_vp.cpu().double(), vref)
+    assert float(d_kp[0].abs().sum()) == 0.0                # page 0 is never written
+
+
+def _attention_ref(q, k, v, window):
+    """One request: q [n, heads, hd] at positions ctx..ctx+n-1, k/v [ctx+n, kvh, hd] (float64)."""
+    n, heads, hd = q.shape
+    total, kvh, _ = k.shape
+    ctx = total - n
+    group = heads // kvh
+    kk = k.repeat_interleave(group, dim=1)
+    vv = v.repeat_interleave(group, dim=1)
+    s = torch.einsum("nhd,thd->hnt", q, kk) / math.sqrt(hd)
+    qpos = ctx + torch.arange(n)[:, None]
+    kpos = torch.arange(total)[None, :]
+    hide = kpos > qpos
+    if window:
+        hide = hide | (kpos <= qpos - window)
+    s = s.masked_fill(hide[None], -torch.inf)
+    return torch.einsum("hnt,thd->nhd", torch.softmax(s, -1), vv)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,page,window,splits", [
+    (4, 2, 16, 16, 0, 1), (3, 1, 32, 8, 0, 1), (28, 4, 128, 16, 0, 3), (6, 6, 48, 4, 0, 1),
+    (20, 1, 64, 16, 0, 2), (4, 2, 16, 16, 13, 1), (8, 2, 80, 32, 29, 4), (2, 1, 256, 16, 0, 1),
+])
+def test_paged_attention(ops, dtype, nh, nkv, hd, page, window, splits):
+    g = torch.Generator().manual_seed(4)
+    lens, ctxs = [37, 1, 9, 1], [0, 150, 70, 0]      # a whole prompt, a decode, a portion, a first token
+    R, T = len(lens), sum(lens)
+    totals = [a + b for a, b in zip(lens, ctxs)]
+    max_blocks = (max(totals) + page - 1) // page + 1
+    pages = R * max_blocks + 1
+    bt = (torch.randperm(pages - 1, generator=g)[: R * max_blocks] + 1).view(R, max_blocks).int()
+    q = torch.randn(T, nh * hd, generator=g).to(dtype)
+    kp = torch.randn(pages, nkv, page, hd, generator=g).to(dtype)      # stale pages hold noise, not zeros
+    vp = torch.randn(pages, nkv, page, hd, generator=g).to(dtype)
+    ks, vs = [], []
+    for r in range(R):
+        k = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
+        v = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
+        if r == 0:
+            k[3] *= 4.0        # a far key stands out: dropping it changes the result visibly
+        for p in range(totals[r]):
+            kp[bt[r, p // page], :, p % page] = k[p]
+            vp[bt[r, p // page], :, p % page] = v[p]
+        ks.append(k); vs.append(v)
+    indptr = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    tq = ops.attention_tile_tokens(nh, nkv)
+    tile_req, tile_tok0 = [], []
+    for r, n in enumerate(lens):
+        for t0 in range(0, n, tq):
+            tile_req.append(r); tile_tok0.append(t0)
+    out = torch.empty(T, nh * hd, dtype=dtype, device="cuda")
+    # q lives inside a wider row, as in the fused projection
+    wide = torch.zeros(T, nh * hd + 32, dtype=dtype, device="cuda")
+    wide[:, : nh * hd] = q.cuda()
+    ops.paged_attention(wide[:, : nh * hd], out, kp.cuda(), vp.cuda(), bt.cuda(), indptr.cuda(),
+                        torch.tensor(ctxs, dtype=torch.int32).cuda(), torch.tensor(tile_req, dtype=torch.int32).cuda(),
+                        torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq, nh, nkv, hd, page, window,
+                        1.0 / math.sqrt(hd), splits)
+    got = out.cpu().double().view(T, nh, hd)
+    for r in range(R):
+        a, b = int(indptr[r]), int(indptr[r + 1])
+        ref = _attention_ref(q[a:b].double().view(-1, nh, hd), ks[r].double(), vs[r].double(), window)
+        torch.testing.assert_close(got[a:b], ref, **_tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(3, 200), (17, 1001)])
+def test_swiglu(ops, dtype, T, I):
+    g = torch.Generator().manual_seed(5)
+    gu = (torch.randn(T, 2 * I, generator=g) * 3).to(dtype).cuda()
+    out = torch.empty(T, I, dtype=dtype, device="cuda")
+    ops.swiglu(gu, out)
+    ref = torch.nn.functional.silu(gu[:, :I].double()) * gu[:, I:].double()
+    torch.testing.assert_close(out.double(), ref, **_tol(dtype))
+
+
+def _mix32(x):
+    x &= 0xFFFFFFFF
+    x ^= x >> 16; x = (x * 0x7FEB352D) & 0xFFFFFFFF
+    x ^= x >> 15; x = (x * 0x846CA68B) & 0xFFFFFFFF
+    x ^= x >> 16
+    return x
+
+
+def test_sample_greedy_and_ties(ops):
+    g = torch.Generator().manual_seed(6)
+    logits = torch.randn(5, 3001, generator=g)
+    logits[1, 77] = logits[1, 2900] = 50.0          # a tie: the lower index wins
+    logits[2, 3000] = 60.0                          # the last column
+    out = torch.empty(5, dtype=torch.int32, device="cuda")
+    ops.sample(logits.cuda(), None, None, out)
+    ref = logits.argmax(-1)
+    ref[1] = 77
+    assert out.cpu().tolist() == ref.tolist()
+    wide = torch.zeros(5, 3100)
+    wide[:, :3001] = logits
+    wide[:, 3001:] = 1000.0                         # beyond the vocabulary: never read
+    ops.sample(wide.cuda()[:, :3001], torch.zeros(5).cuda(), torch.arange(5, dtype=torch.int32).cuda(), out)
+    assert out.cpu().tolist() == ref.tolist()
+
+
+def test_sample_temperature_matches_formula_and_distribution(ops):
+    V = 11
+    logits = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5, 3.0, -2.0, 0.0, 1.5, 2.5, -0.5]])
+    temp = 0.8
+    n = 20000
+    keys = torch.arange(n, dtype=torch.int64)
+    keys = ((keys * 2654435761) % (1 << 32)).to(torch.int64)
+    keys_i32 = torch.where(keys >= (1 << 31), keys - (1 << 32), keys).int()
+    out = torch.empty(n, dtype=torch.int32, device="cuda")
+    ops.sample(logits.expand(n, V).contiguous().cuda(), torch.full((n,), temp).cuda(), keys_i32.cuda(), out)
+    got = out.cpu()
+    # the documented formula, for the first rows, in float64
+    for row in range(50):
+        key = int(keys[row])
+        best, besti = -math.inf, -1
+        for i in range(V):
+            r = _mix32(_mix32(key ^ i) + 0x9E3779B9)
+            u = ((r >> 8) + 0.5) / 16777216.0
+            v = float(logits[0, i]) / temp - math.log(-math.log(u))
+            if v > best:
+                best, besti = v, i
+        assert int(got[row]) == besti
+    freq = torch.bincount(got.long(), minlength=V).double() / n
+    p = torch.softmax(logits[0].double() / temp, -1)
+    # 20000 draws: standard error of a frequency is at most 0.0035; allow 4 of them
+    assert float((freq - p).abs().max()) < 0.015

@@ -1,0 +1,189 @@
+// Row-wise kernels: embedding gather, residual add + RMSNorm, rotary position
+// encoding fused with the write of keys and values into cache pages, SwiGLU gate.
+// Each is templated on the activation type (float or bfloat16); all arithmetic is float.
+#include "common.h"
+
+// ------------------------------------------------------------------ embedding
+// out[t, :] = float(table[ids[t], :]); the residual stream is 32-bit.
+template <typename T>
+__global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                 float* __restrict__ out, int hidden, int vocab) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= vocab) id = 0;  // ids are checked on the host; never read out of bounds
+    const T* src = table + (size_t)id * hidden;
+    float* dst = out + (size_t)t * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+}
+
+extern "C" int tl_embedding(const void* ids, const void* table, int table_dtype, void* out,
+                            int tokens, int hidden, int vocab, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes tokens=%d hidden=%d vocab=%d", tokens, hidden, vocab);
+    if (tokens == 0) return TL_OK;
+    dim3 grid(tokens), block(256);
+    if (table_dtype == TL_DT_F32)
+        embedding_kernel<float><<<grid, block, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab);
+    else if (table_dtype == TL_DT_BF16)
+        embedding_kernel<bf16_t><<<grid, block, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab);
+    else TL_REQUIRE(false, "embedding: unknown dtype %d", table_dtype);
+    TL_CHECK_LAUNCH("embedding");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ add + RMSNorm
+// One block per output row.  r = residual[row] (+ pending[row]); if `update`, r is
+// written back to the residual; out = r * rsqrt(mean(r^2) + eps) * weight.
+// `rows` (optional) selects the source row of each output row; then nothing is written back.
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ pending,
+                                   const void* __restrict__ weight, int weight_f32, float eps,
+                                   T* __restrict__ out, const int* __restrict__ rows, int hidden) {
+    __shared__ float red[16];
+    const int orow = blockIdx.x;
+    const int srow = rows ? rows[orow] : orow;
+    float* res = residual + (size_t)srow * hidden;
+    const T* pen = pending ? pending + (size_t)srow * hidden : nullptr;
+    const bool update = (pen != nullptr) && (rows == nullptr);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float r = res[i];
+        if (pen) r += to_float(pen[i]);
+        if (update) res[i] = r;
+        ss += r * r;
+    }
+    ss = block_sum(ss, red);
+    const float inv = rsqrtf(ss / (float)hidden + eps);
+    T* dst = out + (size_t)orow * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float r = res[i];
+        if (pen && !update) r += to_float(pen[i]);
+        dst[i] = from_float<T>(r * inv * load_vec(weight, weight_f32, i));
+    }
+}
+
+extern "C" int tl_add_rmsnorm(void* residual, const void* pending, const void* weight, int weight_f32,
+                              float eps, void* out, const void* rows, int out_rows, int hidden,
+                              int act_dtype, hipStream_t stream) {
+    TL_REQUIRE(out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d hidden=%d", out_rows, hidden);
+    if (out_rows == 0) return TL_OK;
+    dim3 grid(out_rows), block(hidden >= 2048 ? 512 : 256);
+    if (act_dtype == TL_DT_F32)
+        add_rmsnorm_kernel<float><<<grid, block, 0, stream>>>((float*)residual, (const float*)pending, weight, weight_f32, eps, (float*)out, (const int*)rows, hidden);
+    else if (act_dtype == TL_DT_BF16)
+        add_rmsnorm_kernel<bf16_t><<<grid, block, 0, stream>>>((float*)residual, (const bf16_t*)pending, weight, weight_f32, eps, (bf16_t*)out, (const int*)rows, hidden);
+    else TL_REQUIRE(false, "add_rmsnorm: unknown dtype %d", act_dtype);
+    TL_CHECK_LAUNCH("add_rmsnorm");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ RoPE + cache write
+// One block per token.  Row layout of `qkv`: [q heads | k heads | v heads], each head
+// `head_dim` wide, row stride `row_stride` elements.
+//   * rotate (inv_freq != null): the first `rot_heads` heads (q, then k) are rotated in
+//     place with the split-half pairing (j, j + head_dim/2) by angle = float(pos) * inv_freq[j].
+//   * write (k_plane != null): rotated k and raw v of the token go to the page
+//     block_table[token_req[t]][pos / page] at offset pos % page; planes are
+//     [pages, kv_heads, page, head_dim].
+template <typename T>
+__global__ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, int kv_heads,
+                                        int head_dim, int rot_heads, const int* __restrict__ positions,
+                                        const float* __restrict__ inv_freq, const int* __restrict__ token_req,
+                                        const int* __restrict__ block_table, int bt_stride,
+                                        T* __restrict__ k_plane, T* __restrict__ v_plane, int page_size) {
+    const int t = blockIdx.x;
+    const int pos = positions[t];
+    T* row = qkv + (size_t)t * row_stride;
+    const int half = head_dim / 2;
+    T* kdst = nullptr;
+    T* vdst = nullptr;
+    if (k_plane) {
+        const int page = block_table[(size_t)token_req[t] * bt_stride + pos / page_size];
+        const size_t base = ((size_t)page * kv_heads) * page_size * head_dim + (size_t)(pos % page_size) * head_dim;
+        kdst = k_plane + base;
+        vdst = v_plane + base;
+    }
+    const size_t head_step = (size_t)page_size * head_dim;  // between kv heads inside a page
+    const int pairs = (q_heads + kv_heads) * half;
+    for (int idx = threadIdx.x; idx < pairs; idx += blockDim.x) {
+        const int head = idx / half, j = idx % half;
+        T* x = row + (size_t)head * head_dim;
+        float x1 = to_float(x[j]), x2 = to_float(x[j + half]);
+        if (inv_freq && head < rot_heads) {
+            const float angle = (float)pos * inv_freq[j];
+            const float c = cosf(angle), s = sinf(angle);
+            const float y1 = x1 * c - x2 * s;
+            const float y2 = x2 * c + x1 * s;
+            x1 = y1;
+            x2 = y2;
+            x[j] = from_float<T>(x1);
+            x[j + half] = from_float<T>(x2);
+        }
+        if (kdst && head >= q_heads) {
+            T* d = kdst + (size_t)(head - q_heads) * head_step;
+            d[j] = from_float<T>(x1);
+            d[j + half] = from_float<T>(x2);
+        }
+    }
+    if (vdst) {
+        const T* v = row + (size_t)(q_heads + kv_heads) * head_dim;
+        for (int idx = threadIdx.x; idx < kv_heads * head_dim; idx += blockDim.x) {
+            const int head = idx / head_dim, d = idx % head_dim;
+            vdst[(size_t)head * head_step + d] = v[idx];
+        }
+    }
+}
+
+extern "C" int tl_rope_cache_write(void* qkv, int row_stride, int tokens, int q_heads, int kv_heads,
+                                   int head_dim, int rot_heads, const void* positions, const void* inv_freq,
+                                   const void* token_req, const void* block_table, int bt_stride,
+                                   void* k_plane, void* v_plane, int page_size, int act_dtype,
+                                   hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && q_heads >= 0 && kv_heads >= 0 && head_dim > 0 && head_dim % 2 == 0,
+               "rope_cache_write: bad sizes tokens=%d q_heads=%d kv_heads=%d head_dim=%d", tokens, q_heads, kv_heads, head_dim);
+    TL_REQUIRE(rot_heads <= q_heads + kv_heads, "rope_cache_write: rot_heads %d exceeds q+k heads", rot_heads);
+    TL_REQUIRE((k_plane == nullptr) == (v_plane == nullptr), "rope_cache_write: give both planes or none");
+    TL_REQUIRE(!k_plane || (block_table && token_req && page_size > 0 && bt_stride > 0),
+               "rope_cache_write: cache write needs block table, token_req and page size");
+    TL_REQUIRE(row_stride >= (q_heads + (k_plane ? 2 * kv_heads : kv_heads)) * head_dim,
+               "rope_cache_write: row stride %d too small", row_stride);
+    if (tokens == 0) return TL_OK;
+    dim3 grid(tokens), block(256);
+    if (act_dtype == TL_DT_F32)
+        rope_cache_write_kernel<float><<<grid, block, 0, stream>>>((float*)qkv, row_stride, q_heads, kv_heads, head_dim, rot_heads,
+            (const int*)positions, (const float*)inv_freq, (const int*)token_req, (const int*)block_table, bt_stride,
+            (float*)k_plane, (float*)v_plane, page_size);
+    else if (act_dtype == TL_DT_BF16)
+        rope_cache_write_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)qkv, row_stride, q_heads, kv_heads, head_dim, rot_heads,
+            (const int*)positions, (const float*)inv_freq, (const int*)token_req, (const int*)block_table, bt_stride,
+            (bf16_t*)k_plane, (bf16_t*)v_plane, page_size);
+    else TL_REQUIRE(false, "rope_cache_write: unknown dtype %d", act_dtype);
+    TL_CHECK_LAUNCH("rope_cache_write");
+    return TL_OK;
+}
+
+// ------------------------------------------------------------------ SwiGLU gate
+// out[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(g) = g / (1 + exp(-g)).
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const size_t t = idx / inter;
+    const int i = (int)(idx % inter);
+    const float g = to_float(gu[t * 2 * inter + i]);
+    const float u = to_float(gu[t * 2 * inter + inter + i]);
+    out[idx] = from_float<T>(g / (1.f + expf(-g)) * u);
+}
+
+extern "C" int tl_swiglu(const void* gu, void* out, int tokens, int inter, int act_dtype, hipStream_t stream) {
+    TL_REQUIRE(tokens >= 0 && inter > 0, "swiglu: bad sizes tokens=%d inter=%d", tokens, inter);
+    const size_t total = (size_t)tokens * inter;
+    if (total == 0) return TL_OK;
+    dim3 block(256), grid((unsigned)((total + 255) / 256));
+    if (act_dtype == TL_DT_F32)
+        swiglu_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, inter, total);
+    else if (act_dtype == TL_DT_BF16)
+        swiglu_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total);
+    else TL_REQUIRE(false, "swiglu: unknown dtype %d", act_dtype);
+    TL_CHECK_LAUNCH("swiglu");
+    return TL_OK;
+}

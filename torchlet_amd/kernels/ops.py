@@ -1,0 +1,246 @@
+"""Python face of the HIP kernels: one function per kernel entry point.
+
+Every function takes ``torch`` tensors that already live on the GPU, checks shapes and
+dtypes on the host (a kernel is never launched on operands it was not written for),
+and launches on the current HIP stream.  Outputs are written into tensors the caller
+allocated; nothing here allocates device memory except :func:`paged_attention`'s
+split-merge scratch.  There is no CPU implementation: a missing library, or a tensor
+that is not on the GPU, raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_void_p
+
+import torch
+
+from . import build as _build
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_libs: dict[str, ctypes.CDLL] = {}
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _lib(name: str) -> ctypes.CDLL:
+    lib = _libs.get(name)
+    if lib is None:
+        try:
+            path = _build.build(name)
+        except _build.BuildError as exc:
+            raise KernelError(f"kernel library {name!r} is not built and cannot be built here: {exc}") from exc
+        try:
+            lib = ctypes.CDLL(str(path))
+        except OSError as exc:
+            raise KernelError(f"cannot load {path}: {exc}") from exc
+        lib.tl_last_error.restype = ctypes.c_char_p
+        _libs[name] = lib
+    return lib
+
+
+def load(names) -> None:
+    """Build (in parallel, if needed) and load the named libraries ahead of use."""
+    missing = [n for n in names if n not in _libs]
+    stale = [n for n in missing if not _build.is_current(n)]
+    if stale:
+        _build.build_many(stale)
+    for n in missing:
+        _lib(n)
+
+
+def loaded_libraries() -> list[str]:
+    return sorted(str(_build.lib_path(n)) for n in _libs)
+
+
+def _check(lib: ctypes.CDLL, code: int) -> None:
+    if code != 0:
+        raise KernelError(lib.tl_last_error().decode())
+
+
+def _ptr(t: torch.Tensor | None) -> c_void_p:
+    if t is None:
+        return c_void_p(0)
+    if not t.is_cuda:
+        raise KernelError(f"kernel operand on {t.device}; the kernels run on the GPU only")
+    return c_void_p(t.data_ptr())
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dt(t: torch.Tensor, what: str) -> int:
+    code = _DT.get(t.dtype)
+    if code is None:
+        raise KernelError(f"{what}: dtype {t.dtype} is not built (float32 and bfloat16 are)")
+    return code
+
+
+def _vec(t: torch.Tensor | None, n: int, what: str) -> int:
+    """Check a weight/bias vector; returns 1 when it is float32, 0 for bfloat16."""
+    if t is None:
+        return 0
+    if t.shape != (n,) or not t.is_contiguous():
+        raise KernelError(f"{what}: expected a contiguous vector of {n}, got {tuple(t.shape)}")
+    return 1 if _dt(t, what) == 0 else 0
+
+
+def _i32(t: torch.Tensor | None, what: str, n: int | None = None) -> None:
+    if t is None:
+        return
+    if t.dtype != torch.int32 or not t.is_contiguous() or (n is not None and t.numel() < n):
+        raise KernelError(f"{what}: expected contiguous int32 of at least {n} elements, got {t.dtype} {tuple(t.shape)}")
+
+
+# ----------------------------------------------------------------------------- ops
+
+def embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[t] = float(table[token_ids[t]])``; ``out`` is the 32-bit residual ``[T, H]``."""
+    T = token_ids.numel()
+    V, H = table.shape
+    _i32(token_ids, "embedding ids", T)
+    if out.shape != (T, H) or out.dtype != torch.float32 or not out.is_contiguous() or not table.is_contiguous():
+        raise KernelError(f"embedding: out must be contiguous float32 [{T}, {H}], got {out.dtype} {tuple(out.shape)}")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_embedding(_ptr(token_ids), _ptr(table), c_int(_dt(table, "embedding table")), _ptr(out),
+                                 c_int(T), c_int(H), c_int(V), _stream()))
+
+
+def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
+    """``r = residual (+ pending)``; ``out = r * rsqrt(mean(r^2) + eps) * weight``.
+
+    Without ``rows`` every row is processed and ``r`` is written back into ``residual``;
+    with ``rows`` (int32 source rows) only those are read and ``residual`` is untouched."""
+    T, H = residual.shape
+    n = T if rows is None else rows.numel()
+    if residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise KernelError("add_rmsnorm: the residual must be contiguous float32")
+    if pending is not None and (pending.shape != residual.shape or pending.dtype != out.dtype or not pending.is_contiguous()):
+        raise KernelError(f"add_rmsnorm: pending {pending.dtype} {tuple(pending.shape)} does not match residual/out")
+    if out.shape != (n, H) or not out.is_contiguous():
+        raise KernelError(f"add_rmsnorm: out must be contiguous [{n}, {H}], got {tuple(out.shape)}")
+    _i32(rows, "add_rmsnorm rows")
+    wf = _vec(weight, H, "add_rmsnorm weight")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_add_rmsnorm(_ptr(residual), _ptr(pending), _ptr(weight), c_int(wf), c_float(eps), _ptr(out),
+                                   _ptr(rows), c_int(n), c_int(H), c_int(_dt(out, "add_rmsnorm")), _stream()))
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> None:
+    """``out = x @ weight.T (+ bias)``; ``x [M, K]`` (rows may be strided), ``weight [N, K]``
+    contiguous and of ``x``'s dtype, ``out [M, N]`` of that dtype or float32."""
+    M, K = x.shape
+    N, K2 = weight.shape
+    if K2 != K or out.shape != (M, N):
+        raise KernelError(f"linear: shapes x{tuple(x.shape)} w{tuple(weight.shape)} out{tuple(out.shape)} do not fit")
+    if x.dtype != weight.dtype or x.stride(1) != 1 or out.stride(1) != 1 or not weight.is_contiguous():
+        raise KernelError("linear: x and weight must share a dtype, weight contiguous, unit stride on the last axis")
+    if out.dtype not in (x.dtype, torch.float32):
+        raise KernelError(f"linear: out dtype {out.dtype} must be {x.dtype} or float32")
+    bf = _vec(bias, N, "linear bias")
+    lib = _lib("gemm")
+    _check(lib, lib.tl_gemm_general(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N), c_int(K),
+                                    c_int(x.stride(0)), c_int(out.stride(0)), c_int(_dt(x, "linear")),
+                                    c_int(1 if out.dtype == torch.float32 else 0), _stream()))
+
+
+def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int, rot_heads: int,
+                     positions: torch.Tensor, inv_freq: torch.Tensor | None,
+                     token_req: torch.Tensor | None = None, block_table: torch.Tensor | None = None,
+                     k_plane: torch.Tensor | None = None, v_plane: torch.Tensor | None = None,
+                     page_size: int = 0) -> None:
+    """Rotate the first ``rot_heads`` heads of each row of ``qkv [T, >= (q+2kv)*hd]`` in
+    place by the token's position (``inv_freq`` float32 ``[hd/2]``; ``None``: no rotation)
+    and, when planes are given, store rotated k and raw v of every token in its page."""
+    T = qkv.shape[0]
+    if qkv.stride(1) != 1:
+        raise KernelError("rope_cache_write: qkv needs unit stride on the last axis")
+    _i32(positions, "positions", T)
+    if inv_freq is not None and (inv_freq.dtype != torch.float32 or inv_freq.numel() != head_dim // 2):
+        raise KernelError("rope_cache_write: inv_freq must be float32 [head_dim/2]")
+    bt_stride = 0
+    if k_plane is not None:
+        _i32(token_req, "token_req", T)
+        _i32(block_table, "block_table")
+        bt_stride = block_table.stride(0)
+        for p in (k_plane, v_plane):
+            if p.dtype != qkv.dtype or p.dim() != 4 or p.shape[1:] != (kv_heads, page_size, head_dim) or not p.is_contiguous():
+                raise KernelError(f"rope_cache_write: plane {tuple(p.shape)} {p.dtype} is not [pages, {kv_heads}, {page_size}, {head_dim}] {qkv.dtype}")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_rope_cache_write(_ptr(qkv), c_int(qkv.stride(0)), c_int(T), c_int(q_heads), c_int(kv_heads),
+                                        c_int(head_dim), c_int(rot_heads), _ptr(positions), _ptr(inv_freq), _ptr(token_req),
+                                        _ptr(block_table), c_int(bt_stride), _ptr(k_plane), _ptr(v_plane), c_int(page_size),
+                                        c_int(_dt(qkv, "rope_cache_write")), _stream()))
+
+
+ATTENTION_ROWS = 16   # rows (tokens x heads of one group) a work-group owns
+
+
+def attention_tile_tokens(num_heads: int, num_kv_heads: int) -> int:
+    """New tokens of one request that share a tile, given the group size."""
+    group = num_heads // num_kv_heads
+    return max(1, ATTENTION_ROWS // min(group, ATTENTION_ROWS))
+
+
+def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v_plane: torch.Tensor,
+                    block_table: torch.Tensor, req_indptr: torch.Tensor, ctx_lens: torch.Tensor,
+                    tile_req: torch.Tensor, tile_tok0: torch.Tensor, num_tiles: int, tile_tokens: int,
+                    num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
+                    scale: float, splits: int = 1) -> None:
+    """Causal attention of the step's tokens over their requests' cached keys.
+
+    ``q [T, >= heads*hd]`` (row-strided view), ``out [T, heads*hd]``, planes
+    ``[pages, kv_heads, page, hd]``, ``block_table [R, max_blocks]`` int32; the new token
+    ``i`` of request ``r`` sits at position ``ctx_lens[r] + i``.  ``window`` 0: all keys."""
+    T = q.shape[0]
+    if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelError("paged_attention: q/out shapes or dtypes do not fit")
+    for p in (k_plane, v_plane):
+        if p.dtype != q.dtype or p.dim() != 4 or p.shape[1:] != (num_kv_heads, page_size, head_dim) or not p.is_contiguous():
+            raise KernelError(f"paged_attention: plane {tuple(p.shape)} {p.dtype} is not [pages, {num_kv_heads}, {page_size}, {head_dim}] {q.dtype}")
+    for name, t in (("block_table", block_table), ("req_indptr", req_indptr), ("ctx_lens", ctx_lens),
+                    ("tile_req", tile_req), ("tile_tok0", tile_tok0)):
+        _i32(t, name)
+    if tile_req.numel() < num_tiles or tile_tok0.numel() < num_tiles:
+        raise KernelError("paged_attention: tile arrays shorter than the number of tiles")
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((T * num_heads * splits, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T * num_heads * splits, 2), dtype=torch.float32, device=q.device)
+    lib = _lib(f"attention_hd{head_dim}")
+    _check(lib, lib.tl_paged_attention(_ptr(q), c_int(q.stride(0)), _ptr(out), _ptr(k_plane), _ptr(v_plane),
+                                       _ptr(block_table), c_int(block_table.stride(0)), _ptr(req_indptr), _ptr(ctx_lens),
+                                       _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles), c_int(T), c_int(tile_tokens),
+                                       c_int(num_heads), c_int(num_kv_heads), c_int(page_size), c_int(window),
+                                       c_float(scale), c_int(splits), _ptr(part_o), _ptr(part_ml),
+                                       c_int(_dt(q, "paged_attention")), _stream()))
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]``."""
+    T, I2 = gate_up.shape
+    if I2 % 2 or out.shape != (T, I2 // 2) or out.dtype != gate_up.dtype or not out.is_contiguous() or not gate_up.is_contiguous():
+        raise KernelError("swiglu: shapes or dtypes do not fit")
+    lib = _lib("elementwise")
+    _check(lib, lib.tl_swiglu(_ptr(gate_up), _ptr(out), c_int(T), c_int(I2 // 2), c_int(_dt(out, "swiglu")), _stream()))
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor | None, keys: torch.Tensor | None, out: torch.Tensor) -> None:
+    """Token per row of float32 ``logits [N, V]``: arg max where ``temperature`` is 0 (or
+    absent), else a Gumbel-max draw from ``softmax(logits / temperature)`` seeded by the
+    row's int32 ``keys`` entry."""
+    N, V = logits.shape
+    if logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("sample: logits must be float32 with unit stride on the last axis")
+    if temperature is not None and (temperature.dtype != torch.float32 or temperature.numel() < N or not temperature.is_contiguous()):
+        raise KernelError("sample: temperature must be contiguous float32 [N]")
+    _i32(keys, "sample keys", N)
+    _i32(out, "sample out", N)
+    lib = _lib("sampling")
+    _check(lib, lib.tl_sample(_ptr(logits), c_int(N), c_int(V), c_int(logits.stride(0)), _ptr(temperature), _ptr(keys),
+                              _ptr(out), _stream()))

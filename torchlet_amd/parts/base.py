@@ -1,0 +1,185 @@
+"""Interfaces of the parts a layer is put together from, and their registries.
+
+A part is built from its specification (plain sizes and constants), declares the
+tensors it wants by relative name, receives them, and runs on the tokens of one
+step.  No part sees a configuration, a layer index or the model it is in.
+
+Five kinds of parts, each with a registry from the specification's ``kind`` to a class:
+
+===================  =====================================================================
+``Norm``             ``forward(stream) -> h``: folds the stream's pending branch output
+                     into the 32-bit residual and returns the normalised activations.
+``PositionEncoding`` ``apply(q, k, positions)``: in place on ``[T, heads, head_dim]`` views.
+``Mixer``            ``forward(h, ctx, cache) -> [T, hidden]``: mixes tokens; declares the
+                     cache it needs (pages per token and/or a fixed-size state per request).
+``FeedForward``      ``forward(h, ctx) -> [T, hidden]``: stateless.
+``Block``            ``forward(stream, ctx, cache) -> stream``: arranges the four above.
+===================  =====================================================================
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable
+
+import torch
+
+from ..config.base import ConfigError, PartSpec
+
+
+# ------------------------------------------------------------------ weights of a part
+
+@dataclass(frozen=True)
+class WeightSpec:
+    """One tensor a part wants from the checkpoint.
+
+    ``role``: ``matrix`` tensors are matrix-product operands and take the engine's
+    compute dtype; ``vector`` tensors keep the dtype they are stored in (bfloat16 stays
+    bfloat16, 32-bit stays 32-bit; a 32-bit engine widens them); ``table`` tensors are
+    integer tables kept as int32.
+    ``init``: law of the random-weights mode, ``normal`` = N(0, std),
+    ``one_plus_normal`` = 1 + N(0, std).
+    ``optional``: the checkpoint may leave it out (a tied head).
+    """
+    shape: tuple[int, ...]
+    role: str = "matrix"
+    init: str = "normal"
+    optional: bool = False
+
+
+class Part:
+    """Common protocol: declare tensors, receive them."""
+
+    def __init__(self, spec: PartSpec, dtype: torch.dtype, device: torch.device):
+        self.spec = spec
+        self.dtype = dtype
+        self.device = device
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {}
+
+    def load_weights(self, tensors: dict[str, torch.Tensor]) -> None:
+        """``tensors``: the declared names (those present) -> CPU tensors as stored."""
+
+    # helpers ---------------------------------------------------------------------
+    def _place(self, t: torch.Tensor, role: str) -> torch.Tensor:
+        if role == "matrix":
+            return t.to(device=self.device, dtype=self.dtype).contiguous()
+        if role == "table":
+            return t.to(device=self.device, dtype=torch.int32).contiguous()
+        if self.dtype == torch.float32 or t.dtype not in (torch.bfloat16, torch.float32):
+            t = t.to(torch.float32)
+        return t.to(self.device).contiguous()
+
+
+# ------------------------------------------------------------------------ cache needs
+
+@dataclass(frozen=True)
+class PagedNeed:
+    """Per-token cache: ``planes`` tensors of ``[num_heads, head_dim]`` per token
+    (keys and values are two planes), kept for all tokens (``window=None``) or for the
+    last ``window`` tokens.  Layers with equal needs share a group of pages."""
+    num_heads: int
+    head_dim: int
+    window: int | None = None
+    planes: int = 2
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Fixed-size per-request state: one tensor of ``shape`` per slot, zero when a
+    request is admitted."""
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+# --------------------------------------------------------------------------- streams
+
+class Stream:
+    """The hidden state between parts: a 32-bit residual ``[T, hidden]`` and the output
+    of the last branch that is still to be added to it (``pending``, or ``None``).
+    The next norm adds ``pending`` in 32-bit while it normalises, which saves one pass
+    over the residual per branch."""
+
+    __slots__ = ("residual", "pending")
+
+    def __init__(self, residual: torch.Tensor, pending: torch.Tensor | None = None):
+        self.residual = residual
+        self.pending = pending
+
+
+# ----------------------------------------------------------------------- part kinds
+
+class Norm(Part):
+    def forward(self, stream: Stream, rows: torch.Tensor | None = None) -> torch.Tensor:
+        """Add ``stream.pending`` into ``stream.residual`` (both kept up to date) and
+        return ``norm(residual)`` in the activation dtype.  With ``rows`` (int32 indices)
+        only those rows are read and returned, and the stream is left untouched."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def apply(self, q: torch.Tensor, k: torch.Tensor | None, positions: torch.Tensor) -> None:
+        """Encode ``positions [T]`` into ``q [T, heads, head_dim]`` and ``k`` in place
+        (views with unit stride on the last axis)."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def paged_need(self) -> PagedNeed | None:
+        return None
+
+    def state_need(self) -> StateNeed | None:
+        return None
+
+    def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
+        """``h [T, hidden]`` -> ``[T, hidden]``.  ``cache`` is this run's
+        :class:`torchlet_amd.cache.manager.LayerCache` (or ``None`` when the mixer
+        declared no need)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    mixer: Mixer
+
+    def forward(self, stream: Stream, ctx, cache) -> Stream:
+        raise NotImplementedError
+
+
+# ------------------------------------------------------------------------ registries
+
+class Registry:
+    """``kind`` -> class, with a decorator to add to it and a clear error on a miss."""
+
+    def __init__(self, what: str):
+        self.what = what
+        self._classes: dict[str, type] = {}
+
+    def register(self, kind: str) -> Callable[[type], type]:
+        def add(cls: type) -> type:
+            self._classes[kind] = cls
+            return cls
+        return add
+
+    def unregister(self, kind: str) -> None:
+        self._classes.pop(kind, None)
+
+    def names(self) -> list[str]:
+        return sorted(self._classes)
+
+    def build(self, spec: PartSpec, dtype: torch.dtype, device: torch.device):
+        cls = self._classes.get(spec.kind)
+        if cls is None:
+            raise ConfigError(f"no {self.what} of kind {spec.kind!r}; known: {', '.join(self.names())}")
+        return cls(spec, dtype, device)
+
+
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+BLOCKS = Registry("block")

@@ -24,3 +24,25 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(scope="session")
+def model_folders(tmp_path_factory):
+    """name -> folder of a tiny random-weight model (written once per session, in a temporary folder)."""
+    import tiny_models
+
+    root = tmp_path_factory.mktemp("models")
+    return {name: tiny_models.write(name, root) for name in tiny_models.CONFIGS}
+
+
+@pytest.fixture
+def cpu_ops(monkeypatch):
+    """Patch the CPU stand-ins of ``tests/emulated_ops.py`` over the HIP entry points, so that
+    host logic can run without a GPU.  Never used by GPU tests."""
+    import emulated_ops
+    from torchlet_amd.kernels import ops
+
+    for name in ("attention_tile_tokens", "load", "embedding", "add_rmsnorm", "linear", "rope_cache_write",
+                 "paged_attention", "swiglu", "sample"):
+        monkeypatch.setattr(ops, name, getattr(emulated_ops, name))
+    return ops

@@ -1,0 +1,93 @@
+"""The step function: a batch of ``(request, its next tokens)`` in, logits out.
+
+It runs only the tokens it is given, as one batch, on top of what earlier steps left in
+the cache, and returns the logits at the wanted places.  Pages are reserved before the
+model runs and the new lengths are committed after it; a step that cannot get its pages
+raises :class:`~torchlet_amd.cache.manager.OutOfPages` and leaves the cache as it was.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache.manager import CacheManager, OutOfPages
+from .batch import StepContext, StepEntry
+
+
+class ModelRunner:
+    def __init__(self, model, cache: CacheManager):
+        self.model = model
+        self.cache = cache
+        self.device = model.device
+        self.caches = [cache.layer_cache(i) for i in range(len(model.spec.order))]
+        self.tile_sizes = model.tile_token_sizes()
+        self.max_positions = model.spec.max_positions
+        self.vocab_size = model.spec.vocab_size
+
+    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+        """Logits ``[number of wanted places, vocab]`` (float32, on the GPU), in the order
+        of the entries and of their ``want`` lists; ``None`` if nothing is wanted."""
+        if not entries:
+            return None
+        cache = self.cache
+        added = []
+        try:
+            return self._step(entries, added)
+        except Exception:
+            for req_id in added:            # a failed step leaves no trace of requests it introduced
+                if cache.has(req_id) and cache.length(req_id) == 0:
+                    cache.release(req_id)
+            raise
+
+    def _step(self, entries: list[StepEntry], added: list) -> torch.Tensor | None:
+        cache = self.cache
+        seen = set()
+        for e in entries:
+            if e.req_id in seen:
+                raise ValueError(f"request {e.req_id!r} appears twice in one step")
+            seen.add(e.req_id)
+            if not e.tokens:
+                raise ValueError(f"request {e.req_id!r} brings no tokens")
+            bad = [t for t in e.tokens if not 0 <= t < self.vocab_size]
+            if bad:
+                raise ValueError(f"request {e.req_id!r}: token id {bad[0]} outside the vocabulary of {self.vocab_size}")
+            if any(not 0 <= w < len(e.tokens) for w in e.want):
+                raise ValueError(f"request {e.req_id!r}: wanted place outside its {len(e.tokens)} tokens")
+            if not cache.has(e.req_id):
+                cache.add_request(e.req_id)
+                added.append(e.req_id)
+            if cache.length(e.req_id) + len(e.tokens) > self.max_positions:
+                raise ValueError(f"request {e.req_id!r} would pass max_position_embeddings ({self.max_positions})")
+        ctx_lens = [cache.length(e.req_id) for e in entries]
+        new_lens = [len(e.tokens) for e in entries]
+        # all-or-nothing over the whole step: check first, then take
+        need = [0] * len(cache.groups)
+        for e, c, n in zip(entries, ctx_lens, new_lens):
+            for g, m in enumerate(cache.pages_missing(e.req_id, c + n)):
+                need[g] += m
+        free = cache.free_pages()
+        if any(n > f for n, f in zip(need, free)):
+            raise OutOfPages(f"step needs {need} pages per group, {free} are free")
+        for e, c, n in zip(entries, ctx_lens, new_lens):
+            if not cache.reserve(e.req_id, c + n):      # cannot happen after the check above
+                raise OutOfPages(f"request {e.req_id!r}: reservation failed")
+
+        req_ids = [e.req_id for e in entries]
+        blocks = -(-max(c + n for c, n in zip(ctx_lens, new_lens)) // cache.page_size)
+        token_ids, want_rows, base = [], [], 0
+        for e in entries:
+            token_ids.extend(e.tokens)
+            want_rows.extend(base + w for w in e.want)
+            base += len(e.tokens)
+        ctx = StepContext(
+            new_lens=new_lens, ctx_lens=ctx_lens, slots=[cache.slot(r) for r in req_ids],
+            token_ids=token_ids, want_rows=want_rows,
+            block_tables=[cache.block_table(g, req_ids, blocks) for g in range(len(cache.groups))],
+            tile_sizes=self.tile_sizes, device=self.device)
+        logits = self.model.forward(ctx, self.caches)
+        for e, c, n in zip(entries, ctx_lens, new_lens):
+            cache.commit(e.req_id, c + n)
+        return logits
+
+    def release(self, req_id) -> None:
+        if self.cache.has(req_id):
+            self.cache.release(req_id)

@@ -1,0 +1,121 @@
+"""Grouped-query attention over a paged key/value cache.
+
+Formulas (/root/reference/src/torchlet/v10_triton_paged_gqa/layer/gqa.py:112-146 and
+kernel/gqa.py:58-111): ``q = h Wq^T + bq`` and likewise k, v; heads are split head-major
+(feature ``= head * head_dim + d``); q and k are position-encoded; the encoded k and the
+raw v of every new token are stored in the cache; query head ``i`` reads KV head
+``i // (heads / kv_heads)``; scores are scaled by ``head_dim ** -0.5``, masked causally
+(and to the last ``window`` keys if the layer has a window), soft-maxed in 32-bit, and
+the weighted values go through ``o_proj`` (no bias).
+
+The three projections are stacked into one ``[(heads + 2 kv_heads) * head_dim, hidden]``
+matrix at load time, so one matrix product reads ``h`` once.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.base import ConfigError
+from ..kernels import ops
+from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedNeed, WeightSpec
+
+_TARGET_WORKGROUPS = 512     # enough work-groups to fill 256 compute units twice
+_MIN_KEYS_PER_SPLIT = 256
+
+
+@MIXERS.register("gqa_attention")
+class GQAttention(Mixer):
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.num_heads % spec.num_kv_heads:
+            raise ConfigError(f"attention: {spec.num_heads} heads are not a multiple of {spec.num_kv_heads} KV heads")
+        if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
+            raise ConfigError(f"attention kernels are built for head sizes that are multiples of 16 up to 256, not {spec.head_dim}")
+        if spec.window is not None and spec.window < 1:
+            raise ConfigError(f"attention: a window must hold at least one key, got {spec.window}")
+        self.hidden = spec.hidden
+        self.heads = spec.num_heads
+        self.kv_heads = spec.num_kv_heads
+        self.head_dim = spec.head_dim
+        self.window = spec.window
+        self.scale = float(spec.head_dim) ** -0.5
+        self.q_width = self.heads * self.head_dim
+        self.kv_width = self.kv_heads * self.head_dim
+        self.qkv_bias = spec.qkv_bias
+        self.position = POSITION_ENCODINGS.build(spec.position, dtype, device) if spec.position is not None else None
+        self.tile_tokens = ops.attention_tile_tokens(self.heads, self.kv_heads)
+        self.w_qkv: torch.Tensor | None = None
+        self.b_qkv: torch.Tensor | None = None
+        self.w_o: torch.Tensor | None = None
+
+    # -- declarations -------------------------------------------------------------
+    def paged_need(self):
+        return PagedNeed(num_heads=self.kv_heads, head_dim=self.head_dim, window=self.window, planes=2)
+
+    def kernel_libraries(self):
+        return [f"attention_hd{self.head_dim}"]
+
+    def weight_specs(self):
+        specs = {
+            "q_proj.weight": WeightSpec((self.q_width, self.hidden)),
+            "k_proj.weight": WeightSpec((self.kv_width, self.hidden)),
+            "v_proj.weight": WeightSpec((self.kv_width, self.hidden)),
+            "o_proj.weight": WeightSpec((self.hidden, self.q_width)),
+        }
+        if self.qkv_bias:
+            specs["q_proj.bias"] = WeightSpec((self.q_width,), role="vector")
+            specs["k_proj.bias"] = WeightSpec((self.kv_width,), role="vector")
+            specs["v_proj.bias"] = WeightSpec((self.kv_width,), role="vector")
+        return specs
+
+    def load_weights(self, tensors):
+        self.w_qkv = self._place(torch.cat([tensors[f"{n}_proj.weight"] for n in "qkv"], dim=0), "matrix")
+        if self.qkv_bias:
+            biases = [tensors[f"{n}_proj.bias"] for n in "qkv"]
+            if len({b.dtype for b in biases}) > 1:
+                biases = [b.to(torch.float32) for b in biases]
+            self.b_qkv = self._place(torch.cat(biases), "vector")
+        self.w_o = self._place(tensors["o_proj.weight"], "matrix")
+
+    # -- the step -----------------------------------------------------------------
+    def _splits(self, ctx, tiles: int) -> int:
+        group = self.heads // self.kv_heads
+        chunks = -(-group // ops.ATTENTION_ROWS)
+        base = max(1, tiles * self.kv_heads * chunks)
+        by_fill = -(-_TARGET_WORKGROUPS // base)
+        longest = ctx.max_total_len if self.window is None else min(ctx.max_total_len, self.window + ctx.max_new_tokens)
+        by_keys = max(1, longest // _MIN_KEYS_PER_SPLIT)
+        return max(1, min(by_fill, by_keys, 64))
+
+    def forward(self, h, ctx, cache):
+        T = h.shape[0]
+        writes = cache.writable
+        width = self.q_width + (2 * self.kv_width if writes else 0)
+        w = self.w_qkv if writes else self.w_qkv[: self.q_width]
+        b = self.b_qkv if (self.b_qkv is None or writes) else self.b_qkv[: self.q_width]
+        qkv = torch.empty((T, width), dtype=self.dtype, device=h.device)
+        ops.linear(h, w, b, qkv)
+
+        k_plane, v_plane = cache.planes
+        table = ctx.block_tables[cache.group]
+        kv_heads = self.kv_heads if writes else 0
+        inv_freq = self.position.fused_inv_freq() if hasattr(self.position, "fused_inv_freq") else None
+        if self.position is not None and inv_freq is None:
+            q3 = qkv[:, : self.q_width].unflatten(1, (self.heads, self.head_dim))
+            k3 = qkv[:, self.q_width: self.q_width + self.kv_width].unflatten(1, (self.kv_heads, self.head_dim)) if writes else None
+            self.position.apply(q3, k3, ctx.positions)
+        if inv_freq is not None or writes:
+            ops.rope_cache_write(
+                qkv, self.heads, kv_heads, self.head_dim, self.heads + kv_heads, ctx.positions, inv_freq,
+                ctx.token_req if writes else None, table if writes else None,
+                k_plane if writes else None, v_plane if writes else None, cache.page_size if writes else 0)
+
+        tile_req, tile_tok0, tiles = ctx.tiles(self.tile_tokens)
+        out = torch.empty((T, self.q_width), dtype=self.dtype, device=h.device)
+        ops.paged_attention(
+            qkv[:, : self.q_width], out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
+            tile_req, tile_tok0, tiles, self.tile_tokens, self.heads, self.kv_heads, self.head_dim,
+            cache.page_size, self.window or 0, self.scale, self._splits(ctx, tiles))
+        y = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
+        ops.linear(out, self.w_o, None, y)
+        return y

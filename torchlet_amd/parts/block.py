@@ -1,0 +1,41 @@
+"""Pre-norm residual block: ``x += mixer(norm1(x)); x += ffn(norm2(x))``
+(/root/reference/src/torchlet/v10_triton_paged_gqa/layer/transformer_block.py:37-40).
+
+The additions are deferred: a branch's output is left ``pending`` on the stream and the
+next norm (the block's second one, the next block's first one, or the model's final one)
+adds it in 32-bit while it normalises.
+"""
+from __future__ import annotations
+
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, Stream
+
+
+@BLOCKS.register("prenorm_residual")
+class PreNormBlock(Block):
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.mixer_norm = NORMS.build(spec.mixer_norm, dtype, device)
+        self.mixer = MIXERS.build(spec.mixer, dtype, device)
+        self.ffn_norm = NORMS.build(spec.ffn_norm, dtype, device)
+        self.ffn = FEED_FORWARDS.build(spec.ffn, dtype, device)
+        self._children = {
+            spec.mixer_norm_name: self.mixer_norm,
+            spec.mixer_name: self.mixer,
+            spec.ffn_norm_name: self.ffn_norm,
+            spec.ffn_name: self.ffn,
+        }
+
+    def weight_specs(self):
+        return {f"{name}.{k}": v for name, part in self._children.items() for k, v in part.weight_specs().items()}
+
+    def load_weights(self, tensors):
+        for name, part in self._children.items():
+            prefix = name + "."
+            part.load_weights({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
+
+    def forward(self, stream: Stream, ctx, cache) -> Stream:
+        h = self.mixer_norm.forward(stream)
+        stream.pending = self.mixer.forward(h, ctx, cache)
+        h = self.ffn_norm.forward(stream)
+        stream.pending = self.ffn.forward(h, ctx)
+        return stream

@@ -1,0 +1,56 @@
+"""Random weights from a configuration and a seed.
+
+Law: matrices and biases ``N(0, 0.02)``, norm weights ``1 + N(0, 0.02)``, drawn in 32-bit
+from one ``torch.Generator(seed)`` in the order of the model's tensor declarations, then
+rounded to the storage dtype.  :func:`write_model_folder` writes ``config.json`` and
+``model.safetensors`` so that the engine and any other reader load identical values;
+:func:`random_tensors` makes the same kind of tensors directly on a device (for
+benchmark-size models, where a detour over a file would take minutes).
+"""
+from __future__ import annotations
+
+from pathlib import Path
+
+import torch
+from safetensors.torch import save_file
+
+from ..config.base import ModelConfig
+from ..models.decoder import DecoderModel
+
+STD = 0.02
+
+
+def _draw(spec, gen: torch.Generator, device) -> torch.Tensor:
+    if spec.role == "table":
+        return torch.randint(0, 2 ** 15, spec.shape, generator=gen, device=device, dtype=torch.int32)
+    t = torch.randn(spec.shape, generator=gen, device=device, dtype=torch.float32) * STD
+    if spec.init == "one_plus_normal":
+        t = t + 1.0
+    return t
+
+
+def random_tensors(config: ModelConfig, seed: int, dtype: torch.dtype = torch.bfloat16, device="cpu") -> dict[str, torch.Tensor]:
+    """``name -> tensor`` for every tensor the architecture's model declares (a tied head
+    is left out, as in a checkpoint)."""
+    model = DecoderModel(config.to_spec(), torch.float32, "cpu")
+    gen = torch.Generator(device=device).manual_seed(int(seed))
+    out = {}
+    for name, spec in model.weight_specs().items():
+        if spec.optional:
+            continue
+        t = _draw(spec, gen, device)
+        out[name] = t if spec.role == "table" else t.to(dtype)
+    return out
+
+
+def write_model_folder(config: ModelConfig, seed: int, folder: str | Path, dtype: torch.dtype = torch.bfloat16) -> Path:
+    """Write ``config.json`` and ``model.safetensors`` (tensors stored in ``dtype``)."""
+    folder = Path(folder)
+    folder.mkdir(parents=True, exist_ok=True)
+    d = config.to_dict()
+    d["torch_dtype"] = {torch.bfloat16: "bfloat16", torch.float32: "float32", torch.float16: "float16"}[dtype]
+    import json
+    (folder / "config.json").write_text(json.dumps(d, indent=2) + "\n")
+    tensors = {k: v.contiguous() for k, v in random_tensors(config, seed, dtype, "cpu").items()}
+    save_file(tensors, str(folder / "model.safetensors"), metadata={"format": "pt"})
+    return folder

@@ -1,0 +1,135 @@
+"""Ways of cutting the same requests into steps, and the check of a replay against the
+plain implementation.  A *step* is ``{"step": i, "entries": [{"id", "tokens", "want"}], "end": [...]}``
+as ``bin/trace_run`` reads it."""
+import random
+
+import numpy as np
+import torch
+
+import plain_qwen2
+
+FP32_TOL = dict(atol=4e-6, rtol=2e-5)     # ~10x the 32-bit rounding of the plain implementation itself (3.7e-7)
+BF16_TOL = dict(atol=1e-2, rtol=1e-2)     # ~3x what the design's bfloat16 roundings add on these models (3.3e-3)
+
+
+def make_requests(vocab: int, lengths, seed: int) -> dict[str, list[int]]:
+    g = torch.Generator().manual_seed(seed)
+    return {f"r{i}": torch.randint(0, vocab, (n,), generator=g).tolist() for i, n in enumerate(lengths)}
+
+
+def _round_up(n, m):
+    return -(-n // m) * m
+
+
+def whole(requests):
+    """Each request alone and whole: one step, every logit wanted."""
+    return [dict(entries=[dict(id=r, tokens=t, want=list(range(len(t))))], end=[r]) for r, t in requests.items()]
+
+
+def tail_singles(requests, tail=32):
+    """Most of a request in one step, then its last ``tail`` tokens one by one."""
+    steps = []
+    for r, t in requests.items():
+        head = max(1, len(t) - tail)
+        steps.append(dict(entries=[dict(id=r, tokens=t[:head], want=list(range(head)))], end=[]))
+        for i in range(head, len(t)):
+            steps.append(dict(entries=[dict(id=r, tokens=[t[i]], want=[0])], end=[r] if i == len(t) - 1 else []))
+        if head == len(t):
+            steps[-1]["end"] = [r]
+    return steps
+
+
+def portions(requests, sizes=(7, 16, 2, 5, 3, 33, 2, 9, 17, 2, 64)):
+    """Portions of changing size, down to two tokens, across page edges at odd offsets."""
+    steps = []
+    for k, (r, t) in enumerate(requests.items()):
+        i, j = 0, k
+        while i < len(t):
+            n = min(sizes[j % len(sizes)], len(t) - i)
+            if len(t) - i - n == 1:      # never leave a lone last token: portions are of two or more
+                n += 1
+            steps.append(dict(entries=[dict(id=r, tokens=t[i:i + n], want=list(range(n)))], end=[r] if i + n == len(t) else []))
+            i += n
+            j += 1
+    return steps
+
+
+def mixed(requests, seed=0, max_live=4, prompt_fraction=0.6):
+    """Up to ``max_live`` live requests; portions of some beside single tokens of others; a
+    request is sometimes left out of a step; later requests arrive as earlier ones end."""
+    rng = random.Random(seed)
+    waiting = list(requests.items())
+    live: dict[str, int] = {}
+    steps = []
+    while waiting or live:
+        while waiting and len(live) < max_live and (not live or rng.random() < 0.6):
+            r, _ = waiting.pop(0)
+            live[r] = 0
+        entries, end = [], []
+        for r in list(live):
+            t, done = requests[r], live[r]
+            if len(live) > 1 and rng.random() < 0.2:
+                continue                                  # left out of this step
+            prompt = max(2, int(len(t) * prompt_fraction))
+            if done < prompt:
+                n = min(rng.choice([2, 3, 5, 8, 13, 21]), prompt - done)
+                if prompt - done - n == 1:
+                    n += 1
+            else:
+                n = 1
+            n = min(n, len(t) - done)
+            entries.append(dict(id=r, tokens=t[done:done + n], want=list(range(n))))
+            live[r] = done + n
+            if live[r] == len(t):
+                end.append(r)
+                del live[r]
+        if entries:
+            steps.append(dict(entries=entries, end=end))
+    return steps
+
+
+def number(steps, first=0):
+    return [dict(step=first + i, **s) for i, s in enumerate(steps)]
+
+
+def max_tokens_needed(steps, unit=64) -> int:
+    """Most tokens live requests hold at any time, each rounded up to a multiple of ``unit``."""
+    held: dict[str, int] = {}
+    worst = 0
+    for s in steps:
+        for e in s["entries"]:
+            held[e["id"]] = held.get(e["id"], 0) + len(e["tokens"])
+        worst = max(worst, sum(_round_up(n, unit) for n in held.values()))
+        for r in s["end"]:
+            held.pop(r, None)
+    return worst
+
+
+def expected_logits(folder, requests):
+    cfg, weights = plain_qwen2.load_folder(folder, torch.float64)
+    return {r: plain_qwen2.forward(cfg, weights, t) for r, t in requests.items()}
+
+
+def check(steps, outputs, expected, tol, what=""):
+    """``outputs[step]``: array ``[wanted, vocab]``.  Every row is compared with the plain
+    implementation's logits of its request at its absolute position; the first mismatch
+    is reported with its place."""
+    pos: dict[str, int] = {}
+    for s in steps:
+        rows = outputs.get(s["step"])
+        k = 0
+        for e in s["entries"]:
+            base = pos.get(e["id"], 0)
+            for w in e["want"]:
+                got = torch.from_numpy(np.asarray(rows[k], dtype=np.float32)).double()
+                ref = expected[e["id"]][base + w]
+                if not torch.allclose(got, ref, **tol):
+                    err = float((got - ref).abs().max())
+                    raise AssertionError(
+                        f"{what}: step {s['step']} request {e['id']} position {base + w} "
+                        f"(portion starts at {base}, place {w} of {len(e['tokens'])}): max abs error {err:.3e}")
+                k += 1
+            pos[e["id"]] = base + len(e["tokens"])
+        assert rows is None or k == len(rows), f"{what}: step {s['step']} returned {len(rows)} rows, {k} wanted"
+        for r in s["end"]:
+            pos.pop(r, None)

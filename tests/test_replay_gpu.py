@@ -1,0 +1,86 @@
+"""The step function on the GPU against the plain implementation, under every way of
+cutting the same requests into steps, in 32-bit and in bfloat16."""
+import json
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import scenarios
+import tiny_models
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
+
+LENGTHS = {"A": [70, 33, 97, 5, 120, 64], "B": [40, 129, 9, 64, 200, 1 + 32], "C": [150, 61, 33, 90, 47, 128]}
+TOL = {"float32": scenarios.FP32_TOL, "bfloat16": scenarios.BF16_TOL}
+
+
+def _run_in_process(folder, dtype, steps, page_size, max_tokens, max_requests=4):
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import load_model, make_runner
+
+    _, model = load_model(folder, dtype)
+    runner = make_runner(model, page_size=page_size, num_pages=-(-max_tokens // page_size) + 1, max_requests=max_requests)
+    out = {}
+    for s in steps:
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        if logits is not None:
+            out[s["step"]] = logits.cpu().numpy()
+        for r in s["end"]:
+            runner.release(r)
+    runner.cache.check()
+    assert runner.cache.live_requests() == []
+    return out
+
+
+@pytest.fixture(scope="module")
+def expected(model_folders):
+    cache = {}
+
+    def get(name):
+        if name not in cache:
+            cfg = json.loads((model_folders[name] / "config.json").read_text())
+            reqs = scenarios.make_requests(cfg["vocab_size"], LENGTHS[name], seed=11)
+            cache[name] = (reqs, scenarios.expected_logits(model_folders[name], reqs))
+        return cache[name]
+    return get
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("mode", ["whole", "tail_singles", "portions", "mixed"])
+def test_split(model_folders, expected, name, dtype, mode):
+    reqs, exp = expected(name)
+    build = getattr(scenarios, mode)
+    steps = scenarios.number(build(reqs))
+    page = tiny_models.PAGE_SIZES[name]
+    # the pool holds exactly what the live requests need, so that freed pages are used again
+    out = _run_in_process(model_folders[name], dtype, steps, page, scenarios.max_tokens_needed(steps))
+    scenarios.check(steps, out, exp, TOL[dtype], f"{name}/{dtype}/{mode}")
+
+
+def test_trace_run_program(model_folders, expected, tmp_path):
+    """The replay program itself, as a user starts it: a mixed trace, both dtypes."""
+    reqs, exp = expected("B")
+    steps = scenarios.number(scenarios.mixed(reqs, seed=3))
+    for dtype in ("float32", "bfloat16"):
+        out_dir = tmp_path / dtype
+        proc = subprocess.Popen(
+            [str(ROOT / "bin" / "trace_run"), "--model", str(model_folders["B"]), "--dtype", dtype, "--out", str(out_dir),
+             "--max-tokens", str(scenarios.max_tokens_needed(steps))],
+            stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, env=dict(os.environ, PYTHONUNBUFFERED="1"))
+        for s in steps:
+            proc.stdin.write(json.dumps(s) + "\n")
+            proc.stdin.flush()
+            line = proc.stdout.readline().strip()
+            assert line == f"done {s['step']}", f"expected 'done {s['step']}', got {line!r}"
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+        vocab = len(next(iter(exp.values()))[0])
+        out = {int(p.stem): np.fromfile(p, dtype="<f4").reshape(-1, vocab) for p in out_dir.glob("*.f32")}
+        scenarios.check(steps, out, exp, TOL[dtype], f"trace_run/{dtype}")

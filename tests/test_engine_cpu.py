@@ -1,0 +1,141 @@
+"""The engine's host logic on the CPU: step function over the cache manager, scheduler
+and sampler, with the HIP entry points replaced by the stand-ins of ``emulated_ops.py``.
+The kernels themselves are tested on the GPU (``-m gpu``)."""
+import json
+
+import pytest
+import torch
+
+import plain_qwen2
+import scenarios
+import tiny_models
+from torchlet_amd.cache.manager import OutOfPages
+from torchlet_amd.engine.batch import StepEntry
+from torchlet_amd.engine.engine import Engine
+from torchlet_amd.engine.loading import load_model, make_runner
+from torchlet_amd.engine.request import Request
+from torchlet_amd.sampling.sampler import draw_key
+
+
+def runner_for(folder, name, dtype="float32", pages=64, slots=4):
+    _, model = load_model(folder, dtype, device="cpu")
+    return make_runner(model, page_size=tiny_models.PAGE_SIZES[name], num_pages=pages, max_requests=slots)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("mode", ["whole", "portions", "mixed"])
+def test_step_function_equals_plain_under_every_split(cpu_ops, model_folders, name, mode):
+    cfg = json.loads((model_folders[name] / "config.json").read_text())
+    reqs = scenarios.make_requests(cfg["vocab_size"], [37, 5, 70, 18, 33], seed=5)
+    exp = scenarios.expected_logits(model_folders[name], reqs)
+    steps = scenarios.number(getattr(scenarios, mode)(reqs))
+    page = tiny_models.PAGE_SIZES[name]
+    runner = runner_for(model_folders[name], name, pages=-(-scenarios.max_tokens_needed(steps) // page) + 1)
+    out = {}
+    for s in steps:
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        if logits is not None:
+            out[s["step"]] = logits.numpy()
+        for r in s["end"]:
+            runner.release(r)
+        runner.cache.check()
+    scenarios.check(steps, out, exp, scenarios.FP32_TOL, f"{name}/{mode}")
+    assert runner.cache.live_requests() == []
+
+
+def test_step_refuses_bad_input_and_a_failed_step_leaves_no_trace(cpu_ops, model_folders):
+    runner = runner_for(model_folders["A"], "A", pages=3)          # 2 usable pages = 32 tokens
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        runner.step([StepEntry("a", [1, 256], [])])
+    with pytest.raises(ValueError, match="twice"):
+        runner.step([StepEntry("a", [1], []), StepEntry("a", [2], [])])
+    with pytest.raises(ValueError, match="wanted place"):
+        runner.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry("a", list(range(20)), []), StepEntry("b", list(range(20)), [])])
+    assert runner.cache.live_requests() == [] and runner.cache.free_pages() == [2]
+    with pytest.raises(ValueError, match="max_position_embeddings"):
+        runner_for(model_folders["A"], "A", pages=20).step([StepEntry("a", [1] * 129, [])])
+    assert runner.step([StepEntry("a", [1, 2, 3], [])]) is None     # nothing wanted: no logits
+    assert runner.step([StepEntry("a", [4], [0])]).shape == (1, 256)
+
+
+def _generate(engine, prompts, **kw):
+    reqs = [Request(prompt_tokens=p, seed=i, **kw) for i, p in enumerate(prompts)]
+    for r in reqs:
+        engine.add_request(r)
+    engine.run_until_done()
+    return reqs
+
+
+def test_greedy_generation_equals_the_plain_loop(cpu_ops, model_folders):
+    """Configuration A's workload: prompts of 5, 17 and 33 tokens, 8 greedy tokens each."""
+    cfg, w = plain_qwen2.load_folder(model_folders["A"])
+    prompts = list(scenarios.make_requests(cfg.vocab, [5, 17, 33], seed=2).values())
+    engine = Engine(runner_for(model_folders["A"], "A"), max_tokens_per_step=24)
+    reqs = _generate(engine, prompts, max_new_tokens=8)
+    for r, p in zip(reqs, prompts):
+        assert r.output_tokens == plain_qwen2.greedy(cfg, w, p, 8)
+    assert engine.runner.cache.live_requests() == []
+
+
+def test_temperature_sampling_is_the_same_alone_batched_and_after_preemption(cpu_ops, model_folders):
+    """Configuration B's workload: prompts of 1, 9, 40 and 64 tokens, temperature 0.8 with a
+    fixed sampler seed, 12 new tokens, arrivals at steps 0, 0, 3 and 5."""
+    cfg = json.loads((model_folders["B"] / "config.json").read_text())
+    prompts = list(scenarios.make_requests(cfg["vocab_size"], [1, 9, 40, 64], seed=3).values())
+    kw = dict(max_new_tokens=12, temperature=0.8)
+    alone = []
+    for i, p in enumerate(prompts):
+        e = Engine(runner_for(model_folders["B"], "B"), max_tokens_per_step=256, seed=42)
+        r = Request(prompt_tokens=p, seed=i, **kw)
+        e.add_request(r)
+        e.run_until_done()
+        alone.append(r.output_tokens)
+    assert len({tuple(a) for a in alone}) == 4 and all(len(a) == 12 for a in alone)
+
+    def staggered(pages, budget):
+        e = Engine(runner_for(model_folders["B"], "B", pages=pages), max_tokens_per_step=budget, seed=42)
+        reqs = [Request(prompt_tokens=p, seed=i, **kw) for i, p in enumerate(prompts)]
+        arrivals = {0: [0, 1], 3: [2], 5: [3]}
+        step = 0
+        while step < 6 or e.has_work():
+            for i in arrivals.get(step, []):
+                e.add_request(reqs[i])
+            if e.has_work():
+                e.step()
+            step += 1
+            e.runner.cache.check()
+        return e, reqs
+
+    e, reqs = staggered(pages=64, budget=16)                    # portions of at most 16 beside decode tokens
+    assert [r.output_tokens for r in reqs] == alone
+    e, reqs = staggered(pages=16, budget=32)                    # 15 pages of 8 = 120 tokens for 4 requests that want 150
+    assert e.scheduler.num_preemptions > 0
+    assert [r.output_tokens for r in reqs] == alone
+    assert e.runner.cache.free_pages() == [15]
+    other = Engine(runner_for(model_folders["B"], "B"), max_tokens_per_step=256, seed=43)
+    r = Request(prompt_tokens=prompts[1], seed=1, **kw)
+    other.add_request(r)
+    other.run_until_done()
+    assert r.output_tokens != alone[1]                          # another sampler seed, other draws
+
+
+def test_draw_keys_differ_in_every_argument():
+    keys = {draw_key(s, r, i) for s in (0, 1, 2 ** 40) for r in (0, 1, 2 ** 33) for i in range(4)}
+    assert len(keys) == 36 and all(-2 ** 31 <= k < 2 ** 31 for k in keys)
+
+
+def test_errors_fail_every_unfinished_request(cpu_ops, model_folders, monkeypatch):
+    engine = Engine(runner_for(model_folders["A"], "A"), max_tokens_per_step=64)
+    reqs = [Request(prompt_tokens=[1, 2, 3], max_new_tokens=4), Request(prompt_tokens=[4, 5], max_new_tokens=4)]
+    for r in reqs:
+        engine.add_request(r)
+    engine.step()
+    monkeypatch.setattr(engine.runner, "step", lambda entries: (_ for _ in ()).throw(RuntimeError("device lost")))
+    with pytest.raises(RuntimeError, match="device lost"):
+        engine.run_until_done()
+    assert all(isinstance(r.error, RuntimeError) and r.finish_reason == "error" for r in reqs)
+    assert engine.runner.cache.live_requests() == [] and not engine.has_work()
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        engine.add_request(Request(prompt_tokens=[999]))

@@ -1,0 +1,235 @@
+"""The Python entry point and the command line.
+
+In the manner of the reference's ``LLM`` (/root/reference/src/torchlet/
+v10_triton_paged_gqa/llm.py:20-110): ``LLM(model_id, max_decode_slots=4, kv_block_size=16,
+max_num_blocks=None)`` and ``generate(inputs, max_new_tokens=128)``, with the same names and
+meanings: ``max_decode_slots`` is the most requests live at a time, ``kv_block_size`` the
+tokens per cache page, ``max_num_blocks`` the pages of the pool including the sentinel
+(default ``max_decode_slots * ceil(max_position_embeddings / kv_block_size) + 1``,
+engine.py:40-47 of the reference, capped by free GPU memory).  ``model_id`` is a local
+model folder (nothing is downloaded).  Additions: ``dtype``, ``max_num_batched_tokens`` (the
+step's token budget), ``seed``; ``generate`` also takes ``temperature``, ``seed`` and
+``stop_token_ids``, and accepts prompts as lists of token ids, which bypass the tokenizer.
+
+Strings are wrapped as a single user turn and run through the tokenizer's chat template
+with the generation prompt (llm.py:87-96); the stop ids are the tokenizer's end-of-sequence
+id and ``<|im_end|>`` (llm.py:40-44); output text skips special tokens (engine.py:194-196).
+The tokenizer is read from the folder's ``tokenizer.json`` with the ``tokenizers`` library.
+
+    python -m torchlet_amd --model DIR --prompt "hello" --max-new-tokens 64
+    python -m torchlet_amd --model DIR --prompt-ids 1,2,3 --temperature 0.8 --seed 1
+    python -m torchlet_amd init --config config.json --seed 0 --out DIR     # random weights
+"""
+from __future__ import annotations
+
+import argparse
+import asyncio
+import json
+import math
+import sys
+from pathlib import Path
+
+import torch
+
+from .engine.engine import Engine
+from .engine.loading import load_model, make_runner, require_gpu
+from .engine.request import Request
+
+
+class LLM:
+    def __init__(self, model_id: str, max_decode_slots: int = 4, kv_block_size: int = 16,
+                 max_num_blocks: int | None = None, *, dtype: str = "bfloat16",
+                 max_num_batched_tokens: int = 2048, seed: int = 0):
+        self.device = require_gpu()
+        if kv_block_size <= 0:
+            raise ValueError("kv_block_size must be positive")
+        if max_decode_slots <= 0:
+            raise ValueError("max_decode_slots must be positive")
+        self.model_dir = Path(model_id)
+        self.config, self.model = load_model(self.model_dir, dtype, self.device)
+        spec = self.model.spec
+        blocks_per_request = math.ceil(spec.max_positions / kv_block_size)
+        if max_num_blocks is None:
+            max_num_blocks = max_decode_slots * blocks_per_request + 1
+            probe = make_runner(self.model, page_size=kv_block_size, num_pages=2, max_requests=1)
+            per_page = max(1, probe.cache.bytes_per_page())
+            del probe
+            free, _ = torch.cuda.mem_get_info(self.device)
+            max_num_blocks = max(2, min(max_num_blocks, int(free * 0.8) // per_page))
+        self.runner = make_runner(self.model, page_size=kv_block_size, num_pages=max_num_blocks,
+                                  max_requests=max_decode_slots)
+        self.engine = Engine(self.runner, max_tokens_per_step=max_num_batched_tokens, seed=seed)
+        self.tokenizer = _load_tokenizer(self.model_dir)
+        self.stop_ids = self._stop_ids()
+        self._next_seed = 0
+
+    def _stop_ids(self) -> frozenset:
+        ids = set()
+        eos = getattr(self.config, "eos_token_id", -1)
+        if isinstance(eos, int) and eos >= 0:
+            ids.add(eos)
+        if self.tokenizer is not None:
+            ids |= self.tokenizer.stop_ids()
+        return frozenset(ids)
+
+    def _requests(self, inputs, max_new_tokens, temperature, seed, stop_token_ids) -> list[Request]:
+        stop = self.stop_ids if stop_token_ids is None else frozenset(stop_token_ids)
+        reqs = []
+        for i, item in enumerate(inputs):
+            if isinstance(item, str):
+                if self.tokenizer is None:
+                    raise ValueError(f"{self.model_dir} has no tokenizer.json; give prompts as lists of token ids")
+                text, ids = self.tokenizer.encode_chat(item)
+            else:
+                text, ids = "", [int(t) for t in item]
+            if seed is None:
+                s, self._next_seed = self._next_seed, self._next_seed + 1
+            else:
+                s = int(seed) + i
+            reqs.append(Request(prompt_tokens=ids, max_new_tokens=max_new_tokens, temperature=float(temperature),
+                                seed=s, stop_token_ids=stop, prompt=text))
+        return reqs
+
+    def generate(self, inputs, max_new_tokens: int = 128, *, temperature: float = 0.0, seed: int | None = None,
+                 stop_token_ids=None):
+        """Generate for every input; strings give strings, token-id lists give token-id lists."""
+        if not inputs:
+            return []
+        if max_new_tokens <= 0:
+            return ["" if isinstance(x, str) else [] for x in inputs]
+        reqs = self._requests(inputs, max_new_tokens, temperature, seed, stop_token_ids)
+        for r in reqs:
+            self.engine.add_request(r)
+        self.engine.run_until_done()
+        return self._outputs(inputs, reqs)
+
+    async def generate_async(self, inputs, max_new_tokens: int = 128, **kw):
+        """Coroutine form, as the reference's ``generate`` is from its fourth version on:
+        requests of concurrent callers share the engine's steps (continuous batching)."""
+        if not inputs:
+            return []
+        if max_new_tokens <= 0:
+            return ["" if isinstance(x, str) else [] for x in inputs]
+        reqs = self._requests(inputs, max_new_tokens, kw.get("temperature", 0.0), kw.get("seed"), kw.get("stop_token_ids"))
+        for r in reqs:
+            self.engine.add_request(r)
+        while any(r.finish_reason is None for r in reqs):
+            try:
+                self.engine.step()
+            except Exception as exc:
+                self.engine.scheduler.fail_all(exc)
+                raise
+            await asyncio.sleep(0)
+        self.engine.scheduler.drain_finished()
+        return self._outputs(inputs, reqs)
+
+    def _outputs(self, inputs, reqs):
+        out = []
+        for item, r in zip(inputs, reqs):
+            if r.error is not None:
+                raise r.error
+            if isinstance(item, str):
+                r.output = self.tokenizer.decode(r.output_tokens)
+                out.append(r.output)
+            else:
+                out.append(list(r.output_tokens))
+        return out
+
+
+class _Tokenizer:
+    """``tokenizer.json`` through the ``tokenizers`` library, plus the folder's chat template."""
+
+    def __init__(self, folder: Path):
+        from tokenizers import Tokenizer
+        self.tok = Tokenizer.from_file(str(folder / "tokenizer.json"))
+        cfg_path = folder / "tokenizer_config.json"
+        self.cfg = json.loads(cfg_path.read_text()) if cfg_path.exists() else {}
+        self.template = self.cfg.get("chat_template")
+
+    def _token_text(self, key):
+        v = self.cfg.get(key)
+        return v.get("content") if isinstance(v, dict) else v
+
+    def stop_ids(self) -> set:
+        ids = set()
+        for text in (self._token_text("eos_token"), "<|im_end|>"):
+            if text:
+                i = self.tok.token_to_id(text)
+                if i is not None:
+                    ids.add(i)
+        return ids
+
+    def encode_chat(self, user_text: str):
+        if self.template:
+            import jinja2
+            env = jinja2.Environment(trim_blocks=True, lstrip_blocks=True)
+            text = env.from_string(self.template).render(
+                messages=[{"role": "user", "content": user_text}], add_generation_prompt=True,
+                bos_token=self._token_text("bos_token") or "", eos_token=self._token_text("eos_token") or "")
+        else:
+            text = user_text
+        return text, self.tok.encode(text, add_special_tokens=False).ids
+
+    def decode(self, ids) -> str:
+        return self.tok.decode(list(ids), skip_special_tokens=True)
+
+
+def _load_tokenizer(folder: Path):
+    return _Tokenizer(folder) if (folder / "tokenizer.json").exists() else None
+
+
+# ------------------------------------------------------------------------ command line
+
+def _parser():
+    p = argparse.ArgumentParser(prog="python -m torchlet_amd", description="Qwen2.5 inference on one MI355X")
+    sub = p.add_subparsers(dest="command")
+    g = sub.add_parser("generate", help="generate from prompts (the default command)")
+    for q in (p, g):
+        q.add_argument("--model", help="model folder: config.json, *.safetensors, optionally tokenizer.json")
+        q.add_argument("--prompt", action="append", default=[], help="a prompt string (repeatable)")
+        q.add_argument("--prompt-ids", action="append", default=[], help="a prompt as comma-separated token ids (repeatable)")
+        q.add_argument("--max-new-tokens", type=int, default=128)
+        q.add_argument("--temperature", type=float, default=0.0, help="0: greedy")
+        q.add_argument("--seed", type=int, default=0, help="sampler seed")
+        q.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+        q.add_argument("--max-decode-slots", type=int, default=4)
+        q.add_argument("--kv-block-size", type=int, default=16)
+        q.add_argument("--max-num-blocks", type=int, default=None)
+        q.add_argument("--max-num-batched-tokens", type=int, default=2048)
+    i = sub.add_parser("init", help="write a model folder with random weights from a configuration and a seed")
+    i.add_argument("--config", required=True, help="a config.json")
+    i.add_argument("--seed", type=int, default=0)
+    i.add_argument("--out", required=True)
+    i.add_argument("--store-dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    return p
+
+
+def main(argv=None) -> int:
+    args = _parser().parse_args(argv)
+    if args.command == "init":
+        from .engine.loading import parse_dtype
+        from .registry import config_class
+        from .weights.random_init import write_model_folder
+        d = json.loads(Path(args.config).read_text())
+        cfg = config_class(d["architectures"][0]).from_dict(d)
+        folder = write_model_folder(cfg, args.seed, args.out, parse_dtype(args.store_dtype))
+        print(folder)
+        return 0
+    if not args.model:
+        print("--model is required", file=sys.stderr)
+        return 2
+    prompts = list(args.prompt) + [[int(t) for t in s.split(",") if t.strip()] for s in args.prompt_ids]
+    if not prompts:
+        print("give at least one --prompt or --prompt-ids", file=sys.stderr)
+        return 2
+    llm = LLM(args.model, max_decode_slots=args.max_decode_slots, kv_block_size=args.kv_block_size,
+              max_num_blocks=args.max_num_blocks, dtype=args.dtype,
+              max_num_batched_tokens=args.max_num_batched_tokens, seed=args.seed)
+    outputs = llm.generate(prompts, max_new_tokens=args.max_new_tokens, temperature=args.temperature, seed=0)
+    for prompt, out in zip(prompts, outputs):
+        print(json.dumps({"prompt": prompt, "output": out}))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

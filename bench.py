@@ -107,7 +107,7 @@ def time_decode(model, batch: int, steps: int, warmup: int):
     from torchlet_amd.sampling.sampler import Sampler
 
     pages = batch * (-(-(CONTEXT + steps + warmup + 1) // PAGE)) + 1
-    runner = make_runner(model, page_size=PAGE, num_pages=pages, max_requests=batch)
+    runner = make_runner(model, page_size=PAGE, num_pages=pages, max_requests=batch, use_graphs=True)
     ids = [f"b{i}" for i in range(batch)]
     fill_context(runner, ids, CONTEXT)
     sampler = Sampler(0)

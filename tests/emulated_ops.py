@@ -38,7 +38,7 @@ def add_rmsnorm(residual, pending, weight, eps, out, rows=None):
     out.copy_(y.to(out.dtype))
 
 
-def linear(x, weight, bias, out):
+def linear(x, weight, bias, out, general=False):
     y = x.float() @ weight.float().T
     if bias is not None:
         y = y + bias.float()

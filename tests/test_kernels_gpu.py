@@ -98,6 +98,34 @@ def test_linear(ops, dtype, M, N, K, bias):
     torch.testing.assert_close(out32.double(), ref, **tol32)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(48, 64), (129, 200), (4608, 3584), (3584, 1000), (16400, 256), (33000, 128)])
+def test_linear_few_rows_on_matrix_cores(ops, out_dtype, M, N, K):
+    """The weight-streaming kernel of the decode step: every choice of strips per wave and of
+    waves along K, tails in M, N and K, against a float64 product of the same bfloat16 values."""
+    g = torch.Generator().manual_seed(M * 7 + N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).cuda()
+    b = torch.randn(N, generator=g).to(torch.bfloat16).cuda()
+    ref = x.double() @ w.double().T + b.double()
+    out = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
+    ops.linear(x, w, b, out)
+    # products of bfloat16 values are exact in 32-bit; only the sums round
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    torch.testing.assert_close(out.double(), ref, **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
+    # the same through the general kernel: both are the engine's answer for some shape
+    gen = torch.empty_like(out)
+    ops.linear(x, w, b, gen, general=True)
+    torch.testing.assert_close(out.double(), gen.double(), **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
+    # a strided input view with aligned rows
+    wide = torch.zeros(M, K + 40, dtype=torch.bfloat16, device="cuda")
+    wide[:, 8:8 + K] = x
+    out2 = torch.empty_like(out)
+    ops.linear(wide[:, 8:8 + K], w, None, out2)
+    torch.testing.assert_close(out2.double(), ref - b.double(), **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
+
+
 def _rope_ref(x, pos, theta):
     """x [T, heads, hd] float64; split-half pairing."""
     hd = x.shape[-1]

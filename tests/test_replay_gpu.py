@@ -84,3 +84,27 @@ def test_trace_run_program(model_folders, expected, tmp_path):
         vocab = len(next(iter(exp.values()))[0])
         out = {int(p.stem): np.fromfile(p, dtype="<f4").reshape(-1, vocab) for p in out_dir.glob("*.f32")}
         scenarios.check(steps, out, exp, TOL[dtype], f"trace_run/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_decode_steps_replayed_as_graphs(model_folders, expected, name, dtype):
+    """Decode-only steps under captured HIP graphs: every replay is checked against the plain
+    implementation, with eager steps (prompt portions, other batch widths) and synchronizations
+    between the replays, requests joining and leaving, and pages reused."""
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import load_model, make_runner
+    reqs, exp = expected(name)
+    steps = scenarios.number(scenarios.mixed(reqs, seed=5, prompt_fraction=0.3))
+    page = tiny_models.PAGE_SIZES[name]
+    _, model = load_model(model_folders[name], dtype)
+    runner = make_runner(model, page_size=page, num_pages=-(-scenarios.max_tokens_needed(steps) // page) + 1,
+                         max_requests=4, use_graphs=True)
+    out = {}
+    for s in steps:
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        out[s["step"]] = logits.cpu().numpy()
+        for r in s["end"]:
+            runner.release(r)
+    assert runner.graph_replays >= 20 and len(runner._graphs) >= 2
+    scenarios.check(steps, out, exp, TOL[dtype], f"graphs/{name}/{dtype}")

@@ -86,3 +86,206 @@ extern "C" int tl_gemm_general(const void* x, const void* w, const void* bias, i
     TL_CHECK_LAUNCH("gemm_general");
     return TL_OK;
 }
+
+
+// =====================================================================================
+// bfloat16 on the matrix cores, few rows (M <= 64): the decode step's products.
+//
+// Such a product is a stream of the weight matrix through the chip once; the kernel is
+// built so that nothing but HBM limits it.  out^T tile = W tile * x^T on
+// v_mfma_f32_16x16x32_bf16: the A operand is 16 rows of W, the B operand 16 rows of x, both
+// read straight from memory as 16-byte pieces of a K-contiguous row (no shared-memory
+// staging, no barrier in the loop).  A wave owns R strips of 16 weight rows and MT tiles of
+// 16 activation rows and walks K in steps of 64: lane group g = lane / 16 reads the 32
+// contiguous bytes k = 64 s + 16 g .. + 16 of its row, so the four groups of a row consume
+// one full 128-byte line; the two 16-byte halves feed two MFMAs (how k is dealt to lanes is
+// free as long as A and B agree).  The KS waves of a work-group take the steps s = wave,
+// wave + KS, ... and add their partial tiles through shared memory in a fixed order, so
+// the result is deterministic.  x is small and stays in L2.
+// Needs K % 8 == 0 and 16-byte aligned rows; other shapes go to the general kernel.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+union Frag16 {          // 16 bytes: eight bfloat16 as the MFMA wants them, or one 128-bit load
+    uint4 u;
+    bf16x8_t v;
+};
+
+template <int R, int MT, int KS, typename TOut>
+__global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                              const void* __restrict__ bias, int bias_f32,
+                                                              TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+    __shared__ float red[KS > 1 ? KS * R * MT * 256 : 1];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int li = lane & 15, lg = lane >> 4;
+    const int n0 = blockIdx.x * (16 * R);
+
+    const bf16_t* wrow[R];
+    const bf16_t* xrow[MT];
+#pragma unroll
+    for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + li, N - 1) * K;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) xrow[t] = x + (size_t)min(t * 16 + li, M - 1) * ldx;
+
+    f32x4_t acc[R][MT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    const int full = K / 64;                   // steps that lie wholly inside K
+    Frag16 a0[R], a1[R], b0[MT], b1[MT];
+    int s = wave;
+    if (s < full) {
+        const int k = 64 * s + 16 * lg;
+#pragma unroll
+        for (int r = 0; r < R; ++r) { a0[r].u = *(const uint4*)(wrow[r] + k); a1[r].u = *(const uint4*)(wrow[r] + k + 8); }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) { b0[t].u = *(const uint4*)(xrow[t] + k); b1[t].u = *(const uint4*)(xrow[t] + k + 8); }
+    }
+    for (; s < full; s += KS) {
+        // fetch the next step (the last one fetches itself again: no branch in the loop)
+        Frag16 na0[R], na1[R], nb0[MT], nb1[MT];
+        const int sn = (s + KS < full) ? s + KS : s;
+        const int kn = 64 * sn + 16 * lg;
+#pragma unroll
+        for (int r = 0; r < R; ++r) { na0[r].u = *(const uint4*)(wrow[r] + kn); na1[r].u = *(const uint4*)(wrow[r] + kn + 8); }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) { nb0[t].u = *(const uint4*)(xrow[t] + kn); nb1[t].u = *(const uint4*)(xrow[t] + kn + 8); }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[r].v, b0[t].v, acc[r][t], 0, 0, 0);
+                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[r].v, b1[t].v, acc[r][t], 0, 0, 0);
+            }
+#pragma unroll
+        for (int r = 0; r < R; ++r) { a0[r] = na0[r]; a1[r] = na1[r]; }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) { b0[t] = nb0[t]; b1[t] = nb1[t]; }
+    }
+    // the tail step (K % 64 != 0) belongs to the wave whose turn it is; pieces beyond K count as zero
+    if ((K & 63) && (full % KS) == wave) {
+        const int k = 64 * full + 16 * lg;
+        const bool v0 = k + 8 <= K, v1 = k + 16 <= K;
+        const uint4 zero = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            a0[r].u = v0 ? *(const uint4*)(wrow[r] + k) : zero;
+            a1[r].u = v1 ? *(const uint4*)(wrow[r] + k + 8) : zero;
+        }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            b0[t].u = v0 ? *(const uint4*)(xrow[t] + k) : zero;
+            b1[t].u = v1 ? *(const uint4*)(xrow[t] + k + 8) : zero;
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[r].v, b0[t].v, acc[r][t], 0, 0, 0);
+                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[r].v, b1[t].v, acc[r][t], 0, 0, 0);
+            }
+    }
+
+    // D[i][j]: lane holds i = 4 * (lane / 16) + v (weight row), j = lane % 16 (activation row)
+    if (KS > 1) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                float* dst = red + ((size_t)(wave * R * MT + r * MT + t) * 64 + lane) * 4;
+                *(f32x4_t*)dst = acc[r][t];
+            }
+        __syncthreads();
+    }
+    for (int tile = wave; tile < R * MT; tile += KS) {
+        const int r = tile / MT, t = tile % MT;
+        f32x4_t sum;
+        if (KS > 1) {
+            sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int wv = 0; wv < KS; ++wv) sum += *(const f32x4_t*)(red + ((size_t)(wv * R * MT + tile) * 64 + lane) * 4);
+        } else {
+            sum = acc[0][0];
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+                for (int tt = 0; tt < MT; ++tt)
+                    if (rr == r && tt == t) sum = acc[rr][tt];
+        }
+        const int m = t * 16 + li;
+        const int n = n0 + r * 16 + 4 * lg;
+        if (m < M) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                if (n + v < N) {
+                    float val = sum[v];
+                    if (bias) val += load_vec(bias, bias_f32, n + v);
+                    out[(size_t)m * ldo + n + v] = from_float<TOut>(val);
+                }
+            }
+        }
+    }
+}
+
+template <int R, int MT, int KS>
+static void launch_skinny(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                          int ldx, int ldo, int out_f32, hipStream_t stream) {
+    dim3 grid((N + 16 * R - 1) / (16 * R)), block(KS * 64);
+    if (out_f32)
+        gemm_skinny_kernel<R, MT, KS, float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo);
+    else
+        gemm_skinny_kernel<R, MT, KS, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo);
+}
+
+template <int MT>
+static void pick_skinny(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                        int ldx, int ldo, int out_f32, hipStream_t stream) {
+    // Enough work-groups to fill 256 compute units a few times over, and enough K steps per
+    // wave to keep loads in flight: wide matrices take two strips per wave and four waves
+    // along K, narrow ones one strip and eight waves.
+    const int strips = (N + 15) / 16;
+    if (strips >= 2048 && MT <= 2) launch_skinny<4, MT, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else if (strips >= 1024) launch_skinny<2, MT, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else launch_skinny<1, MT, 8>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+}
+
+// One named instance of the few-rows kernel (tests cover every instance; tuning times them).
+extern "C" int tl_gemm_skinny_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
+                                      int M, int N, int K, int ldx, int ldo, int out_f32, int R, int KS, hipStream_t stream) {
+    TL_REQUIRE(M > 0 && M <= 64 && K % 8 == 0 && ldx % 8 == 0, "gemm_skinny: needs 0 < M <= 64 and K, ldx multiples of 8");
+    const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+#define TL_SKINNY_CASE(r, t, k) \
+    if (R == r && MT == t && KS == k) { launch_skinny<r, t, k>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream); TL_CHECK_LAUNCH("gemm_skinny"); return TL_OK; }
+    TL_SKINNY_CASE(1, 1, 4) TL_SKINNY_CASE(1, 2, 4) TL_SKINNY_CASE(1, 4, 4)
+    TL_SKINNY_CASE(2, 1, 4) TL_SKINNY_CASE(2, 2, 4) TL_SKINNY_CASE(2, 4, 4)
+    TL_SKINNY_CASE(4, 1, 4) TL_SKINNY_CASE(4, 2, 4) TL_SKINNY_CASE(4, 4, 4)
+    TL_SKINNY_CASE(1, 1, 8) TL_SKINNY_CASE(1, 2, 8) TL_SKINNY_CASE(1, 4, 8)
+    TL_SKINNY_CASE(2, 1, 8) TL_SKINNY_CASE(2, 2, 8) TL_SKINNY_CASE(2, 4, 8)
+    TL_SKINNY_CASE(1, 1, 16) TL_SKINNY_CASE(1, 2, 16) TL_SKINNY_CASE(1, 4, 16)
+    TL_SKINNY_CASE(1, 1, 2) TL_SKINNY_CASE(2, 1, 2) TL_SKINNY_CASE(4, 1, 2) TL_SKINNY_CASE(4, 4, 2) TL_SKINNY_CASE(2, 4, 2)
+#undef TL_SKINNY_CASE
+    TL_REQUIRE(false, "gemm_skinny: no instance R=%d MT=%d KS=%d", R, MT, KS);
+}
+
+static bool skinny_fits(const void* x, const void* w, int M, int K, int ldx) {
+    return M <= 64 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
+}
+
+// out = x w^T (+ bias) in the engine's dtype: picks the kernel for the shape.
+//   bfloat16, M <= 64, aligned  -> gemm_skinny (matrix cores, weight streaming)
+//   everything else             -> gemm_tile (true 32-bit arithmetic)
+extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_f32, void* out,
+                       int M, int N, int K, int ldx, int ldo, int dtype, int out_f32, hipStream_t stream) {
+    TL_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldo >= N, "gemm: bad sizes M=%d N=%d K=%d ldx=%d ldo=%d", M, N, K, ldx, ldo);
+    if (M == 0) return TL_OK;
+    if (dtype == TL_DT_BF16 && skinny_fits(x, w, M, K, ldx)) {
+        if (M <= 16) pick_skinny<1>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        else if (M <= 32) pick_skinny<2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        else pick_skinny<4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        TL_CHECK_LAUNCH("gemm_skinny");
+        return TL_OK;
+    }
+    return tl_gemm_general(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, dtype, out_f32, stream);
+}

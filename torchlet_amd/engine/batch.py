@@ -109,3 +109,73 @@ class StepContext:
             v = self._upload({"r": tr, "t": t0})
             t = self._tiles[tq] = (v["r"], v["t"], len(tr))
         return t
+
+
+class StaticDecodeContext:
+    """A step context of fixed shape for decode-only steps: ``width`` requests with one new
+    token each and block tables of ``blocks`` entries, living in one static device buffer
+    that is refilled before every step (one copy from pinned host memory).  Because no
+    address or launch size changes between steps, the model's forward pass over it can be
+    captured once as a HIP graph and replayed.  Unused rows are padded with requests of
+    length zero whose block tables point at the sentinel page.
+    """
+
+    def __init__(self, *, width: int, blocks: int, num_groups: int, tile_sizes, page_size: int, device):
+        S = width
+        self.width = S
+        self.blocks = blocks
+        self.num_tokens = S
+        self.num_requests = S
+        self.num_wanted = S
+        self.max_total_len = blocks * page_size       # an upper bound: fixes the attention's split count
+        self.max_new_tokens = 1
+        self.decode_only = True
+        self.device = device
+        sizes = {"token_ids": S, "positions": S, "ctx_lens": S, "slots": S, "token_req": S, "req_indptr": S + 1,
+                 "want_rows": S, "tile_req": S, "tile_tok0": S}
+        for g in range(num_groups):
+            sizes[f"bt{g}"] = S * blocks
+        self._offsets, total = {}, 0
+        for k, n in sizes.items():
+            self._offsets[k] = (total, n)
+            total += -(-n // 4) * 4
+        self._host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self._np = self._host.numpy()
+        self._dev = torch.zeros(total, dtype=torch.int32, device=device)
+        ar = np.arange(S + 1, dtype=np.int32)
+        self._set("token_req", ar[:S])
+        self._set("req_indptr", ar)
+        self._set("want_rows", ar[:S])
+        self._set("tile_req", ar[:S])
+        v = {k: self._dev[o: o + n] for k, (o, n) in self._offsets.items()}
+        self.token_ids, self.positions, self.ctx_lens, self.slots = v["token_ids"], v["positions"], v["ctx_lens"], v["slots"]
+        self.token_req, self.req_indptr, self.want_rows = v["token_req"], v["req_indptr"], v["want_rows"]
+        self.block_tables = [v[f"bt{g}"].view(S, blocks) for g in range(num_groups)]
+        self._tile = (v["tile_req"], v["tile_tok0"], S)
+        self._dev.copy_(self._host)
+        self._copied = torch.cuda.Event() if torch.device(device).type == "cuda" else None
+
+    def _set(self, key: str, values) -> None:
+        o, n = self._offsets[key]
+        self._np[o: o + n] = 0
+        self._np[o: o + len(values)] = values
+
+    def tiles(self, tq: int):
+        return self._tile                 # one token per request: a tile per request whatever its height
+
+    def fill(self, *, token_ids, ctx_lens, slots, block_tables) -> None:
+        """New tokens, lengths and block-table rows of the live requests (``<= width``)."""
+        if self._copied is not None:
+            self._copied.synchronize()        # the previous copy has read the pinned buffer
+        self._set("token_ids", token_ids)
+        self._set("positions", ctx_lens)
+        self._set("ctx_lens", ctx_lens)
+        self._set("slots", slots)
+        for g, bt in enumerate(block_tables):
+            o, n = self._offsets[f"bt{g}"]
+            dst = self._np[o: o + n].reshape(self.width, self.blocks)
+            dst[:] = 0
+            dst[: bt.shape[0], : bt.shape[1]] = bt
+        self._dev.copy_(self._host, non_blocking=True)
+        if self._copied is not None:
+            self._copied.record()

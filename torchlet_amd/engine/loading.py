@@ -56,7 +56,8 @@ def load_model(folder: str | Path, dtype="bfloat16", device=None) -> tuple[Model
     return config, build_model(config, dtype, device, folder=folder)
 
 
-def make_runner(model: DecoderModel, *, page_size: int, num_pages: int, max_requests: int) -> ModelRunner:
+def make_runner(model: DecoderModel, *, page_size: int, num_pages: int, max_requests: int,
+                use_graphs: bool = False) -> ModelRunner:
     cache = CacheManager(model.cache_plan(), page_size=page_size, num_pages=num_pages,
                          max_requests=max_requests, dtype=model.dtype, device=model.device)
-    return ModelRunner(model, cache)
+    return ModelRunner(model, cache, use_graphs=use_graphs)

@@ -10,11 +10,32 @@ from __future__ import annotations
 import torch
 
 from ..cache.manager import CacheManager, OutOfPages
-from .batch import StepContext, StepEntry
+from .batch import StaticDecodeContext, StepContext, StepEntry
+
+
+def _next_pow2(n: int) -> int:
+    return 1 << max(0, (n - 1).bit_length())
+
+
+class _DecodeGraph:
+    """The forward pass over a :class:`StaticDecodeContext`, captured as a HIP graph."""
+
+    def __init__(self, ctx: StaticDecodeContext):
+        self.ctx = ctx
+        self.graph: torch.cuda.CUDAGraph | None = None
+        self.logits: torch.Tensor | None = None
 
 
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager):
+    """``use_graphs``: decode-only steps (one new token for every request) run from static
+    buffers under a captured HIP graph, one graph per (batch width, context length) bucket,
+    as the reference replays its decode step as a CUDA graph
+    (/root/reference/src/torchlet/v10_triton_paged_gqa/engine.py:137-185).  A bucket's first
+    step runs eagerly from the static buffers and is then captured; capture records without
+    running, so results are only ever read after an eager run or a replay (the reference
+    reads its output buffer right after capture, engine.py:165-176)."""
+
+    def __init__(self, model, cache: CacheManager, use_graphs: bool = False, max_graph_width: int = 256):
         self.model = model
         self.cache = cache
         self.device = model.device
@@ -22,6 +43,10 @@ class ModelRunner:
         self.tile_sizes = model.tile_token_sizes()
         self.max_positions = model.spec.max_positions
         self.vocab_size = model.spec.vocab_size
+        self.use_graphs = use_graphs and torch.device(self.device).type == "cuda" and model.graph_safe()
+        self.max_graph_width = max_graph_width
+        self._graphs: dict[tuple[int, int], _DecodeGraph] = {}
+        self.graph_replays = 0
 
     def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
         """Logits ``[number of wanted places, vocab]`` (float32, on the GPU), in the order
@@ -73,6 +98,12 @@ class ModelRunner:
 
         req_ids = [e.req_id for e in entries]
         blocks = -(-max(c + n for c, n in zip(ctx_lens, new_lens)) // cache.page_size)
+        if (self.use_graphs and max(new_lens) == 1 and len(entries) <= self.max_graph_width
+                and all(e.want == [0] for e in entries)):
+            logits = self._graph_step(entries, req_ids, ctx_lens, blocks)
+            for e, c in zip(entries, ctx_lens):
+                cache.commit(e.req_id, c + 1)
+            return logits
         token_ids, want_rows, base = [], [], 0
         for e in entries:
             token_ids.extend(e.tokens)
@@ -87,6 +118,33 @@ class ModelRunner:
         for e, c, n in zip(entries, ctx_lens, new_lens):
             cache.commit(e.req_id, c + n)
         return logits
+
+    def _graph_step(self, entries, req_ids, ctx_lens, blocks) -> torch.Tensor:
+        cache = self.cache
+        width = _next_pow2(len(entries))
+        most = -(-self.max_positions // cache.page_size)
+        bucket = min(most, max(_next_pow2(blocks), min(most, 256 // cache.page_size or 1)))
+        key = (width, bucket)
+        dg = self._graphs.get(key)
+        if dg is None:
+            dg = self._graphs[key] = _DecodeGraph(StaticDecodeContext(
+                width=width, blocks=bucket, num_groups=len(cache.groups), tile_sizes=self.tile_sizes,
+                page_size=cache.page_size, device=self.device))
+        dg.ctx.fill(token_ids=[e.tokens[0] for e in entries], ctx_lens=ctx_lens,
+                    slots=[cache.slot(r) for r in req_ids],
+                    block_tables=[cache.block_table(g, req_ids, bucket) for g in range(len(cache.groups))])
+        if dg.graph is None:
+            logits = self.model.forward(dg.ctx, self.caches)          # eager: this step's result
+            result = logits[: len(entries)].clone()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):                             # records, does not run
+                dg.logits = self.model.forward(dg.ctx, self.caches)
+            dg.graph = graph
+            return result
+        dg.graph.replay()
+        self.graph_replays += 1
+        return dg.logits[: len(entries)]
 
     def release(self, req_id) -> None:
         if self.cache.has(req_id):

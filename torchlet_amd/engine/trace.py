@@ -35,6 +35,7 @@ def parse_args(argv=None):
                    help="most tokens live requests hold at any time (each rounded up to whole pages)")
     p.add_argument("--page-size", type=int, default=16, help="tokens per cache page (default 16)")
     p.add_argument("--max-requests", type=int, default=8, help="most requests live at a time (default 8)")
+    p.add_argument("--graphs", action="store_true", help="replay decode-only steps as captured HIP graphs")
     return p.parse_args(argv)
 
 
@@ -48,7 +49,8 @@ def run(args, lines, out=sys.stdout) -> int:
     out_dir.mkdir(parents=True, exist_ok=True)
     _, model = load_model(args.model, args.dtype)
     pages = -(-args.max_tokens // args.page_size) + 1          # + the sentinel page
-    runner = make_runner(model, page_size=args.page_size, num_pages=pages, max_requests=args.max_requests)
+    runner = make_runner(model, page_size=args.page_size, num_pages=pages, max_requests=args.max_requests,
+                         use_graphs=args.graphs)
     for line in lines:
         line = line.strip()
         if not line:

@@ -131,9 +131,11 @@ def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: to
                                    _ptr(rows), c_int(n), c_int(H), c_int(_dt(out, "add_rmsnorm")), _stream()))
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor) -> None:
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor,
+           general: bool = False) -> None:
     """``out = x @ weight.T (+ bias)``; ``x [M, K]`` (rows may be strided), ``weight [N, K]``
-    contiguous and of ``x``'s dtype, ``out [M, N]`` of that dtype or float32."""
+    contiguous and of ``x``'s dtype, ``out [M, N]`` of that dtype or float32.  The library picks
+    the kernel for the shape; ``general=True`` forces the general 32-bit-arithmetic kernel."""
     M, K = x.shape
     N, K2 = weight.shape
     if K2 != K or out.shape != (M, N):
@@ -144,9 +146,24 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out
         raise KernelError(f"linear: out dtype {out.dtype} must be {x.dtype} or float32")
     bf = _vec(bias, N, "linear bias")
     lib = _lib("gemm")
-    _check(lib, lib.tl_gemm_general(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N), c_int(K),
+    entry = lib.tl_gemm_general if general else lib.tl_gemm
+    _check(lib, entry(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N), c_int(K),
                                     c_int(x.stride(0)), c_int(out.stride(0)), c_int(_dt(x, "linear")),
                                     c_int(1 if out.dtype == torch.float32 else 0), _stream()))
+
+
+def linear_few_rows_variant(x, weight, bias, out, strips_per_wave: int, waves_along_k: int) -> None:
+    """One named instance of the few-rows matrix-core kernel (for tests and tuning)."""
+    M, K = x.shape
+    N = weight.shape[0]
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or out.shape != (M, N) or not weight.is_contiguous():
+        raise KernelError("linear_few_rows_variant: bfloat16 operands and fitting shapes only")
+    bf = _vec(bias, N, "linear bias")
+    lib = _lib("gemm")
+    _check(lib, lib.tl_gemm_skinny_variant(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N),
+                                           c_int(K), c_int(x.stride(0)), c_int(out.stride(0)),
+                                           c_int(1 if out.dtype == torch.float32 else 0), c_int(strips_per_wave),
+                                           c_int(waves_along_k), _stream()))
 
 
 def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int, rot_heads: int,

@@ -8,7 +8,7 @@ tokens per cache page, ``max_num_blocks`` the pages of the pool including the se
 (default ``max_decode_slots * ceil(max_position_embeddings / kv_block_size) + 1``,
 engine.py:40-47 of the reference, capped by free GPU memory).  ``model_id`` is a local
 model folder (nothing is downloaded).  Additions: ``dtype``, ``max_num_batched_tokens`` (the
-step's token budget), ``seed``; ``generate`` also takes ``temperature``, ``seed`` and
+step's token budget), ``seed``, ``use_graphs`` (decode-only steps replay a captured HIP graph); ``generate`` also takes ``temperature``, ``seed`` and
 ``stop_token_ids``, and accepts prompts as lists of token ids, which bypass the tokenizer.
 
 Strings are wrapped as a single user turn and run through the tokenizer's chat template
@@ -39,7 +39,7 @@ from .engine.request import Request
 class LLM:
     def __init__(self, model_id: str, max_decode_slots: int = 4, kv_block_size: int = 16,
                  max_num_blocks: int | None = None, *, dtype: str = "bfloat16",
-                 max_num_batched_tokens: int = 2048, seed: int = 0):
+                 max_num_batched_tokens: int = 2048, seed: int = 0, use_graphs: bool = True):
         self.device = require_gpu()
         if kv_block_size <= 0:
             raise ValueError("kv_block_size must be positive")
@@ -57,7 +57,7 @@ class LLM:
             free, _ = torch.cuda.mem_get_info(self.device)
             max_num_blocks = max(2, min(max_num_blocks, int(free * 0.8) // per_page))
         self.runner = make_runner(self.model, page_size=kv_block_size, num_pages=max_num_blocks,
-                                  max_requests=max_decode_slots)
+                                  max_requests=max_decode_slots, use_graphs=use_graphs)
         self.engine = Engine(self.runner, max_tokens_per_step=max_num_batched_tokens, seed=seed)
         self.tokenizer = _load_tokenizer(self.model_dir)
         self.stop_ids = self._stop_ids()

@@ -65,6 +65,10 @@ class DecoderModel:
     def tile_token_sizes(self) -> set[int]:
         return {b.mixer.tile_tokens for b in self.blocks if hasattr(b.mixer, "tile_tokens")}
 
+    def graph_safe(self) -> bool:
+        """Every mixer runs from device-side metadata only, so a step can be captured as a graph."""
+        return all(getattr(b.mixer, "graph_safe", False) for b in self.blocks)
+
     def kernel_libraries(self) -> list[str]:
         libs = ["elementwise", "gemm", "sampling"]
         for b in self.blocks:

@@ -25,6 +25,8 @@ _MIN_KEYS_PER_SPLIT = 256
 
 @MIXERS.register("gqa_attention")
 class GQAttention(Mixer):
+    graph_safe = True       # nothing in forward() depends on host-side values of the step
+
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         if spec.num_heads % spec.num_kv_heads:

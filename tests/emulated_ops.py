@@ -63,11 +63,11 @@ def rope_cache_write(qkv, q_heads, kv_heads, head_dim, rot_heads, positions, inv
             p = int(positions[t])
             page = int(block_table[int(token_req[t]), p // page_size])
             k_plane[page, :, p % page_size] = k[t]
-            v_plane[page, :, p % page_size] = v[t]
+            v_plane[page, :, :, p % page_size] = v[t]
 
 
 def paged_attention(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles,
-                    tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale, splits=1):
+                    tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale, splits=1, general=False):
     group = num_heads // num_kv_heads
     covered = torch.zeros(q.shape[0], dtype=torch.bool)
     for tile in range(num_tiles):
@@ -79,7 +79,7 @@ def paged_attention(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens,
             keys = torch.arange(lo, pos + 1)
             pages = block_table[r, keys // page_size].long()
             k = k_plane[pages, :, keys % page_size].float()       # [n, kvh, hd]
-            v = v_plane[pages, :, keys % page_size].float()
+            v = v_plane[pages, :, :, keys % page_size].float()
             qi = q[first + i].float().view(num_heads, head_dim)
             kk = k.repeat_interleave(group, dim=1)
             vv = v.repeat_interleave(group, dim=1)

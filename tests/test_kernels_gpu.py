@@ -153,7 +153,7 @@ def test_rope_cache_write(ops, dtype, nh, nkv, hd, page, theta):
     j = torch.arange(0, hd, 2, dtype=torch.float32)
     inv_freq = (1.0 / (theta ** (j / hd)))
     kp = torch.zeros(pages, nkv, page, hd, dtype=dtype)
-    vp = torch.zeros_like(kp)
+    vp = torch.zeros(pages, nkv, hd, page, dtype=dtype)         # values lie transposed inside a page
     d_qkv, d_kp, d_vp = qkv.cuda(), kp.cuda(), vp.cuda()
     ops.rope_cache_write(d_qkv, nh, nkv, hd, nh + nkv, positions.cuda(), inv_freq.cuda(), token_req.cuda(), bt.cuda(), d_kp, d_vp, page)
     x = qkv.double().view(T, nh + 2 * nkv, hd)
@@ -162,11 +162,11 @@ def test_rope_cache_write(ops, dtype, nh, nkv, hd, page, theta):
     torch.testing.assert_close(got[:, : nh + nkv], ref_qk, **_tol(dtype))
     assert torch.equal(got[:, nh + nkv:], x[:, nh + nkv:])
     kref = torch.zeros(pages, nkv, page, hd, dtype=torch.float64)
-    vref = torch.zeros_like(kref)
+    vref = torch.zeros(pages, nkv, hd, page, dtype=torch.float64)
     for t in range(T):
         p = int(positions[t]); pg = int(bt[token_req[t], p // page])
         kref[pg, :, p % page] = got[t, nh: nh + nkv]       # the rotated k as stored in place
-        vref[pg, :, p % page] = x[t, nh + nkv:]
+        vref[pg, :, :, p % page] = x[t, nh + nkv:]
     assert torch.equal(d_kp.cpu().double(), kref)
     assert torch.equal(d_vp.cpu().double(), vref)
     assert float(d_kp[0].abs().sum()) == 0.0                # page 0 is never written
@@ -190,12 +190,15 @@ def _attention_ref(q, k, v, window):
     return torch.einsum("hnt,thd->nhd", torch.softmax(s, -1), vv)
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dtype,general", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
 @pytest.mark.parametrize("nh,nkv,hd,page,window,splits", [
     (4, 2, 16, 16, 0, 1), (3, 1, 32, 8, 0, 1), (28, 4, 128, 16, 0, 3), (6, 6, 48, 4, 0, 1),
     (20, 1, 64, 16, 0, 2), (4, 2, 16, 16, 13, 1), (8, 2, 80, 32, 29, 4), (2, 1, 256, 16, 0, 1),
+    (5, 5, 32, 2, 0, 2), (14, 2, 128, 64, 40, 5),
 ])
-def test_paged_attention(ops, dtype, nh, nkv, hd, page, window, splits):
+def test_paged_attention(ops, dtype, general, nh, nkv, hd, page, window, splits):
+    """float32 and bfloat16 through the general kernel, bfloat16 through the matrix-core kernel
+    (pages of 2 tokens fall back to the general one by themselves)."""
     g = torch.Generator().manual_seed(4)
     lens, ctxs = [37, 1, 9, 1], [0, 150, 70, 0]      # a whole prompt, a decode, a portion, a first token
     R, T = len(lens), sum(lens)
@@ -205,7 +208,7 @@ def test_paged_attention(ops, dtype, nh, nkv, hd, page, window, splits):
     bt = (torch.randperm(pages - 1, generator=g)[: R * max_blocks] + 1).view(R, max_blocks).int()
     q = torch.randn(T, nh * hd, generator=g).to(dtype)
     kp = torch.randn(pages, nkv, page, hd, generator=g).to(dtype)      # stale pages hold noise, not zeros
-    vp = torch.randn(pages, nkv, page, hd, generator=g).to(dtype)
+    vp = torch.randn(pages, nkv, hd, page, generator=g).to(dtype)      # transposed inside a page
     ks, vs = [], []
     for r in range(R):
         k = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
@@ -214,7 +217,7 @@ def test_paged_attention(ops, dtype, nh, nkv, hd, page, window, splits):
             k[3] *= 4.0        # a far key stands out: dropping it changes the result visibly
         for p in range(totals[r]):
             kp[bt[r, p // page], :, p % page] = k[p]
-            vp[bt[r, p // page], :, p % page] = v[p]
+            vp[bt[r, p // page], :, :, p % page] = v[p]
         ks.append(k); vs.append(v)
     indptr = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
     tq = ops.attention_tile_tokens(nh, nkv)
@@ -229,12 +232,17 @@ def test_paged_attention(ops, dtype, nh, nkv, hd, page, window, splits):
     ops.paged_attention(wide[:, : nh * hd], out, kp.cuda(), vp.cuda(), bt.cuda(), indptr.cuda(),
                         torch.tensor(ctxs, dtype=torch.int32).cuda(), torch.tensor(tile_req, dtype=torch.int32).cuda(),
                         torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq, nh, nkv, hd, page, window,
-                        1.0 / math.sqrt(hd), splits)
+                        1.0 / math.sqrt(hd), splits, general=general)
     got = out.cpu().double().view(T, nh, hd)
     for r in range(R):
         a, b = int(indptr[r]), int(indptr[r + 1])
         ref = _attention_ref(q[a:b].double().view(-1, nh, hd), ks[r].double(), vs[r].double(), window)
-        torch.testing.assert_close(got[a:b], ref, **_tol(dtype))
+        tol = _tol(dtype)
+        if dtype == torch.bfloat16 and not general:
+            # the matrix-core kernel rounds the probabilities to bfloat16 before the product with V
+            # (half an ulp, 2^-9 of each weight), on top of the rounding of the result
+            tol = dict(rtol=tol["rtol"], atol=tol["atol"] + 2 ** -9 * float(vs[r].abs().max()))
+        torch.testing.assert_close(got[a:b], ref, **tol)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -10,24 +10,27 @@
 // keys, with key tiles aligned to absolute positions.  With splits > 1 the range of
 // key tiles is divided over blockIdx.z and a second kernel merges the parts.
 //
+// Keys lie in their pages as [kv_head][position][d]; values lie transposed,
+// [kv_head][d][position], which is the layout the matrix-core kernel below reads directly.
+//
 // Compiled per head size: -DTL_HEAD_DIM=<multiple of 16>.
 #include "common.h"
 
 #ifndef TL_HEAD_DIM
 #error "compile with -DTL_HEAD_DIM=<head size>"
 #endif
-static_assert(TL_HEAD_DIM % 16 == 0 && TL_HEAD_DIM >= 16 && TL_HEAD_DIM <= 512, "head size: multiple of 16 up to 512");
+static_assert(TL_HEAD_DIM % 16 == 0 && TL_HEAD_DIM >= 16 && TL_HEAD_DIM <= 256, "head size: multiple of 16 up to 256");
 
 #define AT_ROWS 16
 #define AT_HD TL_HEAD_DIM
-#define AT_KT (AT_HD <= 128 ? 32 : (AT_HD <= 256 ? 16 : 8))   // keys per tile
+#define AT_KT (AT_HD <= 128 ? 32 : 16)                        // keys per tile
 #define AT_DPT (AT_HD / 16)                                   // output dims per thread
 
 struct AttnArgs {
     const void* q;            // [tokens, q_stride], head h at column h * HD
     void* out;                // [tokens, heads * HD]
     const void* k_plane;      // [pages, kv_heads, page, HD]
-    const void* v_plane;
+    const void* v_plane;      // [pages, kv_heads, HD, page]: values lie transposed inside a page
     const int* block_table;   // [requests, bt_stride]
     const int* req_indptr;    // [requests + 1] first new token of each request
     const int* ctx_lens;      // [requests] tokens cached before this step
@@ -108,9 +111,9 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
             float kv = 0.f, vv = 0.f;
             if (pos < key_hi) {
                 const int pg = bt[pos / a.page];
-                const size_t off = (((size_t)pg * a.kv_heads + kvh) * a.page + (pos % a.page)) * AT_HD + d;
-                kv = to_float(kp[off]);
-                vv = to_float(vp[off]);
+                const size_t head = ((size_t)pg * a.kv_heads + kvh) * a.page * AT_HD;
+                kv = to_float(kp[head + (size_t)(pos % a.page) * AT_HD + d]);
+                vv = to_float(vp[head + (size_t)d * a.page + (pos % a.page)]);
             }
             ks[j][d] = kv;
             vs[j][d] = vv;
@@ -183,6 +186,221 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     }
 }
 
+
+// =====================================================================================
+// The same attention on the matrix cores, for bfloat16 (pages of a multiple of 4 tokens).
+//
+// A wave owns the tile's 16 rows and walks the keys in chunks of 32.  Both products run
+// transposed so that no operand ever changes layout between them:
+//   S^T[key, row] = K[key, :] . Q[row, :]      A = 16 keys of K (rows of a page, d contiguous),
+//                                              B = Q;  a lane ends up with the scores of its
+//                                              row (lane % 16) for the keys 4g .. 4g+3 of each
+//                                              16-key half, g = lane / 16;
+//   O^T[d, row]   = V^T[d, key] . P^T[key, row] A = V^T, read straight from the transposed value
+//                                              pages as two 8-byte pieces (4 keys of each half),
+//                                              B = the lane's own eight probabilities.
+// The k-slots of the second product are dealt to keys as {4g..4g+3 of the first half,
+// 4g..4g+3 of the second}, for A and B alike, which is why no shuffle or shared memory is
+// needed.  The online softmax works in base 2 on scores pre-multiplied by scale * log2(e);
+// running maximum and sum are float, probabilities are rounded to bfloat16 for the product
+// with V.  The four waves of a work-group take the chunks of the tile's key range (or of its
+// split) in turn and merge their states pairwise through shared memory at the end.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+union FragK {
+    uint4 u;
+    uint2 h[2];
+    bf16x8_t v;
+    uint16_t e[8];
+};
+
+#define ATM_DC ((AT_HD + 31) / 32)
+#define ATM_DT (AT_HD / 16)
+#define ATM_SLOT (ATM_DT * 256 + 128)      // floats one wave parks in shared memory
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
+    __shared__ float park[2 * ATM_SLOT];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int li = lane & 15, g = lane >> 4;
+
+    const int tile = blockIdx.x;
+    const int group = a.heads / a.kv_heads;
+    const int chunks_h = (group + a.gcap - 1) / a.gcap;
+    const int kvh = blockIdx.y / chunks_h;
+    const int g0 = (blockIdx.y % chunks_h) * a.gcap;
+    const int gcount = min(a.gcap, group - g0);
+    const int split = blockIdx.z;
+
+    const int req = a.tile_req[tile];
+    const int tok0 = a.tile_tok0[tile];
+    const int first = a.req_indptr[req];
+    const int n_new = a.req_indptr[req + 1] - first;
+    const int ctx = a.ctx_lens[req];
+    const int ntok = min(a.tq, n_new - tok0);
+
+    const int r_tok = li / a.gcap, r_g = li % a.gcap;
+    const bool row_ok = r_tok < ntok && r_g < gcount;
+    const int r_pos = ctx + tok0 + r_tok;
+    const int r_lo = a.window > 0 ? r_pos - a.window + 1 : 0;
+    const int r_head = kvh * group + g0 + r_g;
+    const int r_token = first + tok0 + r_tok;
+
+    // my row's query, as B operand of the first product: d = 32 c + 8 g .. + 8
+    FragK qf[ATM_DC];
+    {
+        const bf16_t* q = (const bf16_t*)a.q + (size_t)r_token * a.q_stride + (size_t)r_head * AT_HD;
+#pragma unroll
+        for (int c = 0; c < ATM_DC; ++c) {
+            const int d = 32 * c + 8 * g;
+            qf[c].u = (row_ok && d + 8 <= AT_HD) ? *(const uint4*)(q + d) : make_uint4(0, 0, 0, 0);
+        }
+    }
+
+    const int key_hi = ctx + tok0 + ntok;
+    const int key_lo = a.window > 0 ? max(0, ctx + tok0 - a.window + 1) : 0;
+    const int ch_first = key_lo / 32;
+    const int ch_last = (key_hi + 31) / 32;
+    const int per_split = (ch_last - ch_first + a.splits - 1) / a.splits;
+    const int ch_begin = ch_first + split * per_split;
+    const int ch_end = min(ch_last, ch_begin + per_split);
+
+    const bf16_t* kp = (const bf16_t*)a.k_plane;
+    const bf16_t* vp = (const bf16_t*)a.v_plane;
+    const int* bt = a.block_table + (size_t)req * a.bt_stride;
+    const int page = a.page;
+    const float scale2 = a.scale * 1.44269504088896341f;
+
+    float m = -INFINITY, l = 0.f;
+    f32x4_t acc[ATM_DT];
+#pragma unroll
+    for (int t = 0; t < ATM_DT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int ch = ch_begin + wave; ch < ch_end; ch += 4) {
+        const int kbase = ch * 32;
+        // ---- scores: two halves of 16 keys
+        f32x4_t sc[2];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const int key = min(kbase + 16 * hf + li, key_hi - 1);
+            const int pg = bt[key / page];
+            const bf16_t* krow = kp + (((size_t)pg * a.kv_heads + kvh) * page + (key % page)) * AT_HD;
+            f32x4_t sacc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < ATM_DC; ++c) {
+                const int d = 32 * c + 8 * g;
+                FragK kf;
+                kf.u = (d + 8 <= AT_HD) ? *(const uint4*)(krow + d) : make_uint4(0, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sacc, 0, 0, 0);
+            }
+            sc[hf] = sacc;
+        }
+        // ---- mask, running maximum, probabilities
+        float s[8];
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int key = kbase + 16 * hf + 4 * g + v;
+                const bool seen = row_ok && key <= r_pos && key >= r_lo;
+                const float x = seen ? sc[hf][v] * scale2 : -INFINITY;
+                s[4 * hf + v] = x;
+                mloc = fmaxf(mloc, x);
+            }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, TL_WAVE));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TL_WAVE));
+        const float m_new = fmaxf(m, mloc);
+        const float alpha = (m == -INFINITY) ? 0.f : fast_exp2(m - m_new);
+        FragK pf;
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float p = (s[i] == -INFINITY) ? 0.f : fast_exp2(s[i] - m_new);
+            psum += p;
+            pf.e[i] = from_float<bf16_t>(p).bits;
+        }
+        l = l * alpha + psum;
+        m = m_new;
+        // ---- values: O^T += V^T . P^T
+        uint2 vfa[ATM_DT], vfb[ATM_DT];
+        {
+            const int ka = kbase + 4 * g, kb = kbase + 16 + 4 * g;
+            const bool oka = ka < key_hi, okb = kb < key_hi;
+            const int pga = oka ? bt[ka / page] : 0, pgb = okb ? bt[kb / page] : 0;
+            const bf16_t* va = vp + ((size_t)pga * a.kv_heads + kvh) * AT_HD * page + (ka % page);
+            const bf16_t* vb = vp + ((size_t)pgb * a.kv_heads + kvh) * AT_HD * page + (kb % page);
+#pragma unroll
+            for (int t = 0; t < ATM_DT; ++t) {
+                const size_t drow = (size_t)(16 * t + li) * page;
+                vfa[t] = oka ? *(const uint2*)(va + drow) : make_uint2(0, 0);
+                vfb[t] = okb ? *(const uint2*)(vb + drow) : make_uint2(0, 0);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < ATM_DT; ++t) {
+            FragK vf;
+            vf.h[0] = vfa[t];
+            vf.h[1] = vfb[t];
+            acc[t] *= alpha;
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[t], 0, 0, 0);
+        }
+    }
+
+    // ---- merge the four waves: 2,3 -> 0,1, then 1 -> 0
+#pragma unroll
+    for (int round = 0; round < 2; ++round) {
+        const int senders_from = round == 0 ? 2 : 1;
+        const int senders_to = round == 0 ? 4 : 2;
+        __syncthreads();
+        if (wave >= senders_from && wave < senders_to) {
+            float* dst = park + (size_t)(wave - senders_from) * ATM_SLOT;
+#pragma unroll
+            for (int t = 0; t < ATM_DT; ++t) *(f32x4_t*)(dst + (t * 64 + lane) * 4) = acc[t];
+            dst[ATM_DT * 256 + lane] = m;
+            dst[ATM_DT * 256 + 64 + lane] = l;
+        }
+        __syncthreads();
+        if (wave < senders_from && wave + senders_from < senders_to) {
+            const float* src = park + (size_t)wave * ATM_SLOT;
+            const float mo = src[ATM_DT * 256 + lane], lo = src[ATM_DT * 256 + 64 + lane];
+            const float mm = fmaxf(m, mo);
+            const float sa = (m == -INFINITY) ? 0.f : fast_exp2(m - mm);
+            const float sb = (mo == -INFINITY) ? 0.f : fast_exp2(mo - mm);
+#pragma unroll
+            for (int t = 0; t < ATM_DT; ++t) acc[t] = acc[t] * sa + *(const f32x4_t*)(src + (t * 64 + lane) * 4) * sb;
+            l = l * sa + lo * sb;
+            m = mm;
+        }
+    }
+    if (wave != 0) return;
+    l += __shfl_xor(l, 16, TL_WAVE);
+    l += __shfl_xor(l, 32, TL_WAVE);
+    if (!row_ok) return;
+    if (a.splits == 1) {
+        bf16_t* o = (bf16_t*)a.out + (size_t)r_token * a.heads * AT_HD + (size_t)r_head * AT_HD;
+        const float inv = 1.f / l;
+#pragma unroll
+        for (int t = 0; t < ATM_DT; ++t) {
+            union { uint2 u; uint16_t e[4]; } pk;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(acc[t][v] * inv).bits;
+            *(uint2*)(o + 16 * t + 4 * g) = pk.u;
+        }
+    } else {
+        const size_t pr = ((size_t)r_token * a.heads + r_head) * a.splits + split;
+        float* o = a.part_o + pr * AT_HD;
+#pragma unroll
+        for (int t = 0; t < ATM_DT; ++t) *(f32x4_t*)(o + 16 * t + 4 * g) = acc[t];
+        if (g == 0) {
+            a.part_ml[pr * 2] = m * 0.69314718055994531f;      // back to natural logarithms for the merge
+            a.part_ml[pr * 2 + 1] = l;
+        }
+    }
+}
+
 // out[row] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s over the parts of a row.
 template <typename T>
 __global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
@@ -210,7 +428,7 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
                                   const void* block_table, int bt_stride, const void* req_indptr, const void* ctx_lens,
                                   const void* tile_req, const void* tile_tok0, int tiles, int tokens, int tq,
                                   int heads, int kv_heads, int page, int window, float scale, int splits,
-                                  void* part_o, void* part_ml, int dtype, hipStream_t stream) {
+                                  void* part_o, void* part_ml, int dtype, int general, hipStream_t stream) {
     TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
     TL_REQUIRE(page > 0 && bt_stride > 0 && tq > 0 && splits > 0 && window >= 0, "attention: bad page/table/tile sizes");
     TL_REQUIRE(splits == 1 || (part_o && part_ml), "attention: splits > 1 needs scratch");
@@ -228,7 +446,10 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
     a.window = window; a.tq = tq; a.gcap = gcap; a.splits = splits; a.scale = scale;
     const int chunks = (group + gcap - 1) / gcap;
     dim3 grid(tiles, kv_heads * chunks, splits), block(256);
+    const bool aligned = ((uintptr_t)q % 16) == 0 && q_stride % 8 == 0 && ((uintptr_t)out % 8) == 0 &&
+                         ((uintptr_t)k_plane % 16) == 0 && ((uintptr_t)v_plane % 8) == 0;
     if (dtype == TL_DT_F32) paged_attention_kernel<float><<<grid, block, 0, stream>>>(a);
+    else if (dtype == TL_DT_BF16 && page % 4 == 0 && aligned && !general) paged_attention_mfma_kernel<<<grid, block, 0, stream>>>(a);
     else if (dtype == TL_DT_BF16) paged_attention_kernel<bf16_t><<<grid, block, 0, stream>>>(a);
     else TL_REQUIRE(false, "attention: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("paged_attention");

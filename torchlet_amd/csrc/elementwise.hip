@@ -82,8 +82,9 @@ extern "C" int tl_add_rmsnorm(void* residual, const void* pending, const void* w
 //   * rotate (inv_freq != null): the first `rot_heads` heads (q, then k) are rotated in
 //     place with the split-half pairing (j, j + head_dim/2) by angle = float(pos) * inv_freq[j].
 //   * write (k_plane != null): rotated k and raw v of the token go to the page
-//     block_table[token_req[t]][pos / page] at offset pos % page; planes are
-//     [pages, kv_heads, page, head_dim].
+//     block_table[token_req[t]][pos / page] at offset pos % page.  The key plane is
+//     [pages, kv_heads, page, head_dim]; the value plane holds each page transposed,
+//     [pages, kv_heads, head_dim, page], the layout the attention kernels read.
 template <typename T>
 __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, int kv_heads,
                                         int head_dim, int rot_heads, const int* __restrict__ positions,
@@ -98,9 +99,9 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int
     T* vdst = nullptr;
     if (k_plane) {
         const int page = block_table[(size_t)token_req[t] * bt_stride + pos / page_size];
-        const size_t base = ((size_t)page * kv_heads) * page_size * head_dim + (size_t)(pos % page_size) * head_dim;
-        kdst = k_plane + base;
-        vdst = v_plane + base;
+        const size_t base = ((size_t)page * kv_heads) * page_size * head_dim;
+        kdst = k_plane + base + (size_t)(pos % page_size) * head_dim;
+        vdst = v_plane + base + (pos % page_size);
     }
     const size_t head_step = (size_t)page_size * head_dim;  // between kv heads inside a page
     const int pairs = (q_heads + kv_heads) * half;
@@ -128,7 +129,7 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int
         const T* v = row + (size_t)(q_heads + kv_heads) * head_dim;
         for (int idx = threadIdx.x; idx < kv_heads * head_dim; idx += blockDim.x) {
             const int head = idx / head_dim, d = idx % head_dim;
-            vdst[(size_t)head * head_step + d] = v[idx];
+            vdst[(size_t)head * head_step + (size_t)d * page_size] = v[idx];
         }
     }
 }

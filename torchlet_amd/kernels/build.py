@@ -64,7 +64,7 @@ def target(name: str) -> tuple[str, list[str]]:
 def _writable(folder: Path) -> bool:
     try:
         folder.mkdir(parents=True, exist_ok=True)
-        probe = folder / f".probe-{os.getpid()}"
+        probe = folder / f".probe-{os.getpid()}-{threading.get_ident()}"
         probe.write_text("")
         probe.unlink()
         return True
@@ -157,6 +157,7 @@ def build(name: str, force: bool = False, quiet: bool = False) -> Path:
 
 def build_many(names, force: bool = False, jobs: int | None = None, quiet: bool = False) -> list[Path]:
     names = list(dict.fromkeys(names))
+    lib_dir()                                   # settle the folder before the threads start
     jobs = jobs or min(8, os.cpu_count() or 1, max(1, len(names)))
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         return list(pool.map(lambda n: build(n, force=force, quiet=quiet), names))

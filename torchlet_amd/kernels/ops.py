@@ -173,7 +173,9 @@ def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: i
                      page_size: int = 0) -> None:
     """Rotate the first ``rot_heads`` heads of each row of ``qkv [T, >= (q+2kv)*hd]`` in
     place by the token's position (``inv_freq`` float32 ``[hd/2]``; ``None``: no rotation)
-    and, when planes are given, store rotated k and raw v of every token in its page."""
+    and, when planes are given, store rotated k and raw v of every token in its page:
+    ``k_plane [pages, kv_heads, page, hd]``, ``v_plane [pages, kv_heads, hd, page]`` (values
+    lie transposed inside a page)."""
     T = qkv.shape[0]
     if qkv.stride(1) != 1:
         raise KernelError("rope_cache_write: qkv needs unit stride on the last axis")
@@ -185,14 +187,20 @@ def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: i
         _i32(token_req, "token_req", T)
         _i32(block_table, "block_table")
         bt_stride = block_table.stride(0)
-        for p in (k_plane, v_plane):
-            if p.dtype != qkv.dtype or p.dim() != 4 or p.shape[1:] != (kv_heads, page_size, head_dim) or not p.is_contiguous():
-                raise KernelError(f"rope_cache_write: plane {tuple(p.shape)} {p.dtype} is not [pages, {kv_heads}, {page_size}, {head_dim}] {qkv.dtype}")
+        _check_planes("rope_cache_write", k_plane, v_plane, qkv.dtype, kv_heads, page_size, head_dim)
     lib = _lib("elementwise")
     _check(lib, lib.tl_rope_cache_write(_ptr(qkv), c_int(qkv.stride(0)), c_int(T), c_int(q_heads), c_int(kv_heads),
                                         c_int(head_dim), c_int(rot_heads), _ptr(positions), _ptr(inv_freq), _ptr(token_req),
                                         _ptr(block_table), c_int(bt_stride), _ptr(k_plane), _ptr(v_plane), c_int(page_size),
                                         c_int(_dt(qkv, "rope_cache_write")), _stream()))
+
+
+def _check_planes(what, k_plane, v_plane, dtype, kv_heads, page_size, head_dim) -> None:
+    for p, shape in ((k_plane, (kv_heads, page_size, head_dim)), (v_plane, (kv_heads, head_dim, page_size))):
+        if p.dtype != dtype or p.dim() != 4 or tuple(p.shape[1:]) != shape or not p.is_contiguous():
+            raise KernelError(f"{what}: plane {tuple(p.shape)} {p.dtype} is not [pages, {', '.join(map(str, shape))}] {dtype}")
+    if k_plane.shape[0] != v_plane.shape[0]:
+        raise KernelError(f"{what}: key and value planes differ in their number of pages")
 
 
 ATTENTION_ROWS = 16   # rows (tokens x heads of one group) a work-group owns
@@ -208,18 +216,18 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
                     block_table: torch.Tensor, req_indptr: torch.Tensor, ctx_lens: torch.Tensor,
                     tile_req: torch.Tensor, tile_tok0: torch.Tensor, num_tiles: int, tile_tokens: int,
                     num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
-                    scale: float, splits: int = 1) -> None:
+                    scale: float, splits: int = 1, general: bool = False) -> None:
     """Causal attention of the step's tokens over their requests' cached keys.
 
-    ``q [T, >= heads*hd]`` (row-strided view), ``out [T, heads*hd]``, planes
-    ``[pages, kv_heads, page, hd]``, ``block_table [R, max_blocks]`` int32; the new token
-    ``i`` of request ``r`` sits at position ``ctx_lens[r] + i``.  ``window`` 0: all keys."""
+    ``q [T, >= heads*hd]`` (row-strided view), ``out [T, heads*hd]``, ``k_plane [pages,
+    kv_heads, page, hd]``, ``v_plane [pages, kv_heads, hd, page]``, ``block_table [R,
+    max_blocks]`` int32; the new token ``i`` of request ``r`` sits at position
+    ``ctx_lens[r] + i``.  ``window`` 0: all keys.  bfloat16 with pages of a multiple of 4
+    tokens runs on the matrix cores; ``general=True`` forces the general kernel."""
     T = q.shape[0]
     if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
         raise KernelError("paged_attention: q/out shapes or dtypes do not fit")
-    for p in (k_plane, v_plane):
-        if p.dtype != q.dtype or p.dim() != 4 or p.shape[1:] != (num_kv_heads, page_size, head_dim) or not p.is_contiguous():
-            raise KernelError(f"paged_attention: plane {tuple(p.shape)} {p.dtype} is not [pages, {num_kv_heads}, {page_size}, {head_dim}] {q.dtype}")
+    _check_planes("paged_attention", k_plane, v_plane, q.dtype, num_kv_heads, page_size, head_dim)
     for name, t in (("block_table", block_table), ("req_indptr", req_indptr), ("ctx_lens", ctx_lens),
                     ("tile_req", tile_req), ("tile_tok0", tile_tok0)):
         _i32(t, name)
@@ -235,7 +243,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
                                        _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles), c_int(T), c_int(tile_tokens),
                                        c_int(num_heads), c_int(num_kv_heads), c_int(page_size), c_int(window),
                                        c_float(scale), c_int(splits), _ptr(part_o), _ptr(part_ml),
-                                       c_int(_dt(q, "paged_attention")), _stream()))
+                                       c_int(_dt(q, "paged_attention")), c_int(1 if general else 0), _stream()))
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:

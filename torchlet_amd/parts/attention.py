@@ -98,7 +98,10 @@ class GQAttention(Mixer):
         qkv = torch.empty((T, width), dtype=self.dtype, device=h.device)
         ops.linear(h, w, b, qkv)
 
+        # the cache hands out two planes of [pages, kv_heads, page, head_dim]; this mixer keeps the
+        # values of a page transposed, [kv_heads, head_dim, page], as its kernels read them
         k_plane, v_plane = cache.planes
+        v_plane = v_plane.view(v_plane.shape[0], self.kv_heads, self.head_dim, cache.page_size)
         table = ctx.block_tables[cache.group]
         kv_heads = self.kv_heads if writes else 0
         inv_freq = self.position.fused_inv_freq() if hasattr(self.position, "fused_inv_freq") else None

@@ -106,6 +106,10 @@ extern "C" int tl_gemm_general(const void* x, const void* w, const void* bias, i
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
+#define SK_KOFF(lg) (16 * (lg))     // a lane reads 32 contiguous bytes per step (other splits measured the same)
+#define SK_SECOND 8
+#define SK_LOAD(p) (*(const uint4*)(p))
+
 union Frag16 {          // 16 bytes: eight bfloat16 as the MFMA wants them, or one 128-bit load
     uint4 u;
     bf16x8_t v;
@@ -137,21 +141,21 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
     Frag16 a0[R], a1[R], b0[MT], b1[MT];
     int s = wave;
     if (s < full) {
-        const int k = 64 * s + 16 * lg;
+        const int k = 64 * s + SK_KOFF(lg);
 #pragma unroll
-        for (int r = 0; r < R; ++r) { a0[r].u = *(const uint4*)(wrow[r] + k); a1[r].u = *(const uint4*)(wrow[r] + k + 8); }
+        for (int r = 0; r < R; ++r) { a0[r].u = SK_LOAD(wrow[r] + k); a1[r].u = SK_LOAD(wrow[r] + k + SK_SECOND); }
 #pragma unroll
-        for (int t = 0; t < MT; ++t) { b0[t].u = *(const uint4*)(xrow[t] + k); b1[t].u = *(const uint4*)(xrow[t] + k + 8); }
+        for (int t = 0; t < MT; ++t) { b0[t].u = *(const uint4*)(xrow[t] + k); b1[t].u = *(const uint4*)(xrow[t] + k + SK_SECOND); }
     }
     for (; s < full; s += KS) {
         // fetch the next step (the last one fetches itself again: no branch in the loop)
         Frag16 na0[R], na1[R], nb0[MT], nb1[MT];
         const int sn = (s + KS < full) ? s + KS : s;
-        const int kn = 64 * sn + 16 * lg;
+        const int kn = 64 * sn + SK_KOFF(lg);
 #pragma unroll
-        for (int r = 0; r < R; ++r) { na0[r].u = *(const uint4*)(wrow[r] + kn); na1[r].u = *(const uint4*)(wrow[r] + kn + 8); }
+        for (int r = 0; r < R; ++r) { na0[r].u = SK_LOAD(wrow[r] + kn); na1[r].u = SK_LOAD(wrow[r] + kn + SK_SECOND); }
 #pragma unroll
-        for (int t = 0; t < MT; ++t) { nb0[t].u = *(const uint4*)(xrow[t] + kn); nb1[t].u = *(const uint4*)(xrow[t] + kn + 8); }
+        for (int t = 0; t < MT; ++t) { nb0[t].u = *(const uint4*)(xrow[t] + kn); nb1[t].u = *(const uint4*)(xrow[t] + kn + SK_SECOND); }
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -166,18 +170,18 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
     }
     // the tail step (K % 64 != 0) belongs to the wave whose turn it is; pieces beyond K count as zero
     if ((K & 63) && (full % KS) == wave) {
-        const int k = 64 * full + 16 * lg;
-        const bool v0 = k + 8 <= K, v1 = k + 16 <= K;
+        const int k = 64 * full + SK_KOFF(lg);
+        const bool v0 = k + 8 <= K, v1 = k + SK_SECOND + 8 <= K;
         const uint4 zero = make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             a0[r].u = v0 ? *(const uint4*)(wrow[r] + k) : zero;
-            a1[r].u = v1 ? *(const uint4*)(wrow[r] + k + 8) : zero;
+            a1[r].u = v1 ? *(const uint4*)(wrow[r] + k + SK_SECOND) : zero;
         }
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
             b0[t].u = v0 ? *(const uint4*)(xrow[t] + k) : zero;
-            b1[t].u = v1 ? *(const uint4*)(xrow[t] + k + 8) : zero;
+            b1[t].u = v1 ? *(const uint4*)(xrow[t] + k + SK_SECOND) : zero;
         }
 #pragma unroll
         for (int r = 0; r < R; ++r)
@@ -242,13 +246,20 @@ static void launch_skinny(const void* x, const void* w, const void* bias, int bi
 template <int MT>
 static void pick_skinny(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                         int ldx, int ldo, int out_f32, hipStream_t stream) {
-    // Enough work-groups to fill 256 compute units a few times over, and enough K steps per
-    // wave to keep loads in flight: wide matrices take two strips per wave and four waves
-    // along K, narrow ones one strip and eight waves.
+    // Measured on MI355X at Qwen2.5-7B sizes (weights streamed from HBM, M = 8 and 64):
+    // with up to 32 rows one strip of 16 weight rows per work-group is best throughout, with
+    // 16 waves along K for wide matrices (gate_up, LM head: 4.7-5.0 TB/s) and 8 for narrow
+    // ones (qkv, o, down); with 64 rows the x operand weighs more and several strips per wave
+    // share each x load.
     const int strips = (N + 15) / 16;
-    if (strips >= 2048 && MT <= 2) launch_skinny<4, MT, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else if (strips >= 1024) launch_skinny<2, MT, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else launch_skinny<1, MT, 8>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    if (MT <= 2) {
+        if (strips >= 1024) launch_skinny<1, MT, 16>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        else launch_skinny<1, MT, 8>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    } else {
+        if (strips >= 2048) launch_skinny<4, MT, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        else if (strips >= 1024) launch_skinny<2, MT, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        else launch_skinny<1, MT, 8>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    }
 }
 
 // One named instance of the few-rows kernel (tests cover every instance; tuning times them).
@@ -269,17 +280,162 @@ extern "C" int tl_gemm_skinny_variant(const void* x, const void* w, const void* 
     TL_REQUIRE(false, "gemm_skinny: no instance R=%d MT=%d KS=%d", R, MT, KS);
 }
 
+// =====================================================================================
+// bfloat16 on the matrix cores, many rows (prompt portions): shared-memory tiles.
+//
+// A work-group of four waves owns a BM x BN tile of the output and walks K in slabs of 32.
+// A slab of x (BM rows) and of w (BN rows) is fetched from memory as 16-byte pieces into
+// registers while the previous slab is being multiplied, then parked in shared memory
+// (two buffers, one barrier per slab).  Rows lie 80 bytes apart in shared memory (64 of
+// data, 16 of padding) so that the 16-byte operand reads of v_mfma_f32_32x32x16_bf16 do not
+// collide on banks.  Waves are laid out WGM x WGN over the tile; each multiplies
+// (BM / WGM) x (BN / WGN) as blocks of 32 x 32 with float accumulators.
+// Needs K % 8 == 0 and 16-byte aligned rows.
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+#define TK 32                 // K elements per slab
+#define TROW 40               // bfloat16 elements between rows in shared memory (32 + 8 padding)
+
+template <int BM, int BN, int WGM, int WGN, typename TOut>
+__global__ __launch_bounds__(256) void gemm_mfma_tile_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                             const void* __restrict__ bias, int bias_f32,
+                                                             TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+    static_assert(WGM * WGN == 4, "four waves");
+    constexpr int WM = BM / WGM, WN = BN / WGN;          // wave tile
+    constexpr int FM = WM / 32, FN = WN / 32;            // 32x32 blocks per wave
+    constexpr int PIECES = (BM + BN) * (TK / 8);         // 16-byte pieces per slab
+    constexpr int PPT = PIECES / 256;                    // pieces per thread
+    static_assert(PIECES % 256 == 0, "slab must divide over the threads");
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2][(BM + BN) * TROW];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    // neighbouring work-groups share weight tiles: walk M fastest within a band of N
+    const int tiles_m = (M + BM - 1) / BM;
+    const int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
+
+    // which pieces this thread fetches: piece p -> (row, 8-element column) of the stacked [x rows; w rows] slab
+    const bf16_t* src[PPT];
+    int dst[PPT];
+    int kcol[PPT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+        const int p = tid + i * 256;
+        const int row = p / (TK / 8), c = p % (TK / 8);
+        kcol[i] = c * 8;
+        dst[i] = row * TROW + c * 8;
+        if (row < BM) src[i] = x + (size_t)min(m0 + row, M - 1) * ldx + c * 8;
+        else src[i] = w + (size_t)min(n0 + row - BM, N - 1) * K + c * 8;
+    }
+
+    f32x16_t acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    const int slabs = (K + TK - 1) / TK;
+    uint4 stage[PPT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) stage[i] = (kcol[i] + 8 <= K) ? *(const uint4*)(src[i]) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) *(uint4*)(&lds[0][dst[i]]) = stage[i];
+    __syncthreads();
+
+    const int fr = lane & 31, fk = (lane >> 5) * 8;      // operand fragment: row within block, k offset
+    for (int sl = 0; sl < slabs; ++sl) {
+        const int cur = sl & 1;
+        if (sl + 1 < slabs) {
+            const int k0 = (sl + 1) * TK;
+#pragma unroll
+            for (int i = 0; i < PPT; ++i)
+                stage[i] = (k0 + kcol[i] + 8 <= K) ? *(const uint4*)(src[i] + k0) : make_uint4(0, 0, 0, 0);
+        }
+        const bf16_t* xs = &lds[cur][0];
+        const bf16_t* ws = &lds[cur][BM * TROW];
+#pragma unroll
+        for (int kk = 0; kk < TK; kk += 16) {
+            Frag16 af[FM], bfr[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) af[i].u = *(const uint4*)(xs + (wm * WM + i * 32 + fr) * TROW + kk + fk);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) bfr[j].u = *(const uint4*)(ws + (wn * WN + j * 32 + fr) * TROW + kk + fk);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i].v, bfr[j].v, acc[i][j], 0, 0, 0);
+        }
+        if (sl + 1 < slabs) {
+#pragma unroll
+            for (int i = 0; i < PPT; ++i) *(uint4*)(&lds[cur ^ 1][dst[i]]) = stage[i];
+        }
+        __syncthreads();
+    }
+
+    // block result: lane holds column (lane % 32), rows 8 * (v / 4) + 4 * (lane / 32) + v % 4
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+        const int n = n0 + wn * WN + j * 32 + (lane & 31);
+        if (n >= N) continue;
+        const float b = bias ? load_vec(bias, bias_f32, n) : 0.f;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                if (m < M) out[(size_t)m * ldo + n] = from_float<TOut>(acc[i][j][v] + b);
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN>
+static void launch_mfma_tile(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                             int ldx, int ldo, int out_f32, hipStream_t stream) {
+    dim3 grid(((M + BM - 1) / BM) * ((N + BN - 1) / BN)), block(256);
+    if (out_f32)
+        gemm_mfma_tile_kernel<BM, BN, WGM, WGN, float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo);
+    else
+        gemm_mfma_tile_kernel<BM, BN, WGM, WGN, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo);
+}
+
+// One named tile shape of the many-rows kernel (tests cover each; tuning times them).
+extern "C" int tl_gemm_tile_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
+                                    int M, int N, int K, int ldx, int ldo, int out_f32, int BM, int BN, hipStream_t stream) {
+    TL_REQUIRE(M > 0 && K % 8 == 0 && ldx % 8 == 0, "gemm_tile: needs M > 0 and K, ldx multiples of 8");
+    if (BM == 128 && BN == 128) launch_mfma_tile<128, 128, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else if (BM == 256 && BN == 128) launch_mfma_tile<256, 128, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else if (BM == 128 && BN == 256) launch_mfma_tile<128, 256, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else if (BM == 64 && BN == 128) launch_mfma_tile<64, 128, 1, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else if (BM == 64 && BN == 256) launch_mfma_tile<64, 256, 1, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else TL_REQUIRE(false, "gemm_tile: no instance BM=%d BN=%d", BM, BN);
+    TL_CHECK_LAUNCH("gemm_mfma_tile");
+    return TL_OK;
+}
+
 static bool skinny_fits(const void* x, const void* w, int M, int K, int ldx) {
     return M <= 64 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
 }
 
 // out = x w^T (+ bias) in the engine's dtype: picks the kernel for the shape.
-//   bfloat16, M <= 64, aligned  -> gemm_skinny (matrix cores, weight streaming)
+//   bfloat16, aligned, M <= 64  -> gemm_skinny (matrix cores, weight streaming), except that
+//                                  33..64 rows against a wide matrix go to the tile kernel
+//   bfloat16, aligned, M > 64   -> gemm_mfma_tile (matrix cores, shared-memory tiles)
 //   everything else             -> gemm_tile (true 32-bit arithmetic)
 extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_f32, void* out,
                        int M, int N, int K, int ldx, int ldo, int dtype, int out_f32, hipStream_t stream) {
     TL_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldo >= N, "gemm: bad sizes M=%d N=%d K=%d ldx=%d ldo=%d", M, N, K, ldx, ldo);
     if (M == 0) return TL_OK;
+    const bool aligned = K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
+    if (dtype == TL_DT_BF16 && aligned && (M > 64 || (M > 32 && N >= 16384))) {
+        if (M > 64) launch_mfma_tile<128, 128, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        else launch_mfma_tile<64, 128, 1, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        TL_CHECK_LAUNCH("gemm_mfma_tile");
+        return TL_OK;
+    }
     if (dtype == TL_DT_BF16 && skinny_fits(x, w, M, K, ldx)) {
         if (M <= 16) pick_skinny<1>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
         else if (M <= 32) pick_skinny<2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);

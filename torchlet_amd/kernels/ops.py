@@ -166,6 +166,19 @@ def linear_few_rows_variant(x, weight, bias, out, strips_per_wave: int, waves_al
                                            c_int(waves_along_k), _stream()))
 
 
+def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int) -> None:
+    """One named tile shape of the many-rows matrix-core kernel (for tests and tuning)."""
+    M, K = x.shape
+    N = weight.shape[0]
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or out.shape != (M, N) or not weight.is_contiguous():
+        raise KernelError("linear_many_rows_variant: bfloat16 operands and fitting shapes only")
+    bf = _vec(bias, N, "linear bias")
+    lib = _lib("gemm")
+    _check(lib, lib.tl_gemm_tile_variant(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N),
+                                         c_int(K), c_int(x.stride(0)), c_int(out.stride(0)),
+                                         c_int(1 if out.dtype == torch.float32 else 0), c_int(tile_m), c_int(tile_n), _stream()))
+
+
 def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int, rot_heads: int,
                      positions: torch.Tensor, inv_freq: torch.Tensor | None,
                      token_req: torch.Tensor | None = None, block_table: torch.Tensor | None = None,

@@ -43,6 +43,6 @@ def cpu_ops(monkeypatch):
     from torchlet_amd.kernels import ops
 
     for name in ("attention_tile_tokens", "load", "embedding", "add_rmsnorm", "linear", "rope_cache_write",
-                 "paged_attention", "swiglu", "sample"):
+                 "paged_attention", "swiglu", "sample", "interleave_gate_up", "linear_swiglu"):
         monkeypatch.setattr(ops, name, getattr(emulated_ops, name))
     return ops

@@ -90,6 +90,24 @@ def paged_attention(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens,
     assert bool(covered.all()), "tiles do not cover every token"
 
 
+def interleave_gate_up(gate, up):
+    I, K = gate.shape
+    blocks = -(-I // 32)
+    g = torch.zeros((blocks * 32, K), dtype=gate.dtype)
+    u = torch.zeros_like(g)
+    g[:I] = gate
+    u[:I] = up
+    return torch.stack((g.view(blocks, 32, K), u.view(blocks, 32, K)), dim=1).reshape(blocks * 64, K).contiguous()
+
+
+def linear_swiglu(x, gate_up, out):
+    I, K = out.shape[1], x.shape[1]
+    w = gate_up.float().view(-1, 2, 32, K)
+    g = x.float() @ w[:, 0].reshape(-1, K)[:I].T
+    u = x.float() @ w[:, 1].reshape(-1, K)[:I].T
+    out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+
+
 def swiglu(gate_up, out):
     I = gate_up.shape[1] // 2
     g, u = gate_up[:, :I].float(), gate_up[:, I:].float()

@@ -35,7 +35,7 @@ def test_embedding(ops, dtype, V, H, T):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("wdtype", DTYPES)
-@pytest.mark.parametrize("T,H,eps", [(5, 96, 1e-5), (19, 1000, 1e-6), (3, 5120, 1e-6)])
+@pytest.mark.parametrize("T,H,eps", [(5, 96, 1e-5), (19, 1000, 1e-6), (3, 5120, 1e-6), (2, 1001, 1e-6), (8, 3584, 1e-6), (2, 10000, 1e-5), (1, 20000, 1e-6)])
 def test_add_rmsnorm(ops, dtype, wdtype, T, H, eps):
     if dtype == torch.float32 and wdtype == torch.bfloat16:
         pytest.skip("a 32-bit engine widens its vectors")
@@ -145,6 +145,24 @@ def test_linear_many_rows_on_matrix_cores(ops, out_dtype, tile, M, N, K):
     out2 = torch.empty_like(out)
     ops.linear_many_rows_variant(wide[:, 16:16 + K], w, None, out2, *tile)
     torch.testing.assert_close(out2.double(), ref - b.double(), **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 32, 33, 64, 65, 300])
+@pytest.mark.parametrize("I,K", [(128, 64), (200, 96), (112, 80), (18944, 256), (32768 + 40, 64)])
+def test_linear_swiglu_fused(ops, M, I, K):
+    """The gate/up product with the gate applied to the accumulators: every kernel behind it
+    (few rows, 64-row tile, 128 and 256-row tiles), with I not a multiple of 32."""
+    g = torch.Generator().manual_seed(M + I)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    gate = (torch.randn(I, K, generator=g) / math.sqrt(K) * 2).to(torch.bfloat16).cuda()
+    up = (torch.randn(I, K, generator=g) / math.sqrt(K) * 2).to(torch.bfloat16).cuda()
+    w = ops.interleave_gate_up(gate, up)
+    assert w.shape == (-(-I // 32) * 64, K)
+    out = torch.full((M, I + 8), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops.linear_swiglu(x, w, out[:, :I])
+    ref = torch.nn.functional.silu(x.double() @ gate.double().T) * (x.double() @ up.double().T)
+    torch.testing.assert_close(out[:, :I].double(), ref, **_tol(torch.bfloat16))
+    assert bool(out[:, I:].isnan().all())          # nothing is written beyond the I columns
 
 
 def _rope_ref(x, pos, theta):

@@ -61,16 +61,111 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __rest
     }
 }
 
+// The same with every element of the row held in registers between the two passes: a thread
+// owns IT groups of 4 contiguous elements, loaded with one 16-byte (float) or 8-byte
+// (bfloat16) access each, so the row is read from memory once and the weight load overlaps
+// the reduction.  Used when hidden % 4 == 0 and hidden <= 16 * blockDim.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+        const float4 t = *(const float4*)p; v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Vec4<bf16_t> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+        const uint2 t = *(const uint2*)p;
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+        uint2 t;
+        t.x = (uint32_t)from_float<bf16_t>(v[0]).bits | ((uint32_t)from_float<bf16_t>(v[1]).bits << 16);
+        t.y = (uint32_t)from_float<bf16_t>(v[2]).bits | ((uint32_t)from_float<bf16_t>(v[3]).bits << 16);
+        *(uint2*)p = t;
+    }
+};
+
+template <typename T, int IT>
+__global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const T* __restrict__ pending,
+                                       const void* __restrict__ weight, int weight_f32, float eps,
+                                       T* __restrict__ out, const int* __restrict__ rows, int hidden) {
+    __shared__ float red[16];
+    const int orow = blockIdx.x;
+    const int srow = rows ? rows[orow] : orow;
+    float* res = residual + (size_t)srow * hidden;
+    const T* pen = pending ? pending + (size_t)srow * hidden : nullptr;
+    const bool update = (pen != nullptr) && (rows == nullptr);
+    float r[IT][4], wv[IT][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int i = (it * blockDim.x + threadIdx.x) * 4;
+        if (i < hidden) {
+            Vec4<float>::load(res + i, r[it]);
+            if (pen) {
+                float p[4];
+                Vec4<T>::load(pen + i, p);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) r[it][v] += p[v];
+            }
+            if (weight_f32) Vec4<float>::load((const float*)weight + i, wv[it]);
+            else Vec4<bf16_t>::load((const bf16_t*)weight + i, wv[it]);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) ss += r[it][v] * r[it][v];
+        }
+    }
+    if (update) {
+#pragma unroll
+        for (int it = 0; it < IT; ++it) {
+            const int i = (it * blockDim.x + threadIdx.x) * 4;
+            if (i < hidden) Vec4<float>::store(res + i, r[it]);
+        }
+    }
+    ss = block_sum(ss, red);
+    const float inv = rsqrtf(ss / (float)hidden + eps);
+    T* dst = out + (size_t)orow * hidden;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int i = (it * blockDim.x + threadIdx.x) * 4;
+        if (i < hidden) {
+            float o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[v] = r[it][v] * inv * wv[it][v];
+            Vec4<T>::store(dst + i, o);
+        }
+    }
+}
+
+template <typename T>
+static void launch_add_rmsnorm(float* residual, const T* pending, const void* weight, int weight_f32, float eps, T* out,
+                               const int* rows, int out_rows, int hidden, hipStream_t stream) {
+    const bool aligned = hidden % 4 == 0 && ((uintptr_t)residual % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                         ((uintptr_t)pending % 16) == 0 && ((uintptr_t)weight % 16) == 0;
+    dim3 grid(out_rows);
+    if (aligned && hidden <= 1024)
+        add_rmsnorm_reg_kernel<T, 1><<<grid, 256, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+    else if (aligned && hidden <= 2048)
+        add_rmsnorm_reg_kernel<T, 2><<<grid, 256, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+    else if (aligned && hidden <= 4096)
+        add_rmsnorm_reg_kernel<T, 2><<<grid, 512, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+    else if (aligned && hidden <= 8192)
+        add_rmsnorm_reg_kernel<T, 4><<<grid, 512, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+    else if (aligned && hidden <= 16384)
+        add_rmsnorm_reg_kernel<T, 4><<<grid, 1024, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+    else
+        add_rmsnorm_kernel<T><<<grid, hidden >= 2048 ? 512 : 256, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+}
+
 extern "C" int tl_add_rmsnorm(void* residual, const void* pending, const void* weight, int weight_f32,
                               float eps, void* out, const void* rows, int out_rows, int hidden,
                               int act_dtype, hipStream_t stream) {
     TL_REQUIRE(out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d hidden=%d", out_rows, hidden);
     if (out_rows == 0) return TL_OK;
-    dim3 grid(out_rows), block(hidden >= 2048 ? 512 : 256);
     if (act_dtype == TL_DT_F32)
-        add_rmsnorm_kernel<float><<<grid, block, 0, stream>>>((float*)residual, (const float*)pending, weight, weight_f32, eps, (float*)out, (const int*)rows, hidden);
+        launch_add_rmsnorm<float>((float*)residual, (const float*)pending, weight, weight_f32, eps, (float*)out, (const int*)rows, out_rows, hidden, stream);
     else if (act_dtype == TL_DT_BF16)
-        add_rmsnorm_kernel<bf16_t><<<grid, block, 0, stream>>>((float*)residual, (const bf16_t*)pending, weight, weight_f32, eps, (bf16_t*)out, (const int*)rows, hidden);
+        launch_add_rmsnorm<bf16_t>((float*)residual, (const bf16_t*)pending, weight, weight_f32, eps, (bf16_t*)out, (const int*)rows, out_rows, hidden, stream);
     else TL_REQUIRE(false, "add_rmsnorm: unknown dtype %d", act_dtype);
     TL_CHECK_LAUNCH("add_rmsnorm");
     return TL_OK;
@@ -104,14 +199,23 @@ __global__ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int
         vdst = v_plane + base + (pos % page_size);
     }
     const size_t head_step = (size_t)page_size * head_dim;  // between kv heads inside a page
+    // cosine and sine of the token's angles, once per frequency (every head shares them)
+    __shared__ float cs[2][128];
+    if (inv_freq) {
+        for (int j = threadIdx.x; j < half; j += blockDim.x) {
+            const float angle = (float)pos * inv_freq[j];
+            cs[0][j] = cosf(angle);
+            cs[1][j] = sinf(angle);
+        }
+        __syncthreads();
+    }
     const int pairs = (q_heads + kv_heads) * half;
     for (int idx = threadIdx.x; idx < pairs; idx += blockDim.x) {
         const int head = idx / half, j = idx % half;
         T* x = row + (size_t)head * head_dim;
         float x1 = to_float(x[j]), x2 = to_float(x[j + half]);
         if (inv_freq && head < rot_heads) {
-            const float angle = (float)pos * inv_freq[j];
-            const float c = cosf(angle), s = sinf(angle);
+            const float c = cs[0][j], s = cs[1][j];
             const float y1 = x1 * c - x2 * s;
             const float y2 = x2 * c + x1 * s;
             x1 = y1;
@@ -139,8 +243,8 @@ extern "C" int tl_rope_cache_write(void* qkv, int row_stride, int tokens, int q_
                                    const void* token_req, const void* block_table, int bt_stride,
                                    void* k_plane, void* v_plane, int page_size, int act_dtype,
                                    hipStream_t stream) {
-    TL_REQUIRE(tokens >= 0 && q_heads >= 0 && kv_heads >= 0 && head_dim > 0 && head_dim % 2 == 0,
-               "rope_cache_write: bad sizes tokens=%d q_heads=%d kv_heads=%d head_dim=%d", tokens, q_heads, kv_heads, head_dim);
+    TL_REQUIRE(tokens >= 0 && q_heads >= 0 && kv_heads >= 0 && head_dim > 0 && head_dim % 2 == 0 && head_dim <= 256,
+               "rope_cache_write: bad sizes tokens=%d q_heads=%d kv_heads=%d head_dim=%d (even, at most 256)", tokens, q_heads, kv_heads, head_dim);
     TL_REQUIRE(rot_heads <= q_heads + kv_heads, "rope_cache_write: rot_heads %d exceeds q+k heads", rot_heads);
     TL_REQUIRE((k_plane == nullptr) == (v_plane == nullptr), "rope_cache_write: give both planes or none");
     TL_REQUIRE(!k_plane || (block_table && token_req && page_size > 0 && bt_stride > 0),

@@ -115,10 +115,17 @@ union Frag16 {          // 16 bytes: eight bfloat16 as the MFMA wants them, or o
     bf16x8_t v;
 };
 
-template <int R, int MT, int KS, typename TOut>
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + expf(-g)) * u; }
+
+// SW (gate/up product with the SwiGLU gate applied to the accumulators): w holds blocks of 64
+// rows, 32 gate rows followed by the 32 up rows of the same columns; needs R == 4, so that a
+// work-group's strips are [gate 0-15, gate 16-31, up 0-15, up 16-31]; out has N / 2 columns.
+template <int R, int MT, int KS, typename TOut, bool SW = false>
 __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                               const void* __restrict__ bias, int bias_f32,
-                                                              TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+                                                              TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
+                                                              int out_cols = 0) {
+    static_assert(!SW || (R == 4 && KS > 1), "the fused gate needs four strips per work-group");
     __shared__ float red[KS > 1 ? KS * R * MT * 256 : 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
@@ -203,6 +210,25 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
             }
         __syncthreads();
     }
+    if (SW) {
+        for (int pt = wave; pt < 2 * MT; pt += KS) {
+            const int pr = pt / MT, t = pt % MT;
+            f32x4_t gs = f32x4_t{0.f, 0.f, 0.f, 0.f}, us = gs;
+#pragma unroll
+            for (int wv = 0; wv < KS; ++wv) {
+                gs += *(const f32x4_t*)(red + ((size_t)(wv * R * MT + pr * MT + t) * 64 + lane) * 4);
+                us += *(const f32x4_t*)(red + ((size_t)(wv * R * MT + (pr + 2) * MT + t) * 64 + lane) * 4);
+            }
+            const int m = t * 16 + li;
+            const int col = (n0 / 64) * 32 + pr * 16 + 4 * lg;
+            if (m < M) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (col + v < out_cols) out[(size_t)m * ldo + col + v] = from_float<TOut>(silu_mul(gs[v], us[v]));
+            }
+        }
+        return;
+    }
     for (int tile = wave; tile < R * MT; tile += KS) {
         const int r = tile / MT, t = tile % MT;
         f32x4_t sum;
@@ -283,7 +309,7 @@ extern "C" int tl_gemm_skinny_variant(const void* x, const void* w, const void* 
 // =====================================================================================
 // bfloat16 on the matrix cores, many rows (prompt portions): shared-memory tiles.
 //
-// A work-group of four waves owns a BM x BN tile of the output and walks K in slabs of 32.
+// A work-group of four or eight waves owns a BM x BN tile of the output and walks K in slabs of 32.
 // A slab of x (BM rows) and of w (BN rows) is fetched from memory as 16-byte pieces into
 // registers while the previous slab is being multiplied, then parked in shared memory
 // (two buffers, one barrier per slab).  Rows lie 80 bytes apart in shared memory (64 of
@@ -296,16 +322,18 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 #define TK 32                 // K elements per slab
 #define TROW 40               // bfloat16 elements between rows in shared memory (32 + 8 padding)
 
-template <int BM, int BN, int WGM, int WGN, typename TOut>
-__global__ __launch_bounds__(256) void gemm_mfma_tile_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+template <int BM, int BN, int WGM, int WGN, typename TOut, bool SW = false>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tile_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                              const void* __restrict__ bias, int bias_f32,
-                                                             TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
-    static_assert(WGM * WGN == 4, "four waves");
+                                                             TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
+                                                             int out_cols = 0) {
+    static_assert(!SW || (BN / WGN) % 64 == 0, "the fused gate needs whole 64-row blocks per wave");
+    constexpr int NT = 64 * WGM * WGN;                   // threads
     constexpr int WM = BM / WGM, WN = BN / WGN;          // wave tile
     constexpr int FM = WM / 32, FN = WN / 32;            // 32x32 blocks per wave
     constexpr int PIECES = (BM + BN) * (TK / 8);         // 16-byte pieces per slab
-    constexpr int PPT = PIECES / 256;                    // pieces per thread
-    static_assert(PIECES % 256 == 0, "slab must divide over the threads");
+    constexpr int PPT = PIECES / NT;                     // pieces per thread
+    static_assert(PIECES % NT == 0, "slab must divide over the threads");
     __shared__ __attribute__((aligned(16))) bf16_t lds[2][(BM + BN) * TROW];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -320,7 +348,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tile_kernel(const bf16_t* __res
     int kcol[PPT];
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
-        const int p = tid + i * 256;
+        const int p = tid + i * NT;
         const int row = p / (TK / 8), c = p % (TK / 8);
         kcol[i] = c * 8;
         dst[i] = row * TROW + c * 8;
@@ -376,6 +404,22 @@ __global__ __launch_bounds__(256) void gemm_mfma_tile_kernel(const bf16_t* __res
     }
 
     // block result: lane holds column (lane % 32), rows 8 * (v / 4) + 4 * (lane / 32) + v % 4
+    if (SW) {   // even blocks hold gate columns, the next block the up columns of the same outputs
+#pragma unroll
+        for (int j = 0; j + 1 < FN; j += 2) {
+            const int col = (n0 + wn * WN + j * 32) / 2 + (lane & 31);
+            if (col >= out_cols) continue;
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                    if (m < M) out[(size_t)m * ldo + col] = from_float<TOut>(silu_mul(acc[i][j][v], acc[i][j + 1][v]));
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < FN; ++j) {
         const int n = n0 + wn * WN + j * 32 + (lane & 31);
@@ -395,7 +439,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_tile_kernel(const bf16_t* __res
 template <int BM, int BN, int WGM, int WGN>
 static void launch_mfma_tile(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                              int ldx, int ldo, int out_f32, hipStream_t stream) {
-    dim3 grid(((M + BM - 1) / BM) * ((N + BN - 1) / BN)), block(256);
+    dim3 grid(((M + BM - 1) / BM) * ((N + BN - 1) / BN)), block(64 * WGM * WGN);
     if (out_f32)
         gemm_mfma_tile_kernel<BM, BN, WGM, WGN, float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo);
     else
@@ -407,10 +451,11 @@ extern "C" int tl_gemm_tile_variant(const void* x, const void* w, const void* bi
                                     int M, int N, int K, int ldx, int ldo, int out_f32, int BM, int BN, hipStream_t stream) {
     TL_REQUIRE(M > 0 && K % 8 == 0 && ldx % 8 == 0, "gemm_tile: needs M > 0 and K, ldx multiples of 8");
     if (BM == 128 && BN == 128) launch_mfma_tile<128, 128, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else if (BM == 256 && BN == 128) launch_mfma_tile<256, 128, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else if (BM == 128 && BN == 256) launch_mfma_tile<128, 256, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else if (BM == 256 && BN == 128) launch_mfma_tile<256, 128, 4, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else if (BM == 128 && BN == 256) launch_mfma_tile<128, 256, 2, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
     else if (BM == 64 && BN == 128) launch_mfma_tile<64, 128, 1, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
     else if (BM == 64 && BN == 256) launch_mfma_tile<64, 256, 1, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    else if (BM == 256 && BN == 256) launch_mfma_tile<256, 256, 4, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
     else TL_REQUIRE(false, "gemm_tile: no instance BM=%d BN=%d", BM, BN);
     TL_CHECK_LAUNCH("gemm_mfma_tile");
     return TL_OK;
@@ -431,7 +476,12 @@ extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_
     if (M == 0) return TL_OK;
     const bool aligned = K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
     if (dtype == TL_DT_BF16 && aligned && (M > 64 || (M > 32 && N >= 16384))) {
-        if (M > 64) launch_mfma_tile<128, 128, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        // 256 x 128 tiles (eight waves) reuse operands better but need twice as many tiles'
+        // worth of rows and columns to fill the 256 compute units (measured: 750 vs 600 TFLOP/s
+        // on the gate/up product of 2048 tokens, slower than 128 x 128 on the narrow products)
+        const long big_tiles = (long)((M + 255) / 256) * ((N + 127) / 128);
+        if (M > 64 && big_tiles >= 512) launch_mfma_tile<256, 128, 4, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        else if (M > 64) launch_mfma_tile<128, 128, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
         else launch_mfma_tile<64, 128, 1, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
         TL_CHECK_LAUNCH("gemm_mfma_tile");
         return TL_OK;
@@ -444,4 +494,37 @@ extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_
         return TL_OK;
     }
     return tl_gemm_general(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, dtype, out_f32, stream);
+}
+
+// out[M, I] = silu(x g^T) * (x u^T) for bfloat16, with w = the gate and up matrices interleaved
+// in blocks of 32 rows (rows 64 b .. 64 b + 31: gate rows 32 b .., rows 64 b + 32 ..: the up rows
+// of the same columns), padded with zero rows to a multiple of 64.  The gate is applied to the
+// float accumulators, as the reference's fused kernel does
+// (/root/reference/src/torchlet/v10_triton_paged_gqa/kernel/ffn_swiglu.py:139-160).
+extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, int I, int K, int ldx, int ldo,
+                              hipStream_t stream) {
+    TL_REQUIRE(M >= 0 && I > 0 && K > 0 && ldx >= K && ldo >= I, "gemm_swiglu: bad sizes M=%d I=%d K=%d", M, I, K);
+    TL_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
+               "gemm_swiglu: needs K and the row stride of x to be multiples of 8 and 16-byte aligned operands");
+    if (M == 0) return TL_OK;
+    const int N = ((I + 31) / 32) * 64;          // rows of the interleaved matrix
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wb = (const bf16_t*)w;
+    bf16_t* ob = (bf16_t*)out;
+    if (M <= 32) {
+        dim3 grid(N / 64), block(4 * 64);
+        if (M <= 16) gemm_skinny_kernel<4, 1, 4, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
+        else gemm_skinny_kernel<4, 2, 4, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
+    } else if (M <= 64) {
+        dim3 grid(((M + 63) / 64) * ((N + 127) / 128)), block(256);
+        gemm_mfma_tile_kernel<64, 128, 2, 2, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
+    } else if ((long)((M + 255) / 256) * ((N + 127) / 128) >= 512) {
+        dim3 grid(((M + 255) / 256) * ((N + 127) / 128)), block(512);
+        gemm_mfma_tile_kernel<256, 128, 4, 2, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
+    } else {
+        dim3 grid(((M + 127) / 128) * ((N + 127) / 128)), block(256);
+        gemm_mfma_tile_kernel<128, 128, 2, 2, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
+    }
+    TL_CHECK_LAUNCH("gemm_swiglu");
+    return TL_OK;
 }

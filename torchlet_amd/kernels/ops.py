@@ -179,6 +179,33 @@ def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int) -> 
                                          c_int(1 if out.dtype == torch.float32 else 0), c_int(tile_m), c_int(tile_n), _stream()))
 
 
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """The layout :func:`linear_swiglu` wants: blocks of 64 rows, 32 rows of ``gate`` then the
+    32 rows of ``up`` with the same indices; the last block is padded with zero rows."""
+    I, K = gate.shape
+    blocks = -(-I // 32)
+    g = torch.zeros((blocks * 32, K), dtype=gate.dtype, device=gate.device)
+    u = torch.zeros_like(g)
+    g[:I] = gate
+    u[:I] = up
+    return torch.stack((g.view(blocks, 32, K), u.view(blocks, 32, K)), dim=1).reshape(blocks * 64, K).contiguous()
+
+
+def linear_swiglu(x: torch.Tensor, gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = silu(x @ gate.T) * (x @ up.T)`` on the matrix cores with the gate applied to the
+    32-bit accumulators; ``gate_up`` from :func:`interleave_gate_up`, bfloat16 only,
+    ``x [M, K]`` with K a multiple of 8."""
+    M, K = x.shape
+    I = out.shape[1]
+    if x.dtype != torch.bfloat16 or gate_up.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise KernelError("linear_swiglu: bfloat16 only")
+    if gate_up.shape != (-(-I // 32) * 64, K) or out.shape[0] != M or not gate_up.is_contiguous() or x.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError(f"linear_swiglu: shapes x{tuple(x.shape)} w{tuple(gate_up.shape)} out{tuple(out.shape)} do not fit")
+    lib = _lib("gemm")
+    _check(lib, lib.tl_gemm_swiglu(_ptr(x), _ptr(gate_up), _ptr(out), c_int(M), c_int(I), c_int(K),
+                                   c_int(x.stride(0)), c_int(out.stride(0)), _stream()))
+
+
 def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int, rot_heads: int,
                      positions: torch.Tensor, inv_freq: torch.Tensor | None,
                      token_req: torch.Tensor | None = None, block_table: torch.Tensor | None = None,

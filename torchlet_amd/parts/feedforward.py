@@ -1,8 +1,11 @@
 """Dense SwiGLU feed-forward: ``down(silu(gate(h)) * up(h))``, no biases
 (/root/reference/src/torchlet/v10_triton_paged_gqa/layer/ffn_swiglu.py:22-59).
 
-``gate_proj`` and ``up_proj`` are stacked into one ``[2I, H]`` matrix at load time so that
-one matrix product reads ``h`` once; the gate is applied to the two halves of its result.
+``gate_proj`` and ``up_proj`` are put into one matrix at load time so that one matrix
+product reads ``h`` once.  In bfloat16 (hidden a multiple of 8) the two are interleaved in
+blocks of 32 rows and the gate ``silu(g) * u`` is applied to the 32-bit accumulators inside
+the product's kernel, as the reference's fused kernel does (kernel/ffn_swiglu.py:139-160);
+otherwise they are stacked ``[gate; up]`` and a separate kernel applies the gate.
 """
 from __future__ import annotations
 
@@ -29,15 +32,24 @@ class SwiGLU(FeedForward):
         }
 
     def load_weights(self, tensors):
-        self.gate_up = self._place(torch.cat((tensors["gate_proj.weight"], tensors["up_proj.weight"]), dim=0), "matrix")
+        self.fused_gate = self.dtype == torch.bfloat16 and self.hidden % 8 == 0
+        if self.fused_gate:
+            gate = self._place(tensors["gate_proj.weight"], "matrix")
+            up = self._place(tensors["up_proj.weight"], "matrix")
+            self.gate_up = ops.interleave_gate_up(gate, up)
+        else:
+            self.gate_up = self._place(torch.cat((tensors["gate_proj.weight"], tensors["up_proj.weight"]), dim=0), "matrix")
         self.down = self._place(tensors["down_proj.weight"], "matrix")
 
     def forward(self, h, ctx):
         T = h.shape[0]
-        gu = torch.empty((T, 2 * self.inter), dtype=self.dtype, device=h.device)
-        ops.linear(h, self.gate_up, None, gu)
         z = torch.empty((T, self.inter), dtype=self.dtype, device=h.device)
-        ops.swiglu(gu, z)
+        if self.fused_gate:
+            ops.linear_swiglu(h, self.gate_up, z)
+        else:
+            gu = torch.empty((T, 2 * self.inter), dtype=self.dtype, device=h.device)
+            ops.linear(h, self.gate_up, None, gu)
+            ops.swiglu(gu, z)
         y = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
         ops.linear(z, self.down, None, y)
         return y

@@ -47,6 +47,8 @@ def parse_args(argv=None):
     p.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    p.add_argument("--only", choices=["decode", "prefill"], default=None,
+                   help="run one part only (for profiling): the decode steps at --batch, or the 2048-token prefill")
     return p.parse_args(argv)
 
 
@@ -165,12 +167,21 @@ def main(argv=None) -> int:
         print("bench.py needs an MI355X; no GPU is visible", file=sys.stderr)
         return 1
     cfg, model = build(args.layers, args.dtype)
+    if args.only == "prefill":
+        pms = time_prefill(model, 2048)
+        flops = prefill_flops(cfg, 2048)
+        print(json.dumps({"prefill": {"value": round(2048 * 1e3 / pms, 1), "tokens": 2048, "ms": round(pms, 3),
+                                      "frac": round(flops / (pms * 1e-3) / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12), 4)},
+                          "layers": args.layers}))
+        return 0
+    if args.only == "decode":
+        args.no_points = True
     ms = time_decode(model, args.batch, args.steps, args.warmup)
     mean_ctx = CONTEXT + args.warmup + args.steps / 2.0
     nbytes = decode_bytes(cfg, model, args.batch, mean_ctx)
     achieved = nbytes / (ms * 1e-3) / 1e9
     result = {
-        "metric": "decode tokens/s, Qwen2.5-7B shape, batch 8, 2048-token contexts, one MI355X",
+        "metric": f"decode tokens/s, Qwen2.5-7B shape, batch {args.batch}, 2048-token contexts, one MI355X",
         "value": round(args.batch * 1e3 / ms, 2),
         "unit": "tokens/s",
         "n_gpus": 1,

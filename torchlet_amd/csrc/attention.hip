@@ -278,23 +278,47 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
 #pragma unroll
     for (int t = 0; t < ATM_DT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int ch = ch_begin + wave; ch < ch_end; ch += 4) {
+    // Keys and values of a chunk are fetched together: the value loads do not wait for the
+    // scores.  (Fetching the next chunk ahead as well doubles the registers, halves the waves
+    // per SIMD and measured slower for decode and prompt steps alike.)
+    FragK kf[2][ATM_DC];
+    uint2 vfa[ATM_DT], vfb[ATM_DT];
+#define ATM_FETCH(KF, VA, VB, chunk)                                                                         \
+    {                                                                                                        \
+        const int kb_ = (chunk) * 32;                                                                        \
+        _Pragma("unroll") for (int hf = 0; hf < 2; ++hf) {                                                   \
+            const int key = min(kb_ + 16 * hf + li, key_hi - 1);                                             \
+            const int pg = bt[key / page];                                                                   \
+            const bf16_t* krow = kp + (((size_t)pg * a.kv_heads + kvh) * page + (key % page)) * AT_HD;       \
+            _Pragma("unroll") for (int c = 0; c < ATM_DC; ++c) {                                             \
+                const int d = 32 * c + 8 * g;                                                                \
+                KF[hf][c].u = (d + 8 <= AT_HD) ? *(const uint4*)(krow + d) : make_uint4(0, 0, 0, 0);         \
+            }                                                                                                \
+        }                                                                                                    \
+        const int ka = kb_ + 4 * g, kb = kb_ + 16 + 4 * g;                                                   \
+        const bool oka = ka < key_hi, okb = kb < key_hi;                                                     \
+        const int pga = oka ? bt[ka / page] : 0, pgb = okb ? bt[kb / page] : 0;                              \
+        const bf16_t* va = vp + ((size_t)pga * a.kv_heads + kvh) * AT_HD * page + (ka % page);               \
+        const bf16_t* vb = vp + ((size_t)pgb * a.kv_heads + kvh) * AT_HD * page + (kb % page);               \
+        _Pragma("unroll") for (int t = 0; t < ATM_DT; ++t) {                                                 \
+            const size_t drow = (size_t)(16 * t + li) * page;                                                \
+            VA[t] = oka ? *(const uint2*)(va + drow) : make_uint2(0, 0);                                     \
+            VB[t] = okb ? *(const uint2*)(vb + drow) : make_uint2(0, 0);                                     \
+        }                                                                                                    \
+    }
+
+    int ch = ch_begin + wave;
+    if (ch < ch_end) ATM_FETCH(kf, vfa, vfb, ch)
+    for (; ch < ch_end; ch += 4) {
         const int kbase = ch * 32;
         // ---- scores: two halves of 16 keys
         f32x4_t sc[2];
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            const int key = min(kbase + 16 * hf + li, key_hi - 1);
-            const int pg = bt[key / page];
-            const bf16_t* krow = kp + (((size_t)pg * a.kv_heads + kvh) * page + (key % page)) * AT_HD;
             f32x4_t sacc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < ATM_DC; ++c) {
-                const int d = 32 * c + 8 * g;
-                FragK kf;
-                kf.u = (d + 8 <= AT_HD) ? *(const uint4*)(krow + d) : make_uint4(0, 0, 0, 0);
-                sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sacc, 0, 0, 0);
-            }
+            for (int c = 0; c < ATM_DC; ++c)
+                sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[hf][c].v, qf[c].v, sacc, 0, 0, 0);
             sc[hf] = sacc;
         }
         // ---- mask, running maximum, probabilities
@@ -325,20 +349,6 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
         l = l * alpha + psum;
         m = m_new;
         // ---- values: O^T += V^T . P^T
-        uint2 vfa[ATM_DT], vfb[ATM_DT];
-        {
-            const int ka = kbase + 4 * g, kb = kbase + 16 + 4 * g;
-            const bool oka = ka < key_hi, okb = kb < key_hi;
-            const int pga = oka ? bt[ka / page] : 0, pgb = okb ? bt[kb / page] : 0;
-            const bf16_t* va = vp + ((size_t)pga * a.kv_heads + kvh) * AT_HD * page + (ka % page);
-            const bf16_t* vb = vp + ((size_t)pgb * a.kv_heads + kvh) * AT_HD * page + (kb % page);
-#pragma unroll
-            for (int t = 0; t < ATM_DT; ++t) {
-                const size_t drow = (size_t)(16 * t + li) * page;
-                vfa[t] = oka ? *(const uint2*)(va + drow) : make_uint2(0, 0);
-                vfb[t] = okb ? *(const uint2*)(vb + drow) : make_uint2(0, 0);
-            }
-        }
 #pragma unroll
         for (int t = 0; t < ATM_DT; ++t) {
             FragK vf;
@@ -347,7 +357,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
             acc[t] *= alpha;
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[t], 0, 0, 0);
         }
+        if (ch + 4 < ch_end) ATM_FETCH(kf, vfa, vfb, ch + 4)
     }
+#undef ATM_FETCH
 
     // ---- merge the four waves: 2,3 -> 0,1, then 1 -> 0
 #pragma unroll
@@ -402,22 +414,41 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
 }
 
 // out[row] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s over the parts of a row.
+// The parts are read eight at a time with all loads issued before the first use.
 template <typename T>
 __global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                        T* __restrict__ out, int splits) {
     const size_t r = blockIdx.x;
-    const float* ml = part_ml + r * splits * 2;
-    float mx = -INFINITY;
-    for (int s = 0; s < splits; ++s) mx = fmaxf(mx, ml[2 * s]);
-    float denom = 0.f;
-    for (int s = 0; s < splits; ++s)
-        if (ml[2 * s] != -INFINITY) denom += expf(ml[2 * s] - mx) * ml[2 * s + 1];
-    for (int d = threadIdx.x; d < AT_HD; d += blockDim.x) {
-        float num = 0.f;
-        for (int s = 0; s < splits; ++s)
-            if (ml[2 * s] != -INFINITY) num += expf(ml[2 * s] - mx) * part_o[(r * splits + s) * AT_HD + d];
-        out[r * AT_HD + d] = from_float<T>(num / denom);
+    const float2* ml = (const float2*)(part_ml + r * splits * 2);
+    const float* po = part_o + r * splits * AT_HD;
+    const int d = threadIdx.x;                     // blockDim.x == AT_HD
+    float mx = -INFINITY, denom = 0.f, num = 0.f;
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+        float2 w[8];
+        float o[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int sp = min(s0 + i, splits - 1);
+            w[i] = ml[sp];
+            o[i] = po[(size_t)sp * AT_HD + d];
+        }
+        float m8 = mx;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (s0 + i < splits) m8 = fmaxf(m8, w[i].x);
+        const float rescale = (mx == -INFINITY) ? 0.f : expf(mx - m8);
+        denom *= rescale;
+        num *= rescale;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (s0 + i < splits && w[i].x != -INFINITY) {
+                const float e = expf(w[i].x - m8);
+                denom += e * w[i].y;
+                num += e * o[i];
+            }
+        mx = m8;
     }
+    out[r * AT_HD + d] = from_float<T>(num / denom);
 }
 
 extern "C" int tl_attention_head_dim() { return AT_HD; }
@@ -454,7 +485,7 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
     else TL_REQUIRE(false, "attention: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("paged_attention");
     if (splits > 1) {
-        dim3 mgrid((unsigned)((size_t)tokens * heads)), mblock(AT_HD < 64 ? 64 : (AT_HD > 256 ? 256 : AT_HD));
+        dim3 mgrid((unsigned)((size_t)tokens * heads)), mblock(AT_HD);
         if (dtype == TL_DT_F32) attention_merge_kernel<float><<<mgrid, mblock, 0, stream>>>((const float*)part_o, (const float*)part_ml, (float*)out, splits);
         else attention_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, splits);
         TL_CHECK_LAUNCH("attention_merge");

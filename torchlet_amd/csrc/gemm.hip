@@ -309,32 +309,49 @@ extern "C" int tl_gemm_skinny_variant(const void* x, const void* w, const void* 
 // =====================================================================================
 // bfloat16 on the matrix cores, many rows (prompt portions): shared-memory tiles.
 //
-// A work-group of four or eight waves owns a BM x BN tile of the output and walks K in slabs of 32.
+// A work-group of four or eight waves owns a BM x BN tile of the output and walks K in slabs of TK
+// (32 or 64) elements.
 // A slab of x (BM rows) and of w (BN rows) is fetched from memory as 16-byte pieces into
 // registers while the previous slab is being multiplied, then parked in shared memory
-// (two buffers, one barrier per slab).  Rows lie 80 bytes apart in shared memory (64 of
-// data, 16 of padding) so that the 16-byte operand reads of v_mfma_f32_32x32x16_bf16 do not
+// (two buffers, one barrier per slab).  Rows lie 2 TK + 16 bytes apart in shared memory (16 of
+// padding) so that the 16-byte operand reads of v_mfma_f32_32x32x16_bf16 do not
 // collide on banks.  Waves are laid out WGM x WGN over the tile; each multiplies
 // (BM / WGM) x (BN / WGN) as blocks of 32 x 32 with float accumulators.
 // Needs K % 8 == 0 and 16-byte aligned rows.
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-#define TK 32                 // K elements per slab
-#define TROW 40               // bfloat16 elements between rows in shared memory (32 + 8 padding)
+// Which tile a shape gets (measured on MI355X at Qwen2.5-7B sizes, 2048 and 512 rows):
+//   * 256 x 256 with slabs of 64 (eight waves) reuses operands best (840 TFLOP/s on the
+//     gate/up product) but needs over a thousand such tiles to keep 256 compute units busy;
+//   * otherwise 128 x 128 with slabs of 64 (two work-groups fit a compute unit: 512 at once),
+//     except when the tile count lies between 512 and 768, where slabs of 32 (three fit) avoid
+//     a second, nearly empty round;
+//   * up to 64 rows: 64 x 128.
+enum TileChoice { TILE_64x128, TILE_128x128_K32, TILE_128x128_K64, TILE_256x256 };
+static TileChoice pick_tile(int M, int N) {
+    if (M <= 64) return TILE_64x128;
+    const long big = (long)((M + 255) / 256) * ((N + 255) / 256);
+    if (big >= 1024) return TILE_256x256;
+    const long wgs = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (wgs > 512 && wgs <= 768) return TILE_128x128_K32;
+    return TILE_128x128_K64;
+}
 
-template <int BM, int BN, int WGM, int WGN, typename TOut, bool SW = false>
+template <int BM, int BN, int WGM, int WGN, typename TOut, bool SW = false, int TK = 32>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tile_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                              const void* __restrict__ bias, int bias_f32,
                                                              TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
                                                              int out_cols = 0) {
     static_assert(!SW || (BN / WGN) % 64 == 0, "the fused gate needs whole 64-row blocks per wave");
+    constexpr int TROW = TK + 8;                         // elements between rows in shared memory (16 bytes of padding)
     constexpr int NT = 64 * WGM * WGN;                   // threads
     constexpr int WM = BM / WGM, WN = BN / WGN;          // wave tile
     constexpr int FM = WM / 32, FN = WN / 32;            // 32x32 blocks per wave
     constexpr int PIECES = (BM + BN) * (TK / 8);         // 16-byte pieces per slab
     constexpr int PPT = PIECES / NT;                     // pieces per thread
     static_assert(PIECES % NT == 0, "slab must divide over the threads");
-    __shared__ __attribute__((aligned(16))) bf16_t lds[2][(BM + BN) * TROW];
+    extern __shared__ __attribute__((aligned(16))) bf16_t lds_raw[];
+    bf16_t (*lds)[(BM + BN) * TROW] = (bf16_t (*)[(BM + BN) * TROW])lds_raw;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -436,27 +453,51 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tile_kernel(const bf
     }
 }
 
-template <int BM, int BN, int WGM, int WGN>
-static void launch_mfma_tile(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
-                             int ldx, int ldo, int out_f32, hipStream_t stream) {
+// Shared memory of a tile kernel: two buffers of (BM + BN) rows of TK + 8 elements.  Beyond 64 KB
+// the kernel has to be allowed its size once per process.
+template <typename Kernel>
+static hipError_t allow_lds(Kernel kernel, size_t bytes) {
+    if (bytes <= 65536) return hipSuccess;
+    return hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+template <int BM, int BN, int WGM, int WGN, typename TOut, bool SW, int TK>
+static int launch_mfma_tile_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                              int ldx, int ldo, int out_cols, hipStream_t stream) {
+    constexpr size_t lds = 2 * (size_t)(BM + BN) * (TK + 8) * sizeof(bf16_t);
+    auto kernel = gemm_mfma_tile_kernel<BM, BN, WGM, WGN, TOut, SW, TK>;
+    static hipError_t allowed = allow_lds(kernel, lds);
+    if (allowed != hipSuccess) {
+        tl_set_error("gemm_mfma_tile: cannot get %zu bytes of shared memory: %s", lds, hipGetErrorString(allowed));
+        return TL_ERR_HIP;
+    }
     dim3 grid(((M + BM - 1) / BM) * ((N + BN - 1) / BN)), block(64 * WGM * WGN);
-    if (out_f32)
-        gemm_mfma_tile_kernel<BM, BN, WGM, WGN, float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo);
-    else
-        gemm_mfma_tile_kernel<BM, BN, WGM, WGN, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo);
+    kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols);
+    return TL_OK;
+}
+
+template <int BM, int BN, int WGM, int WGN, int TK = 32>
+static int launch_mfma_tile(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                            int ldx, int ldo, int out_f32, hipStream_t stream) {
+    if (out_f32) return launch_mfma_tile_t<BM, BN, WGM, WGN, float, false, TK>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
+    return launch_mfma_tile_t<BM, BN, WGM, WGN, bf16_t, false, TK>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
 }
 
 // One named tile shape of the many-rows kernel (tests cover each; tuning times them).
 extern "C" int tl_gemm_tile_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
-                                    int M, int N, int K, int ldx, int ldo, int out_f32, int BM, int BN, hipStream_t stream) {
+                                    int M, int N, int K, int ldx, int ldo, int out_f32, int BM, int BN, int TK, hipStream_t stream) {
     TL_REQUIRE(M > 0 && K % 8 == 0 && ldx % 8 == 0, "gemm_tile: needs M > 0 and K, ldx multiples of 8");
-    if (BM == 128 && BN == 128) launch_mfma_tile<128, 128, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else if (BM == 256 && BN == 128) launch_mfma_tile<256, 128, 4, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else if (BM == 128 && BN == 256) launch_mfma_tile<128, 256, 2, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else if (BM == 64 && BN == 128) launch_mfma_tile<64, 128, 1, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else if (BM == 64 && BN == 256) launch_mfma_tile<64, 256, 1, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else if (BM == 256 && BN == 256) launch_mfma_tile<256, 256, 4, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-    else TL_REQUIRE(false, "gemm_tile: no instance BM=%d BN=%d", BM, BN);
+    int rc = -1;
+#define TL_TILE_CASE(bm, bn, gm, gn, tk) \
+    if (BM == bm && BN == bn && TK == tk) rc = launch_mfma_tile<bm, bn, gm, gn, tk>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    TL_TILE_CASE(128, 128, 2, 2, 32) TL_TILE_CASE(128, 128, 2, 2, 64)
+    TL_TILE_CASE(256, 128, 4, 2, 32) TL_TILE_CASE(256, 128, 4, 2, 64)
+    TL_TILE_CASE(128, 256, 2, 4, 32) TL_TILE_CASE(128, 256, 2, 4, 64)
+    TL_TILE_CASE(64, 128, 1, 4, 32) TL_TILE_CASE(64, 128, 2, 2, 64)
+    TL_TILE_CASE(256, 256, 4, 2, 32) TL_TILE_CASE(256, 256, 4, 2, 64)
+#undef TL_TILE_CASE
+    TL_REQUIRE(rc != -1, "gemm_tile: no instance BM=%d BN=%d TK=%d", BM, BN, TK);
+    if (rc != TL_OK) return rc;
     TL_CHECK_LAUNCH("gemm_mfma_tile");
     return TL_OK;
 }
@@ -476,13 +517,14 @@ extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_
     if (M == 0) return TL_OK;
     const bool aligned = K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
     if (dtype == TL_DT_BF16 && aligned && (M > 64 || (M > 32 && N >= 16384))) {
-        // 256 x 128 tiles (eight waves) reuse operands better but need twice as many tiles'
-        // worth of rows and columns to fill the 256 compute units (measured: 750 vs 600 TFLOP/s
-        // on the gate/up product of 2048 tokens, slower than 128 x 128 on the narrow products)
-        const long big_tiles = (long)((M + 255) / 256) * ((N + 127) / 128);
-        if (M > 64 && big_tiles >= 512) launch_mfma_tile<256, 128, 4, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-        else if (M > 64) launch_mfma_tile<128, 128, 2, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
-        else launch_mfma_tile<64, 128, 1, 4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+        int rc;
+        switch (pick_tile(M, N)) {
+        case TILE_256x256: rc = launch_mfma_tile<256, 256, 4, 2, 64>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream); break;
+        case TILE_128x128_K32: rc = launch_mfma_tile<128, 128, 2, 2, 32>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream); break;
+        case TILE_128x128_K64: rc = launch_mfma_tile<128, 128, 2, 2, 64>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream); break;
+        default: rc = launch_mfma_tile<64, 128, 2, 2, 64>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream); break;
+        }
+        if (rc != TL_OK) return rc;
         TL_CHECK_LAUNCH("gemm_mfma_tile");
         return TL_OK;
     }
@@ -515,15 +557,15 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
         dim3 grid(N / 64), block(4 * 64);
         if (M <= 16) gemm_skinny_kernel<4, 1, 4, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
         else gemm_skinny_kernel<4, 2, 4, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
-    } else if (M <= 64) {
-        dim3 grid(((M + 63) / 64) * ((N + 127) / 128)), block(256);
-        gemm_mfma_tile_kernel<64, 128, 2, 2, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
-    } else if ((long)((M + 255) / 256) * ((N + 127) / 128) >= 512) {
-        dim3 grid(((M + 255) / 256) * ((N + 127) / 128)), block(512);
-        gemm_mfma_tile_kernel<256, 128, 4, 2, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
     } else {
-        dim3 grid(((M + 127) / 128) * ((N + 127) / 128)), block(256);
-        gemm_mfma_tile_kernel<128, 128, 2, 2, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
+        int rc;
+        switch (pick_tile(M, N)) {
+        case TILE_256x256: rc = launch_mfma_tile_t<256, 256, 4, 2, bf16_t, true, 64>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
+        case TILE_128x128_K32: rc = launch_mfma_tile_t<128, 128, 2, 2, bf16_t, true, 32>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
+        case TILE_128x128_K64: rc = launch_mfma_tile_t<128, 128, 2, 2, bf16_t, true, 64>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
+        default: rc = launch_mfma_tile_t<64, 128, 2, 2, bf16_t, true, 64>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream); break;
+        }
+        if (rc != TL_OK) return rc;
     }
     TL_CHECK_LAUNCH("gemm_swiglu");
     return TL_OK;

@@ -166,7 +166,7 @@ def linear_few_rows_variant(x, weight, bias, out, strips_per_wave: int, waves_al
                                            c_int(waves_along_k), _stream()))
 
 
-def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int) -> None:
+def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int, slab: int = 32) -> None:
     """One named tile shape of the many-rows matrix-core kernel (for tests and tuning)."""
     M, K = x.shape
     N = weight.shape[0]
@@ -176,7 +176,7 @@ def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int) -> 
     lib = _lib("gemm")
     _check(lib, lib.tl_gemm_tile_variant(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N),
                                          c_int(K), c_int(x.stride(0)), c_int(out.stride(0)),
-                                         c_int(1 if out.dtype == torch.float32 else 0), c_int(tile_m), c_int(tile_n), _stream()))
+                                         c_int(1 if out.dtype == torch.float32 else 0), c_int(tile_m), c_int(tile_n), c_int(slab), _stream()))
 
 
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

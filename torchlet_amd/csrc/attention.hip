@@ -272,6 +272,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
     const int* bt = a.block_table + (size_t)req * a.bt_stride;
     const int page = a.page;
     const float scale2 = a.scale * 1.44269504088896341f;
+    // smallest query position and largest window start over the rows of the tile (uniform)
+    const int tile_pos_min = ctx + tok0;
+    const int tile_lo_max = a.window > 0 ? max(0, ctx + tok0 + ntok - 1 - a.window + 1) : 0;
 
     float m = -INFINITY, l = 0.f;
     f32x4_t acc[ATM_DT];
@@ -322,18 +325,31 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
             sc[hf] = sacc;
         }
         // ---- mask, running maximum, probabilities
+        // A chunk that every row of the tile sees whole (all but those on the diagonal, at a
+        // window's edge or at the end of the keys) needs no mask: the branch is uniform.
         float s[8];
         float mloc = -INFINITY;
+        if (kbase + 31 <= tile_pos_min && kbase >= tile_lo_max) {
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
+            for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int key = kbase + 16 * hf + 4 * g + v;
-                const bool seen = row_ok && key <= r_pos && key >= r_lo;
-                const float x = seen ? sc[hf][v] * scale2 : -INFINITY;
-                s[4 * hf + v] = x;
-                mloc = fmaxf(mloc, x);
-            }
+                for (int v = 0; v < 4; ++v) {
+                    const float x = sc[hf][v] * scale2;
+                    s[4 * hf + v] = x;
+                    mloc = fmaxf(mloc, x);
+                }
+        } else {
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int key = kbase + 16 * hf + 4 * g + v;
+                    const bool seen = row_ok && key <= r_pos && key >= r_lo;
+                    const float x = seen ? sc[hf][v] * scale2 : -INFINITY;
+                    s[4 * hf + v] = x;
+                    mloc = fmaxf(mloc, x);
+                }
+        }
         mloc = fmaxf(mloc, __shfl_xor(mloc, 16, TL_WAVE));
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TL_WAVE));
         const float m_new = fmaxf(m, mloc);
@@ -344,17 +360,18 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
         for (int i = 0; i < 8; ++i) {
             const float p = (s[i] == -INFINITY) ? 0.f : fast_exp2(s[i] - m_new);
             psum += p;
-            pf.e[i] = from_float<bf16_t>(p).bits;
+            pf.v[i] = (__bf16)p;
         }
         l = l * alpha + psum;
+        // ---- values: O^T += V^T . P^T; the accumulators are rescaled only when some row's maximum moved
+        const bool moved = __any(m_new != m);
         m = m_new;
-        // ---- values: O^T += V^T . P^T
 #pragma unroll
         for (int t = 0; t < ATM_DT; ++t) {
             FragK vf;
             vf.h[0] = vfa[t];
             vf.h[1] = vfb[t];
-            acc[t] *= alpha;
+            if (moved) acc[t] *= alpha;
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[t], 0, 0, 0);
         }
         if (ch + 4 < ch_end) ATM_FETCH(kf, vfa, vfb, ch + 4)

@@ -14,14 +14,10 @@ __device__ __forceinline__ float to_float(bf16_t v) { return __uint_as_float(((u
 template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) {
-    uint32_t u = __float_as_uint(v);
+    // gfx950 converts in hardware (v_cvt_pk_bf16_f32): round to nearest, ties to even, NaN kept
+    const __bf16 h = (__bf16)v;
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) {           // NaN stays NaN
-        r.bits = (uint16_t)((u >> 16) | 0x0040u);
-    } else {
-        u += 0x7fffu + ((u >> 16) & 1u);             // round to nearest, ties to even
-        r.bits = (uint16_t)(u >> 16);
-    }
+    __builtin_memcpy(&r.bits, &h, sizeof(r.bits));
     return r;
 }
 

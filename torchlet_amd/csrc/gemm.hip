@@ -355,9 +355,26 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tile_kernel(const bf
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
-    // neighbouring work-groups share weight tiles: walk M fastest within a band of N
-    const int tiles_m = (M + BM - 1) / BM;
-    const int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
+    // Which tile this work-group owns.  Work-groups are dealt to the 8 XCDs round-robin by
+    // blockIdx, and each XCD has an L2 of its own: give every XCD a contiguous range of
+    // "logical" tile numbers, and number tiles so that 64 consecutive ones (what an XCD runs at
+    // a time) form an 8 x 8 block of the output, so that each operand tile it fetches is used
+    // by eight work-groups out of its L2.
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    int lid;
+    {
+        const int total = gridDim.x, xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
+        lid = xcd * (total / 8) + min(xcd, total % 8) + idx;
+    }
+    int tm, tn;
+    {
+        const int per_group = 8 * tiles_n;
+        const int first_m = (lid / per_group) * 8;
+        const int rows = min(tiles_m - first_m, 8);
+        tm = first_m + (lid % per_group) % rows;
+        tn = (lid % per_group) / rows;
+    }
+    const int m0 = tm * BM, n0 = tn * BN;
 
     // which pieces this thread fetches: piece p -> (row, 8-element column) of the stacked [x rows; w rows] slab
     const bf16_t* src[PPT];

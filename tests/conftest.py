@@ -43,6 +43,7 @@ def cpu_ops(monkeypatch):
     from torchlet_amd.kernels import ops
 
     for name in ("attention_tile_tokens", "load", "embedding", "add_rmsnorm", "linear", "rope_cache_write",
-                 "paged_attention", "swiglu", "sample", "interleave_gate_up", "linear_swiglu"):
+                 "paged_attention", "swiglu", "sample", "interleave_gate_up", "linear_swiglu",
+                 "prefill_attention_tile_tokens", "paged_attention_prefill"):
         monkeypatch.setattr(ops, name, getattr(emulated_ops, name))
     return ops

@@ -68,8 +68,13 @@ def rope_cache_write(qkv, q_heads, kv_heads, head_dim, rot_heads, positions, inv
 
 def paged_attention(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles,
                     tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale, splits=1, general=False):
+    _attend(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles,
+            tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale)
+
+
+def _attend(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles,
+            tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale):
     group = num_heads // num_kv_heads
-    covered = torch.zeros(q.shape[0], dtype=torch.bool)
     for tile in range(num_tiles):
         r = int(tile_req[tile]); t0 = int(tile_tok0[tile])
         first = int(req_indptr[r]); n_new = int(req_indptr[r + 1]) - first; ctx = int(ctx_lens[r])
@@ -86,8 +91,6 @@ def paged_attention(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens,
             s = torch.einsum("hd,nhd->hn", qi, kk) * scale
             o = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
             out[first + i] = o.reshape(-1).to(out.dtype)
-            covered[first + i] = True
-    assert bool(covered.all()), "tiles do not cover every token"
 
 
 def interleave_gate_up(gate, up):
@@ -106,6 +109,21 @@ def linear_swiglu(x, gate_up, out):
     g = x.float() @ w[:, 0].reshape(-1, K)[:I].T
     u = x.float() @ w[:, 1].reshape(-1, K)[:I].T
     out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+
+
+PREFILL_ATTENTION_ROWS = 64
+PREFILL_ATTENTION_MAX_HEAD_DIM = 128
+
+
+def prefill_attention_tile_tokens(num_heads, num_kv_heads):
+    group = num_heads // num_kv_heads
+    return max(1, PREFILL_ATTENTION_ROWS // min(group, ATTENTION_ROWS))
+
+
+def paged_attention_prefill(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles,
+                            tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale):
+    _attend(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles,
+            tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale)
 
 
 def swiglu(gate_up, out):

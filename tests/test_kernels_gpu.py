@@ -285,6 +285,55 @@ def test_paged_attention(ops, dtype, general, nh, nkv, hd, page, window, splits)
         torch.testing.assert_close(got[a:b], ref, **tol)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page,window", [
+    (4, 2, 16, 16, 0), (3, 1, 32, 8, 0), (28, 4, 128, 16, 0), (6, 6, 48, 4, 0), (20, 1, 64, 16, 0),
+    (4, 2, 16, 16, 13), (8, 2, 80, 32, 29), (14, 2, 128, 64, 40), (5, 5, 112, 12, 70),
+])
+def test_paged_attention_prompt_portions(ops, nh, nkv, hd, page, window):
+    """The shared-memory kernel for prompt portions: whole prompts, portions on top of a cached
+    context (also one that starts inside a page and inside a 32-key chunk), a single token."""
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(14)
+    lens, ctxs = [150, 37, 70, 1, 64], [0, 150, 43, 99, 64]
+    R, T = len(lens), sum(lens)
+    totals = [a + b for a, b in zip(lens, ctxs)]
+    max_blocks = (max(totals) + page - 1) // page + 1
+    pages = R * max_blocks + 1
+    bt = (torch.randperm(pages - 1, generator=g)[: R * max_blocks] + 1).view(R, max_blocks).int()
+    q = torch.randn(T, nh * hd, generator=g).to(dtype)
+    kp = torch.randn(pages, nkv, page, hd, generator=g).to(dtype)
+    vp = torch.randn(pages, nkv, hd, page, generator=g).to(dtype)
+    ks, vs = [], []
+    for r in range(R):
+        k = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
+        v = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
+        k[min(3, totals[r] - 1)] *= 3.0
+        for p in range(totals[r]):
+            kp[bt[r, p // page], :, p % page] = k[p]
+            vp[bt[r, p // page], :, :, p % page] = v[p]
+        ks.append(k); vs.append(v)
+    indptr = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    tq = ops.prefill_attention_tile_tokens(nh, nkv)
+    tile_req, tile_tok0 = [], []
+    for r, n in enumerate(lens):
+        for t0 in range(0, n, tq):
+            tile_req.append(r); tile_tok0.append(t0)
+    out = torch.full((T, nh * hd), float("nan"), dtype=dtype, device="cuda")
+    wide = torch.zeros(T, nh * hd + 32, dtype=dtype, device="cuda")
+    wide[:, : nh * hd] = q.cuda()
+    ops.paged_attention_prefill(wide[:, : nh * hd], out, kp.cuda(), vp.cuda(), bt.cuda(), indptr.cuda(),
+                                torch.tensor(ctxs, dtype=torch.int32).cuda(), torch.tensor(tile_req, dtype=torch.int32).cuda(),
+                                torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq, nh, nkv, hd, page, window,
+                                1.0 / math.sqrt(hd))
+    got = out.cpu().double().view(T, nh, hd)
+    for r in range(R):
+        a, b = int(indptr[r]), int(indptr[r + 1])
+        ref = _attention_ref(q[a:b].double().view(-1, nh, hd), ks[r].double(), vs[r].double(), window)
+        tol = _tol(dtype)
+        tol = dict(rtol=tol["rtol"], atol=tol["atol"] + 2 ** -9 * float(vs[r].abs().max()))
+        torch.testing.assert_close(got[a:b], ref, **tol)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,I", [(3, 200), (17, 1001)])
 def test_swiglu(ops, dtype, T, I):

@@ -108,3 +108,18 @@ def test_decode_steps_replayed_as_graphs(model_folders, expected, name, dtype):
             runner.release(r)
     assert runner.graph_replays >= 20 and len(runner._graphs) >= 2
     scenarios.check(steps, out, exp, TOL[dtype], f"graphs/{name}/{dtype}")
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("mode", ["portions", "mixed"])
+def test_prompt_portion_attention_kernel_in_the_engine(model_folders, expected, monkeypatch, name, mode):
+    """The shared-memory attention kernel for prompt portions is used from 4096-token contexts
+    on; here it is switched on for every step so that the tiny models exercise it, together
+    with the split of a step's requests between the two attention kernels."""
+    from torchlet_amd.parts import attention
+    monkeypatch.setattr(attention, "_PORTION_MIN_CONTEXT", 0)
+    monkeypatch.setattr(attention, "_PORTION_MIN_TOKENS", 3)
+    reqs, exp = expected(name)
+    steps = scenarios.number(getattr(scenarios, mode)(reqs))
+    out = _run_in_process(model_folders[name], "bfloat16", steps, tiny_models.PAGE_SIZES[name], scenarios.max_tokens_needed(steps))
+    scenarios.check(steps, out, exp, TOL["bfloat16"], f"portion kernel/{name}/{mode}")

@@ -39,8 +39,21 @@ struct AttnArgs {
     float* part_o;            // [tokens * heads, splits, HD] (splits > 1)
     float* part_ml;           // [tokens * heads, splits, 2]
     int q_stride, bt_stride, heads, kv_heads, page, window, tq, gcap, splits;
+    int page_shift;           // log2(page) when page is a power of two, else -1
     float scale;
 };
+
+// key position -> (logical block, offset in its page); a shift and a mask for the usual
+// power-of-two pages (an integer division by a run-time page size costs ~25 instructions)
+__device__ __forceinline__ void split_key(int key, int page, int shift, int& blk, int& off) {
+    if (shift >= 0) {
+        blk = key >> shift;
+        off = key & (page - 1);
+    } else {
+        blk = key / page;
+        off = key - blk * page;
+    }
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
@@ -218,6 +231,7 @@ union FragK {
 #define ATM_DC ((AT_HD + 31) / 32)
 #define ATM_DT (AT_HD / 16)
 #define ATM_SLOT (ATM_DT * 256 + 128)      // floats one wave parks in shared memory
+#define ATM_BT_MAX 2048                    // block-table entries a work-group keeps in shared memory
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -269,8 +283,20 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
 
     const bf16_t* kp = (const bf16_t*)a.k_plane;
     const bf16_t* vp = (const bf16_t*)a.v_plane;
-    const int* bt = a.block_table + (size_t)req * a.bt_stride;
     const int page = a.page;
+    // The block-table entries of the keys this work-group reads go to shared memory first: a
+    // page lookup in the loop is then a shared-memory read instead of a memory access that the
+    // key and value loads would have to wait for (two memory latencies in a row per chunk).
+    __shared__ int bt_s[ATM_BT_MAX];
+    const int* bt_g = a.block_table + (size_t)req * a.bt_stride;
+    const int blk0 = (ch_begin * 32) / page;
+    const int blk_n = ch_begin < ch_end ? (min(ch_end * 32, key_hi) - 1) / page - blk0 + 1 : 0;
+    const bool bt_local = blk_n <= ATM_BT_MAX;
+    if (bt_local) {
+        for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
+        __syncthreads();
+    }
+#define ATM_PAGE_OF(blk) (bt_local ? bt_s[(blk) - blk0] : bt_g[(blk)])
     const float scale2 = a.scale * 1.44269504088896341f;
     // smallest query position and largest window start over the rows of the tile (uniform)
     const int tile_pos_min = ctx + tok0;
@@ -290,9 +316,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
     {                                                                                                        \
         const int kb_ = (chunk) * 32;                                                                        \
         _Pragma("unroll") for (int hf = 0; hf < 2; ++hf) {                                                   \
-            const int key = min(kb_ + 16 * hf + li, key_hi - 1);                                             \
-            const int pg = bt[key / page];                                                                   \
-            const bf16_t* krow = kp + (((size_t)pg * a.kv_heads + kvh) * page + (key % page)) * AT_HD;       \
+            int blk, off;                                                                                    \
+            split_key(min(kb_ + 16 * hf + li, key_hi - 1), page, a.page_shift, blk, off);                    \
+            const bf16_t* krow = kp + ((size_t)ATM_PAGE_OF(blk) * kv_stride + kvh_off + off * AT_HD);        \
             _Pragma("unroll") for (int c = 0; c < ATM_DC; ++c) {                                             \
                 const int d = 32 * c + 8 * g;                                                                \
                 KF[hf][c].u = (d + 8 <= AT_HD) ? *(const uint4*)(krow + d) : make_uint4(0, 0, 0, 0);         \
@@ -300,15 +326,19 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
         }                                                                                                    \
         const int ka = kb_ + 4 * g, kb = kb_ + 16 + 4 * g;                                                   \
         const bool oka = ka < key_hi, okb = kb < key_hi;                                                     \
-        const int pga = oka ? bt[ka / page] : 0, pgb = okb ? bt[kb / page] : 0;                              \
-        const bf16_t* va = vp + ((size_t)pga * a.kv_heads + kvh) * AT_HD * page + (ka % page);               \
-        const bf16_t* vb = vp + ((size_t)pgb * a.kv_heads + kvh) * AT_HD * page + (kb % page);               \
+        int blka, offa, blkb, offb;                                                                          \
+        split_key(ka, page, a.page_shift, blka, offa);                                                       \
+        split_key(kb, page, a.page_shift, blkb, offb);                                                       \
+        const bf16_t* va = vp + ((size_t)(oka ? ATM_PAGE_OF(blka) : 0) * kv_stride + kvh_off + offa + li * page); \
+        const bf16_t* vb = vp + ((size_t)(okb ? ATM_PAGE_OF(blkb) : 0) * kv_stride + kvh_off + offb + li * page); \
         _Pragma("unroll") for (int t = 0; t < ATM_DT; ++t) {                                                 \
-            const size_t drow = (size_t)(16 * t + li) * page;                                                \
-            VA[t] = oka ? *(const uint2*)(va + drow) : make_uint2(0, 0);                                     \
-            VB[t] = okb ? *(const uint2*)(vb + drow) : make_uint2(0, 0);                                     \
+            VA[t] = oka ? *(const uint2*)(va + 16 * t * page) : make_uint2(0, 0);                            \
+            VB[t] = okb ? *(const uint2*)(vb + 16 * t * page) : make_uint2(0, 0);                            \
         }                                                                                                    \
     }
+
+    const size_t kv_stride = (size_t)a.kv_heads * page * AT_HD;     /* elements per page, all KV heads */
+    const int kvh_off = kvh * page * AT_HD;
 
     int ch = ch_begin + wave;
     if (ch < ch_end) ATM_FETCH(kf, vfa, vfb, ch)
@@ -377,6 +407,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
         if (ch + 4 < ch_end) ATM_FETCH(kf, vfa, vfb, ch + 4)
     }
 #undef ATM_FETCH
+#undef ATM_PAGE_OF
 
     // ---- merge the four waves: 2,3 -> 0,1, then 1 -> 0
 #pragma unroll
@@ -429,6 +460,242 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
         }
     }
 }
+
+// =====================================================================================
+// Prompt portions on the matrix cores: 64 rows per work-group, keys and values through
+// shared memory.
+//
+// The kernel above lets every wave fetch its own keys, which is right when the waves of a
+// work-group split the keys of one 16-row tile among themselves (decode).  For a prompt
+// portion there are many row tiles over the same keys: here the four waves of a work-group
+// each own one 16-row tile (64 rows: consecutive tokens x the heads of one KV group), fetch
+// every 32-key chunk once, together, into shared memory (two buffers; the next chunk is on
+// its way from memory while the current one is multiplied), and read their operands from
+// there.  The arithmetic per wave is the same as above (transposed products, base-2 online
+// softmax in float).  A wave skips the chunks that lie beyond all of its rows.
+// Built for head sizes up to 128.
+#if AT_HD <= 128
+#define ATP_KROW (AT_HD + 8)          // bfloat16 elements between key rows in shared memory
+#define ATP_VROW 36                   // between value rows (32 keys + 4 of padding)
+#define ATP_KPIECES (32 * AT_HD / 8)  // 16-byte pieces of a key chunk
+#define ATP_VPIECES (AT_HD * 8)       // 8-byte pieces (4 keys of one d) of a value chunk
+#define ATP_KPT ((ATP_KPIECES + 255) / 256)
+#define ATP_VPT ((ATP_VPIECES + 255) / 256)
+
+__global__ __launch_bounds__(256) void paged_attention_prefill_kernel(AttnArgs a) {
+    __shared__ __attribute__((aligned(16))) bf16_t ks[2][32 * ATP_KROW];
+    __shared__ __attribute__((aligned(16))) bf16_t vs[2][AT_HD * ATP_VROW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, g = lane >> 4;
+
+    // later tiles of a prompt see more keys: start them first, so that the short ones fill the end
+    const int tile = gridDim.x - 1 - blockIdx.x;
+    const int group = a.heads / a.kv_heads;
+    const int chunks_h = (group + a.gcap - 1) / a.gcap;
+    const int kvh = blockIdx.y / chunks_h;
+    const int g0 = (blockIdx.y % chunks_h) * a.gcap;
+    const int gcount = min(a.gcap, group - g0);
+
+    const int req = a.tile_req[tile];
+    const int tok0 = a.tile_tok0[tile];
+    const int first = a.req_indptr[req];
+    const int n_new = a.req_indptr[req + 1] - first;
+    const int ctx = a.ctx_lens[req];
+    const int ntok = min(a.tq, n_new - tok0);           // a.tq: tokens of a 64-row tile
+
+    const int row = wave * 16 + li;                      // my row among the 64
+    const int r_tok = row / a.gcap, r_g = row % a.gcap;
+    const bool row_ok = r_tok < ntok && r_g < gcount;
+    const int r_pos = ctx + tok0 + r_tok;
+    const int r_lo = a.window > 0 ? r_pos - a.window + 1 : 0;
+    const int r_head = kvh * group + g0 + r_g;
+    const int r_token = first + tok0 + r_tok;
+    // positions of my wave's rows (uniform per wave)
+    const int w_tok_lo = min((wave * 16) / a.gcap, ntok - 1), w_tok_hi = min((wave * 16 + 15) / a.gcap, ntok - 1);
+    const int w_pos_min = ctx + tok0 + w_tok_lo, w_pos_max = ctx + tok0 + w_tok_hi;
+    const int w_lo_max = a.window > 0 ? max(0, w_pos_max - a.window + 1) : 0;
+    const int w_lo_min = a.window > 0 ? max(0, w_pos_min - a.window + 1) : 0;
+    const bool wave_has_rows = (wave * 16) / a.gcap < ntok;
+
+    FragK qf[ATM_DC];
+    {
+        const bf16_t* q = (const bf16_t*)a.q + (size_t)r_token * a.q_stride + (size_t)r_head * AT_HD;
+#pragma unroll
+        for (int c = 0; c < ATM_DC; ++c) {
+            const int d = 32 * c + 8 * g;
+            qf[c].u = (row_ok && d + 8 <= AT_HD) ? *(const uint4*)(q + d) : make_uint4(0, 0, 0, 0);
+        }
+    }
+
+    const int key_hi = ctx + tok0 + ntok;
+    const int key_lo = a.window > 0 ? max(0, ctx + tok0 - a.window + 1) : 0;
+    const int ch_begin = key_lo / 32, ch_end = (key_hi + 31) / 32;
+
+    const bf16_t* kp = (const bf16_t*)a.k_plane;
+    const bf16_t* vp = (const bf16_t*)a.v_plane;
+    const int page = a.page;
+    const float scale2 = a.scale * 1.44269504088896341f;
+    // block-table entries of the tile's keys, in shared memory (see the kernel above)
+    __shared__ int bt_s[ATM_BT_MAX];
+    const int* bt_g = a.block_table + (size_t)req * a.bt_stride;
+    const int blk0 = (ch_begin * 32) / page;
+    const int blk_n = ch_begin < ch_end ? (key_hi - 1) / page - blk0 + 1 : 0;
+    const bool bt_local = blk_n <= ATM_BT_MAX;
+    if (bt_local) {
+        for (int i = tid; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
+        __syncthreads();
+    }
+#define ATP_PAGE_OF(blk) (bt_local ? bt_s[(blk) - blk0] : bt_g[(blk)])
+
+    // two register stages: chunk c+1 (fetched during the previous iteration) and chunk c+2
+    uint4 kst[ATP_KPT], kst2[ATP_KPT];
+    uint2 vst[ATP_VPT], vst2[ATP_VPT];
+    // which pieces of a chunk this thread fetches does not change from chunk to chunk
+    int kj[ATP_KPT], kpc[ATP_KPT], vd[ATP_VPT], vq[ATP_VPT];
+#pragma unroll
+    for (int i = 0; i < ATP_KPT; ++i) { const int idx = tid + 256 * i; kj[i] = idx / (AT_HD / 8); kpc[i] = (idx % (AT_HD / 8)) * 8; }
+#pragma unroll
+    for (int i = 0; i < ATP_VPT; ++i) { const int idx = tid + 256 * i; vd[i] = idx / 8; vq[i] = (idx % 8) * 4; }
+    const size_t kv_stride = (size_t)a.kv_heads * page * AT_HD;     // elements per page, all KV heads
+    const int kvh_off = kvh * page * AT_HD;
+#define ATP_FETCH(KS_, VS_, chunk)                                                                         \
+    {                                                                                                      \
+        const int kb_ = (chunk) * 32;                                                                      \
+        _Pragma("unroll") for (int i = 0; i < ATP_KPT; ++i) {                                              \
+            KS_[i] = make_uint4(0, 0, 0, 0);                                                               \
+            if (tid + 256 * i < ATP_KPIECES) {                                                             \
+                int blk, off;                                                                              \
+                split_key(min(kb_ + kj[i], key_hi - 1), page, a.page_shift, blk, off);                     \
+                KS_[i] = *(const uint4*)(kp + ((size_t)ATP_PAGE_OF(blk) * kv_stride + kvh_off + off * AT_HD + kpc[i])); \
+            }                                                                                              \
+        }                                                                                                  \
+        _Pragma("unroll") for (int i = 0; i < ATP_VPT; ++i) {                                              \
+            const int key4 = kb_ + vq[i];                                                                  \
+            VS_[i] = make_uint2(0, 0);                                                                     \
+            if (tid + 256 * i < ATP_VPIECES && key4 < key_hi) {                                            \
+                int blk, off;                                                                              \
+                split_key(key4, page, a.page_shift, blk, off);                                             \
+                VS_[i] = *(const uint2*)(vp + ((size_t)ATP_PAGE_OF(blk) * kv_stride + kvh_off + vd[i] * page + off)); \
+            }                                                                                              \
+        }                                                                                                  \
+    }
+#define ATP_PARK(KS_, VS_, buf)                                                                            \
+    {                                                                                                      \
+        _Pragma("unroll") for (int i = 0; i < ATP_KPT; ++i) {                                              \
+            const int idx = tid + 256 * i;                                                                 \
+            if (idx < ATP_KPIECES) *(uint4*)(&ks[buf][(idx / (AT_HD / 8)) * ATP_KROW + (idx % (AT_HD / 8)) * 8]) = KS_[i]; \
+        }                                                                                                  \
+        _Pragma("unroll") for (int i = 0; i < ATP_VPT; ++i) {                                              \
+            const int idx = tid + 256 * i;                                                                 \
+            if (idx < ATP_VPIECES) *(uint2*)(&vs[buf][(idx / 8) * ATP_VROW + (idx % 8) * 4]) = VS_[i];     \
+        }                                                                                                  \
+    }
+
+    float m = -INFINITY, l = 0.f;
+    f32x4_t acc[ATM_DT];
+#pragma unroll
+    for (int t = 0; t < ATM_DT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // Pipeline: while chunk c is multiplied out of shared memory, chunk c+1 sits in registers
+    // (fetched one iteration ago, parked at the end of this one) and chunk c+2 is being fetched:
+    // a fetch has two iterations to arrive.
+    if (ch_begin < ch_end) {
+        ATP_FETCH(kst, vst, ch_begin)
+        ATP_PARK(kst, vst, 0)
+    }
+    if (ch_begin + 1 < ch_end) ATP_FETCH(kst, vst, ch_begin + 1)
+    __syncthreads();
+    for (int ch = ch_begin; ch < ch_end; ++ch) {
+        const int cur = (ch - ch_begin) & 1;
+        const int kbase = ch * 32;
+        if (ch + 2 < ch_end) ATP_FETCH(kst2, vst2, ch + 2)
+        if (wave_has_rows && kbase <= w_pos_max && kbase + 31 >= w_lo_min) {
+            f32x4_t sc[2];
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                f32x4_t sacc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < ATM_DC; ++c) {
+                    const int d = 32 * c + 8 * g;
+                    FragK kf;
+                    kf.u = (d + 8 <= AT_HD) ? *(const uint4*)(&ks[cur][(16 * hf + li) * ATP_KROW + d]) : make_uint4(0, 0, 0, 0);
+                    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sacc, 0, 0, 0);
+                }
+                sc[hf] = sacc;
+            }
+            float s[8];
+            float mloc = -INFINITY;
+            if (kbase + 31 <= w_pos_min && kbase >= w_lo_max) {
+#pragma unroll
+                for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float x = sc[hf][v] * scale2;
+                        s[4 * hf + v] = x;
+                        mloc = fmaxf(mloc, x);
+                    }
+            } else {
+#pragma unroll
+                for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int key = kbase + 16 * hf + 4 * g + v;
+                        const bool seen = row_ok && key <= r_pos && key >= r_lo;
+                        const float x = seen ? sc[hf][v] * scale2 : -INFINITY;
+                        s[4 * hf + v] = x;
+                        mloc = fmaxf(mloc, x);
+                    }
+            }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, TL_WAVE));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TL_WAVE));
+            const float m_new = fmaxf(m, mloc);
+            const float alpha = (m == -INFINITY) ? 0.f : fast_exp2(m - m_new);
+            FragK pf;
+            float psum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p = (s[i] == -INFINITY) ? 0.f : fast_exp2(s[i] - m_new);
+                psum += p;
+                pf.v[i] = (__bf16)p;
+            }
+            l = l * alpha + psum;
+            const bool moved = __any(m_new != m);
+            m = m_new;
+#pragma unroll
+            for (int t = 0; t < ATM_DT; ++t) {
+                FragK vf;
+                vf.h[0] = *(const uint2*)(&vs[cur][(16 * t + li) * ATP_VROW + 4 * g]);
+                vf.h[1] = *(const uint2*)(&vs[cur][(16 * t + li) * ATP_VROW + 16 + 4 * g]);
+                if (moved) acc[t] *= alpha;
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[t], 0, 0, 0);
+            }
+        }
+        if (ch + 1 < ch_end) ATP_PARK(kst, vst, cur ^ 1)
+#pragma unroll
+        for (int i = 0; i < ATP_KPT; ++i) kst[i] = kst2[i];
+#pragma unroll
+        for (int i = 0; i < ATP_VPT; ++i) vst[i] = vst2[i];
+        // A barrier that waits for this wave's shared-memory traffic only: __syncthreads() would
+        // also wait for the fetch of chunk c+2, which is meant to stay in flight across it.
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+#undef ATP_FETCH
+#undef ATP_PARK
+#undef ATP_PAGE_OF
+    l += __shfl_xor(l, 16, TL_WAVE);
+    l += __shfl_xor(l, 32, TL_WAVE);
+    if (!row_ok) return;
+    bf16_t* o = (bf16_t*)a.out + (size_t)r_token * a.heads * AT_HD + (size_t)r_head * AT_HD;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int t = 0; t < ATM_DT; ++t) {
+        union { uint2 u; uint16_t e[4]; } pk;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(acc[t][v] * inv).bits;
+        *(uint2*)(o + 16 * t + 4 * g) = pk.u;
+    }
+}
+#endif
 
 // out[row] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s over the parts of a row.
 // The parts are read eight at a time with all loads issued before the first use.
@@ -492,6 +759,7 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
     a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
     a.q_stride = q_stride; a.bt_stride = bt_stride; a.heads = heads; a.kv_heads = kv_heads; a.page = page;
     a.window = window; a.tq = tq; a.gcap = gcap; a.splits = splits; a.scale = scale;
+    a.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz(page) : -1;
     const int chunks = (group + gcap - 1) / gcap;
     dim3 grid(tiles, kv_heads * chunks, splits), block(256);
     const bool aligned = ((uintptr_t)q % 16) == 0 && q_stride % 8 == 0 && ((uintptr_t)out % 8) == 0 &&
@@ -508,4 +776,40 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
         TL_CHECK_LAUNCH("attention_merge");
     }
     return TL_OK;
+}
+
+// Rows of a prompt-portion tile: a.tq tokens x gcap heads must fit 64.
+#define ATP_ROWS 64
+
+// The prompt-portion kernel (bfloat16, head sizes up to 128, pages of a multiple of 4 tokens):
+// tiles of `tq` tokens with tq * min(group, 16) <= 64.  Returns an error where it is not built;
+// callers fall back to tl_paged_attention, which takes every case.
+extern "C" int tl_paged_attention_prefill(const void* q, int q_stride, void* out, const void* k_plane, const void* v_plane,
+                                          const void* block_table, int bt_stride, const void* req_indptr, const void* ctx_lens,
+                                          const void* tile_req, const void* tile_tok0, int tiles, int tq,
+                                          int heads, int kv_heads, int page, int window, float scale, hipStream_t stream) {
+#if AT_HD <= 128
+    TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
+    TL_REQUIRE(page > 0 && page % 4 == 0 && bt_stride > 0 && tq > 0 && window >= 0, "attention_prefill: bad page/table/tile sizes");
+    const int group = heads / kv_heads;
+    const int gcap = group < AT_ROWS ? group : AT_ROWS;
+    TL_REQUIRE(tq * gcap <= ATP_ROWS, "attention_prefill: tile of %d tokens x %d heads exceeds %d rows", tq, gcap, ATP_ROWS);
+    TL_REQUIRE(q_stride >= heads * AT_HD && q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0 &&
+               ((uintptr_t)k_plane % 16) == 0 && ((uintptr_t)v_plane % 8) == 0, "attention_prefill: operands not aligned");
+    if (tiles == 0) return TL_OK;
+    AttnArgs a;
+    a.q = q; a.out = out; a.k_plane = k_plane; a.v_plane = v_plane;
+    a.block_table = (const int*)block_table; a.req_indptr = (const int*)req_indptr; a.ctx_lens = (const int*)ctx_lens;
+    a.tile_req = (const int*)tile_req; a.tile_tok0 = (const int*)tile_tok0;
+    a.part_o = nullptr; a.part_ml = nullptr;
+    a.q_stride = q_stride; a.bt_stride = bt_stride; a.heads = heads; a.kv_heads = kv_heads; a.page = page;
+    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = 1; a.scale = scale;
+    a.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz(page) : -1;
+    const int chunks = (group + gcap - 1) / gcap;
+    paged_attention_prefill_kernel<<<dim3(tiles, kv_heads * chunks), dim3(256), 0, stream>>>(a);
+    TL_CHECK_LAUNCH("paged_attention_prefill");
+    return TL_OK;
+#else
+    TL_REQUIRE(false, "attention_prefill: built for head sizes up to 128, this library is for %d", AT_HD);
+#endif
 }

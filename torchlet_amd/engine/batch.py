@@ -80,9 +80,12 @@ class StepContext:
         for tq, n in host_tiles.items():
             self._tiles[tq] = (views[f"tile_req{tq}"], views[f"tile_tok0{tq}"], n)
 
-    def _build_tiles(self, tq: int):
-        """Tiles of up to ``tq`` consecutive new tokens of one request."""
+    def _build_tiles(self, tq: int, select=None):
+        """Tiles of up to ``tq`` consecutive new tokens of one request (of the requests where
+        ``select`` is true, if given)."""
         counts = -(-self._host_new_lens // tq)
+        if select is not None:
+            counts = np.where(select, counts, 0)
         tile_req = np.repeat(np.arange(self.num_requests, dtype=np.int32), counts)
         first = np.zeros(self.num_requests + 1, dtype=np.int64)
         np.cumsum(counts, out=first[1:])
@@ -108,6 +111,19 @@ class StepContext:
             tr, t0 = self._build_tiles(tq)
             v = self._upload({"r": tr, "t": t0})
             t = self._tiles[tq] = (v["r"], v["t"], len(tr))
+        return t
+
+    def tiles_by_length(self, tq_short: int, tq_long: int, threshold: int):
+        """Two tile lists: requests that bring fewer than ``threshold`` tokens in tiles of
+        ``tq_short`` tokens, the others in tiles of ``tq_long``."""
+        key = (tq_short, tq_long, threshold)
+        t = self._tiles.get(key)
+        if t is None:
+            long = self._host_new_lens >= threshold
+            sr, s0 = self._build_tiles(tq_short, ~long)
+            lr, l0 = self._build_tiles(tq_long, long)
+            v = self._upload({"sr": sr, "s0": s0, "lr": lr, "l0": l0})
+            t = self._tiles[key] = ((v["sr"], v["s0"], len(sr)), (v["lr"], v["l0"], len(lr)))
         return t
 
 

@@ -286,6 +286,42 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
                                        c_int(_dt(q, "paged_attention")), c_int(1 if general else 0), _stream()))
 
 
+PREFILL_ATTENTION_ROWS = 64      # rows a work-group of the prompt-portion kernel owns
+PREFILL_ATTENTION_MAX_HEAD_DIM = 128
+
+
+def prefill_attention_tile_tokens(num_heads: int, num_kv_heads: int) -> int:
+    group = num_heads // num_kv_heads
+    return max(1, PREFILL_ATTENTION_ROWS // min(group, ATTENTION_ROWS))
+
+
+def paged_attention_prefill(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v_plane: torch.Tensor,
+                            block_table: torch.Tensor, req_indptr: torch.Tensor, ctx_lens: torch.Tensor,
+                            tile_req: torch.Tensor, tile_tok0: torch.Tensor, num_tiles: int, tile_tokens: int,
+                            num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
+                            scale: float) -> None:
+    """The attention of :func:`paged_attention` for prompt portions: bfloat16, head sizes up
+    to 128, pages of a multiple of 4 tokens; tiles of ``tile_tokens`` tokens (64 rows) whose keys
+    and values pass through shared memory once per work-group.  Writes the rows of its tiles only."""
+    T = q.shape[0]
+    if q.dtype != torch.bfloat16 or head_dim > PREFILL_ATTENTION_MAX_HEAD_DIM or page_size % 4:
+        raise KernelError("paged_attention_prefill: bfloat16, head sizes up to 128 and pages of a multiple of 4 tokens only")
+    if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelError("paged_attention_prefill: q/out shapes or dtypes do not fit")
+    _check_planes("paged_attention_prefill", k_plane, v_plane, q.dtype, num_kv_heads, page_size, head_dim)
+    for name, t in (("block_table", block_table), ("req_indptr", req_indptr), ("ctx_lens", ctx_lens),
+                    ("tile_req", tile_req), ("tile_tok0", tile_tok0)):
+        _i32(t, name)
+    if tile_req.numel() < num_tiles or tile_tok0.numel() < num_tiles:
+        raise KernelError("paged_attention_prefill: tile arrays shorter than the number of tiles")
+    lib = _lib(f"attention_hd{head_dim}")
+    _check(lib, lib.tl_paged_attention_prefill(_ptr(q), c_int(q.stride(0)), _ptr(out), _ptr(k_plane), _ptr(v_plane),
+                                               _ptr(block_table), c_int(block_table.stride(0)), _ptr(req_indptr),
+                                               _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles),
+                                               c_int(tile_tokens), c_int(num_heads), c_int(num_kv_heads), c_int(page_size),
+                                               c_int(window), c_float(scale), _stream()))
+
+
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     """``out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]``."""
     T, I2 = gate_up.shape

@@ -21,6 +21,9 @@ from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedNeed, WeightSpec
 
 _TARGET_WORKGROUPS = 512     # enough work-groups to fill 256 compute units twice
 _MIN_KEYS_PER_SPLIT = 256
+_PORTION_MIN_TOKENS = 16     # requests that bring at least this many tokens go to the prompt-portion kernel ...
+_PORTION_MIN_CONTEXT = 4096  # ... in steps whose longest sequence has at least this many tokens (measured on
+                             # MI355X: the shared-memory kernel wins from about 4k keys on, 13 % at 8k)
 
 
 @MIXERS.register("gqa_attention")
@@ -46,6 +49,7 @@ class GQAttention(Mixer):
         self.qkv_bias = spec.qkv_bias
         self.position = POSITION_ENCODINGS.build(spec.position, dtype, device) if spec.position is not None else None
         self.tile_tokens = ops.attention_tile_tokens(self.heads, self.kv_heads)
+        self.portion_tile_tokens = ops.prefill_attention_tile_tokens(self.heads, self.kv_heads)
         self.w_qkv: torch.Tensor | None = None
         self.b_qkv: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
@@ -115,12 +119,25 @@ class GQAttention(Mixer):
                 ctx.token_req if writes else None, table if writes else None,
                 k_plane if writes else None, v_plane if writes else None, cache.page_size if writes else 0)
 
-        tile_req, tile_tok0, tiles = ctx.tiles(self.tile_tokens)
         out = torch.empty((T, self.q_width), dtype=self.dtype, device=h.device)
-        ops.paged_attention(
-            qkv[:, : self.q_width], out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
-            tile_req, tile_tok0, tiles, self.tile_tokens, self.heads, self.kv_heads, self.head_dim,
-            cache.page_size, self.window or 0, self.scale, self._splits(ctx, tiles))
+        q = qkv[:, : self.q_width]
+        common = (self.heads, self.kv_heads, self.head_dim, cache.page_size, self.window or 0, self.scale)
+        portions = (self.dtype == torch.bfloat16 and self.head_dim <= ops.PREFILL_ATTENTION_MAX_HEAD_DIM
+                    and cache.page_size % 4 == 0 and ctx.max_new_tokens >= _PORTION_MIN_TOKENS
+                    and ctx.max_total_len >= _PORTION_MIN_CONTEXT)
+        if portions:
+            # prompt portions: 64-row tiles with keys and values through shared memory; the other
+            # requests of the step (decode tokens, short portions): 16-row tiles, keys split over waves
+            short, long = ctx.tiles_by_length(self.tile_tokens, self.portion_tile_tokens, _PORTION_MIN_TOKENS)
+            ops.paged_attention_prefill(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
+                                        long[0], long[1], long[2], self.portion_tile_tokens, *common)
+            if short[2]:     # one split: the merge of several would run over the rows of the long requests too
+                ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
+                                    short[0], short[1], short[2], self.tile_tokens, *common, 1)
+        else:
+            tile_req, tile_tok0, tiles = ctx.tiles(self.tile_tokens)
+            ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
+                                tile_req, tile_tok0, tiles, self.tile_tokens, *common, self._splits(ctx, tiles))
         y = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
         ops.linear(out, self.w_o, None, y)
         return y

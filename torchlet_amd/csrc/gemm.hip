@@ -120,23 +120,43 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + 
 // SW (gate/up product with the SwiGLU gate applied to the accumulators): w holds blocks of 64
 // rows, 32 gate rows followed by the 32 up rows of the same columns; needs R == 4, so that a
 // work-group's strips are [gate 0-15, gate 16-31, up 0-15, up 16-31]; out has N / 2 columns.
-template <int R, int MT, int KS, typename TOut, bool SW = false>
+// XL (x through shared memory): with more than one activation row the 16 lanes of a group read
+// 16 different rows of x, which no longer fit the L1 cache once M * K * 2 bytes exceed it, and
+// every operand load of x becomes a trip to L2 that competes with the weight stream (measured:
+// 5.6 TB/s at M = 1, 4.6 at M = 8, 3.7 at M = 16 without it).  With XL the work-group copies
+// its M rows of x into shared memory once, coalesced, and reads the operands from there.
+template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false>
 __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                               const void* __restrict__ bias, int bias_f32,
                                                               TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
                                                               int out_cols = 0) {
     static_assert(!SW || (R == 4 && KS > 1), "the fused gate needs four strips per work-group");
-    __shared__ float red[KS > 1 ? KS * R * MT * 256 : 1];
+    extern __shared__ __attribute__((aligned(16))) float skinny_lds[];
+    float* red = skinny_lds;                                             // KS * R * MT * 256 floats
+    bf16_t* xs = (bf16_t*)(skinny_lds + KS * R * MT * 256);             // XL: M rows of K + 8 elements
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
     const int n0 = blockIdx.x * (16 * R);
 
     const bf16_t* wrow[R];
     const bf16_t* xrow[MT];
+    int xoff[MT];
 #pragma unroll
     for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + li, N - 1) * K;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) xrow[t] = x + (size_t)min(t * 16 + li, M - 1) * ldx;
+    for (int t = 0; t < MT; ++t) {
+        xrow[t] = x + (size_t)min(t * 16 + li, M - 1) * ldx;
+        xoff[t] = min(t * 16 + li, M - 1) * (K + 8);
+    }
+    if (XL) {
+        const int pieces = K / 8;                     // 16-byte pieces per row
+        for (int i = threadIdx.x; i < M * pieces; i += KS * 64) {
+            const int row = i / pieces, pc = i % pieces;
+            *(uint4*)(&xs[row * (K + 8) + pc * 8]) = *(const uint4*)(x + (size_t)row * ldx + pc * 8);
+        }
+        __syncthreads();
+    }
+#define SK_LOADB(t, k) (XL ? *(const uint4*)(&xs[xoff[t] + (k)]) : *(const uint4*)(xrow[t] + (k)))
 
     f32x4_t acc[R][MT];
 #pragma unroll
@@ -152,7 +172,7 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
 #pragma unroll
         for (int r = 0; r < R; ++r) { a0[r].u = SK_LOAD(wrow[r] + k); a1[r].u = SK_LOAD(wrow[r] + k + SK_SECOND); }
 #pragma unroll
-        for (int t = 0; t < MT; ++t) { b0[t].u = *(const uint4*)(xrow[t] + k); b1[t].u = *(const uint4*)(xrow[t] + k + SK_SECOND); }
+        for (int t = 0; t < MT; ++t) { b0[t].u = SK_LOADB(t, k); b1[t].u = SK_LOADB(t, k + SK_SECOND); }
     }
     for (; s < full; s += KS) {
         // fetch the next step (the last one fetches itself again: no branch in the loop)
@@ -162,7 +182,7 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
 #pragma unroll
         for (int r = 0; r < R; ++r) { na0[r].u = SK_LOAD(wrow[r] + kn); na1[r].u = SK_LOAD(wrow[r] + kn + SK_SECOND); }
 #pragma unroll
-        for (int t = 0; t < MT; ++t) { nb0[t].u = *(const uint4*)(xrow[t] + kn); nb1[t].u = *(const uint4*)(xrow[t] + kn + SK_SECOND); }
+        for (int t = 0; t < MT; ++t) { nb0[t].u = SK_LOADB(t, kn); nb1[t].u = SK_LOADB(t, kn + SK_SECOND); }
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -187,8 +207,8 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
         }
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-            b0[t].u = v0 ? *(const uint4*)(xrow[t] + k) : zero;
-            b1[t].u = v1 ? *(const uint4*)(xrow[t] + k + SK_SECOND) : zero;
+            b0[t].u = v0 ? SK_LOADB(t, k) : zero;
+            b1[t].u = v1 ? SK_LOADB(t, k + SK_SECOND) : zero;
         }
 #pragma unroll
         for (int r = 0; r < R; ++r)
@@ -259,14 +279,173 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
     }
 }
 
+// Shared memory beyond 64 KB has to be allowed per kernel, once per process.
+template <typename Kernel>
+static hipError_t allow_lds(Kernel kernel, size_t bytes) {
+    if (bytes <= 65536) return hipSuccess;
+    return hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+#define SKINNY_XL_MAX_BYTES (60 * 1024)      // x may take this much shared memory: with the reduction buffer two
+                                             // work-groups still fit the 160 KB of a compute unit
+
+template <int R, int MT, int KS, typename TOut, bool SW>
+static void launch_skinny_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                            int ldx, int ldo, int out_cols, hipStream_t stream) {
+    dim3 grid((N + 16 * R - 1) / (16 * R)), block(KS * 64);
+    const size_t red_bytes = (size_t)KS * R * MT * 1024;
+    const size_t x_bytes = (size_t)M * (K + 8) * 2;
+    // (not with few waves per work-group: the copy of x then takes longer than it saves; measured on the
+    // fused gate/up kernel, 87 us with against 64 us without at M = 8)
+    if (M > 1 && KS >= 8 && x_bytes <= SKINNY_XL_MAX_BYTES) {
+        auto kernel = gemm_skinny_kernel<R, MT, KS, TOut, SW, true>;
+        static hipError_t allowed = allow_lds(kernel, 96 * 1024);
+        if (allowed == hipSuccess) {
+            kernel<<<grid, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols);
+            return;
+        }
+    }
+    gemm_skinny_kernel<R, MT, KS, TOut, SW, false><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols);
+}
+
 template <int R, int MT, int KS>
 static void launch_skinny(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                           int ldx, int ldo, int out_f32, hipStream_t stream) {
-    dim3 grid((N + 16 * R - 1) / (16 * R)), block(KS * 64);
-    if (out_f32)
-        gemm_skinny_kernel<R, MT, KS, float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo);
-    else
-        gemm_skinny_kernel<R, MT, KS, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo);
+    if (out_f32) launch_skinny_t<R, MT, KS, float, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
+    else launch_skinny_t<R, MT, KS, bf16_t, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
+}
+
+// =====================================================================================
+// The same product for up to 16 rows against a matrix with many strips (gate/up, LM head):
+// one work-group per compute unit that walks a range of strips.
+//
+// Every wave keeps its share of x (the K steps s = wave, wave + KS, ...) in registers for the
+// whole kernel, so after the first strip only weights are read; the weights of strip i + 1
+// are fetched while strip i is multiplied, reduced and stored, and the reduction of a strip
+// (through shared memory, two buffers) is done by one wave in turn while the others go on:
+// the weight stream never stops for a strip's epilogue.  Needs K <= 64 * KS * DS.
+// SW: the matrix is the interleaved gate/up matrix (see gemm_skinny_kernel); a work item is a
+// (gate strip, up strip) pair, processed as two strips whose sums the same wave combines.
+__device__ __forceinline__ void lds_barrier() {
+    // waits for this wave's shared-memory traffic only: weight fetches stay in flight across it
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <int KS, int DS, typename TOut, bool SW>
+__global__ __launch_bounds__(KS * 64) void gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                              const void* __restrict__ bias, int bias_f32,
+                                                              TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
+                                                              int out_cols, int items, int items_per_group) {
+    __shared__ float red[2][KS * 256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int li = lane & 15, lg = lane >> 4;
+
+    // my K steps and which 8-element pieces of them lie inside K
+    int koff[DS];
+    bool v0[DS], v1[DS];
+    Frag16 xb0[DS], xb1[DS];
+    const bf16_t* xrow = x + (size_t)min(li, M - 1) * ldx;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int d = 0; d < DS; ++d) {
+        koff[d] = 64 * (wave + d * KS) + 16 * lg;
+        v0[d] = koff[d] + 8 <= K;
+        v1[d] = koff[d] + 16 <= K;
+        xb0[d].u = v0[d] ? *(const uint4*)(xrow + koff[d]) : zero;
+        xb1[d].u = v1[d] ? *(const uint4*)(xrow + koff[d] + 8) : zero;
+    }
+
+    const int first = blockIdx.x * items_per_group;
+    const int last = min(first + items_per_group, items);
+    // first weight row of a work item's strip
+    auto strip_row = [&](int item) -> int {
+        if (!SW) return 16 * item;
+        const int pair = item >> 1, sub = item & 1;
+        return 16 * (4 * (pair >> 1) + (pair & 1) + 2 * sub);
+    };
+    Frag16 a0[DS], a1[DS], n0[DS], n1[DS];
+#define ST_FETCH(A0, A1, item)                                                                  \
+    {                                                                                           \
+        const bf16_t* wr = w + (size_t)min(strip_row(item) + li, N - 1) * K;                    \
+        _Pragma("unroll") for (int d = 0; d < DS; ++d) {                                        \
+            A0[d].u = v0[d] ? *(const uint4*)(wr + koff[d]) : zero;                             \
+            A1[d].u = v1[d] ? *(const uint4*)(wr + koff[d] + 8) : zero;                         \
+        }                                                                                       \
+    }
+    if (first < last) ST_FETCH(a0, a1, first)
+    f32x4_t gate_sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int item = first; item < last; ++item) {
+        if (item + 1 < last) ST_FETCH(n0, n1, item + 1)
+        f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int d = 0; d < DS; ++d) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[d].v, xb0[d].v, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[d].v, xb1[d].v, acc, 0, 0, 0);
+        }
+        const int buf = (item - first) & 1;
+        *(f32x4_t*)(&red[buf][(wave * 64 + lane) * 4]) = acc;
+        lds_barrier();
+        const int unit = SW ? (item >> 1) : item;
+        if (wave == unit % KS) {
+            f32x4_t sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int wv = 0; wv < KS; ++wv) sum += *(const f32x4_t*)(&red[buf][(wv * 64 + lane) * 4]);
+            // D[i][j]: i = 4 * lg + v (weight row of the strip), j = li (activation row)
+            if (SW) {
+                if ((item & 1) == 0) {
+                    gate_sum = sum;
+                } else if (li < M) {
+                    const int col = 16 * unit + 4 * lg;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (col + v < out_cols) out[(size_t)li * ldo + col + v] = from_float<TOut>(silu_mul(gate_sum[v], sum[v]));
+                }
+            } else if (li < M) {
+                const int n = 16 * item + 4 * lg;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (n + v < N) {
+                        float val = sum[v];
+                        if (bias) val += load_vec(bias, bias_f32, n + v);
+                        out[(size_t)li * ldo + n + v] = from_float<TOut>(val);
+                    }
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < DS; ++d) { a0[d] = n0[d]; a1[d] = n1[d]; }
+    }
+#undef ST_FETCH
+}
+
+// Launches gemm_stream_kernel if the shape fits it (M <= 16, K <= 4096, at least 1024 strips);
+// returns false otherwise.
+template <typename TOut, bool SW>
+static bool launch_stream(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                          int ldx, int ldo, int out_cols, hipStream_t stream) {
+    const int strips = (N + 15) / 16;
+    if (M > 16 || K > 4096 || strips < 1024) return false;
+    const int units = SW ? strips / 4 * 2 : strips;          // SW: N is a multiple of 64 rows
+    const int groups = units < 512 ? units : 512;             // two work-groups' worth per compute unit, walked in order
+    const int per_group = (units + groups - 1) / groups * (SW ? 2 : 1);
+    const int items = SW ? units * 2 : units;
+    const int grid = (items + per_group - 1) / per_group;
+    const int ds = ((K + 63) / 64 + 15) / 16;
+#define TL_STREAM_CASE(d) \
+    if (ds == d) gemm_stream_kernel<16, d, TOut, SW><<<dim3(grid), dim3(1024), 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, items, per_group);
+    TL_STREAM_CASE(1) TL_STREAM_CASE(2) TL_STREAM_CASE(3) TL_STREAM_CASE(4)
+#undef TL_STREAM_CASE
+    return true;
+}
+
+// The streaming kernel by itself (tests and tuning).
+extern "C" int tl_gemm_stream_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
+                                      int M, int N, int K, int ldx, int ldo, int out_f32, hipStream_t stream) {
+    TL_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_stream: needs K, ldx multiples of 8");
+    const bool ok = out_f32 ? launch_stream<float, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream)
+                            : launch_stream<bf16_t, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
+    TL_REQUIRE(ok, "gemm_stream: shape M=%d N=%d K=%d does not fit (M <= 16, K <= 4096, N >= 16384)", M, N, K);
+    TL_CHECK_LAUNCH("gemm_stream");
+    return TL_OK;
 }
 
 template <int MT>
@@ -470,13 +649,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_mfma_tile_kernel(const bf
     }
 }
 
-// Shared memory of a tile kernel: two buffers of (BM + BN) rows of TK + 8 elements.  Beyond 64 KB
-// the kernel has to be allowed its size once per process.
-template <typename Kernel>
-static hipError_t allow_lds(Kernel kernel, size_t bytes) {
-    if (bytes <= 65536) return hipSuccess;
-    return hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-}
+// Shared memory of a tile kernel: two buffers of (BM + BN) rows of TK + 8 elements.
 
 template <int BM, int BN, int WGM, int WGN, typename TOut, bool SW, int TK>
 static int launch_mfma_tile_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
@@ -571,9 +744,8 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
     const bf16_t* wb = (const bf16_t*)w;
     bf16_t* ob = (bf16_t*)out;
     if (M <= 32) {
-        dim3 grid(N / 64), block(4 * 64);
-        if (M <= 16) gemm_skinny_kernel<4, 1, 4, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
-        else gemm_skinny_kernel<4, 2, 4, bf16_t, true><<<grid, block, 0, stream>>>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I);
+        if (M <= 16) launch_skinny_t<4, 1, 4, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
+        else launch_skinny_t<4, 2, 4, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
     } else {
         int rc;
         switch (pick_tile(M, N)) {

@@ -27,6 +27,8 @@ def embedding(token_ids, table, out):
 
 
 def add_rmsnorm(residual, pending, weight, eps, out, rows=None):
+    if pending is not None and pending.dim() == 3:
+        pending = pending.sum(0)
     if rows is None:
         if pending is not None:
             residual += pending.float()
@@ -124,6 +126,14 @@ def paged_attention_prefill(q, out, k_plane, v_plane, block_table, req_indptr, c
                             tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale):
     _attend(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles,
             tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale)
+
+
+def linear_partials(x, weight):
+    K = x.shape[1]
+    half = (K // 2 // 8) * 8 or K
+    a = x[:, :half].float() @ weight[:, :half].float().T
+    b = x[:, half:].float() @ weight[:, half:].float().T
+    return torch.stack((a, b))
 
 
 def swiglu(gate_up, out):

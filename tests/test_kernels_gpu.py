@@ -66,6 +66,36 @@ def test_add_rmsnorm(ops, dtype, wdtype, T, H, eps):
     torch.testing.assert_close(out3.double(), ref[rows.long()], **_tol(dtype))
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 33, 64])
+@pytest.mark.parametrize("N,K", [(3584, 18944), (100, 8192 + 200), (64, 64), (130, 4096)])
+def test_linear_partials_and_their_sum_in_the_norm(ops, M, N, K):
+    """Split-K slabs of partial sums: their sum is the product, and add_rmsnorm adds them up."""
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).cuda()
+    parts = ops.linear_partials(x, w)
+    assert parts.dim() == 3 and parts.shape[1:] == (M, N) and parts.dtype == torch.float32
+    assert parts.shape[0] == min(8, max(1, -(-K // 64) // 32)) or parts.shape[0] >= 1
+    ref = x.double() @ w.double().T
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    torch.testing.assert_close(parts.double().sum(0), ref, **tol32)
+    res = torch.randn(M, N, generator=g).cuda()
+    wn = (1 + 0.1 * torch.randn(N, generator=g)).to(torch.bfloat16).cuda()
+    r = res.clone()
+    out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    ops.add_rmsnorm(r, parts, wn, 1e-6, out)
+    total = res.double() + ref
+    torch.testing.assert_close(r.double(), total, rtol=1e-5, atol=2e-5)
+    refn = total * torch.rsqrt(total.pow(2).mean(-1, keepdim=True) + 1e-6) * wn.double()
+    torch.testing.assert_close(out.double(), refn, **_tol(torch.bfloat16))
+    rows = torch.tensor([M - 1, 0], dtype=torch.int32, device="cuda")
+    out2 = torch.empty(2, N, dtype=torch.bfloat16, device="cuda")
+    r2 = res.clone()
+    ops.add_rmsnorm(r2, parts, wn, 1e-6, out2, rows)
+    assert torch.equal(r2, res)
+    torch.testing.assert_close(out2.double(), refn[rows.long()], **_tol(torch.bfloat16))
+
+
 def test_rmsnorm_zero_row_is_zero_not_nan(ops):
     res = torch.zeros(2, 64, device="cuda")
     w = torch.ones(64, device="cuda")

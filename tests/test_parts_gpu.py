@@ -92,6 +92,31 @@ def test_swiglu_part_alone(dtype):
     torch.testing.assert_close(y.cpu().double(), ref, **_tol(dtype, ref))
 
 
+def test_swiglu_part_with_a_long_intermediate_hands_partial_sums_to_the_next_norm():
+    """17 to 64 rows over a long intermediate size: the down product comes back as slabs of
+    partial sums, which the next norm adds into the residual in 32-bit."""
+    from torchlet_amd.config import RMSNormSpec, SwiGLUSpec
+    from torchlet_amd.parts import FEED_FORWARDS, NORMS, Stream
+    hidden, inter, rows = 72, 8200, 24
+    dev = torch.device("cuda")
+    ffn = FEED_FORWARDS.build(SwiGLUSpec(hidden=hidden, intermediate=inter), torch.bfloat16, dev)
+    w = {"gate_proj.weight": torch.randn(inter, hidden) * 0.2, "up_proj.weight": torch.randn(inter, hidden) * 0.2,
+         "down_proj.weight": torch.randn(hidden, inter) * 0.03}
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    ffn.load_weights(w)
+    h = torch.randn(rows, hidden).to(torch.bfloat16)
+    y = ffn.forward(h.cuda(), None)
+    assert y.dim() == 3 and y.dtype == torch.float32 and y.shape[1:] == (rows, hidden)
+    ref = plain.swiglu_ffn(h.double(), {k: v.double() for k, v in w.items()})
+    torch.testing.assert_close(y.sum(0).cpu().double(), ref, **_tol(torch.bfloat16, ref))
+    norm = NORMS.build(RMSNormSpec(dim=hidden, eps=1e-6), torch.bfloat16, dev)
+    norm.load_weights({"weight": torch.ones(hidden, dtype=torch.bfloat16)})
+    res = torch.randn(rows, hidden).cuda()
+    stream = Stream(res.clone(), y)
+    norm.forward(stream)
+    torch.testing.assert_close(stream.residual.cpu().double(), res.cpu().double() + y.sum(0).cpu().double(), atol=1e-5, rtol=1e-6)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kvh,hd,window,bias", [(6, 2, 32, None, True), (4, 4, 16, 9, False), (7, 1, 64, None, True)])
 def test_attention_part_alone_whole_and_in_two_portions(dtype, heads, kvh, hd, window, bias):

@@ -34,20 +34,26 @@ extern "C" int tl_embedding(const void* ids, const void* table, int table_dtype,
 // One block per output row.  r = residual[row] (+ pending[row]); if `update`, r is
 // written back to the residual; out = r * rsqrt(mean(r^2) + eps) * weight.
 // `rows` (optional) selects the source row of each output row; then nothing is written back.
+// The pending branch output comes either as one [rows, hidden] tensor of the activation type
+// (parts == 0) or as `parts` float slabs [parts, total_rows, hidden] of partial sums that are
+// added up here (the split-K products write such slabs).
 template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ pending,
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const void* __restrict__ pending, int parts, size_t part_stride,
                                    const void* __restrict__ weight, int weight_f32, float eps,
                                    T* __restrict__ out, const int* __restrict__ rows, int hidden) {
     __shared__ float red[16];
     const int orow = blockIdx.x;
     const int srow = rows ? rows[orow] : orow;
     float* res = residual + (size_t)srow * hidden;
-    const T* pen = pending ? pending + (size_t)srow * hidden : nullptr;
-    const bool update = (pen != nullptr) && (rows == nullptr);
+    const T* pen = (pending && parts == 0) ? (const T*)pending + (size_t)srow * hidden : nullptr;
+    const float* pparts = (pending && parts > 0) ? (const float*)pending + (size_t)srow * hidden : nullptr;
+    const bool update = (pending != nullptr) && (rows == nullptr);
     float ss = 0.f;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float r = res[i];
         if (pen) r += to_float(pen[i]);
+        if (pparts)
+            for (int p = 0; p < parts; ++p) r += pparts[p * part_stride + i];
         if (update) res[i] = r;
         ss += r * r;
     }
@@ -56,7 +62,11 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __rest
     T* dst = out + (size_t)orow * hidden;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float r = res[i];
-        if (pen && !update) r += to_float(pen[i]);
+        if (!update) {
+            if (pen) r += to_float(pen[i]);
+            if (pparts)
+                for (int p = 0; p < parts; ++p) r += pparts[p * part_stride + i];
+        }
         dst[i] = from_float<T>(r * inv * load_vec(weight, weight_f32, i));
     }
 }
@@ -87,15 +97,16 @@ template <> struct Vec4<bf16_t> {
 };
 
 template <typename T, int IT>
-__global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const T* __restrict__ pending,
+__global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const void* __restrict__ pending, int parts, size_t part_stride,
                                        const void* __restrict__ weight, int weight_f32, float eps,
                                        T* __restrict__ out, const int* __restrict__ rows, int hidden) {
     __shared__ float red[16];
     const int orow = blockIdx.x;
     const int srow = rows ? rows[orow] : orow;
     float* res = residual + (size_t)srow * hidden;
-    const T* pen = pending ? pending + (size_t)srow * hidden : nullptr;
-    const bool update = (pen != nullptr) && (rows == nullptr);
+    const T* pen = (pending && parts == 0) ? (const T*)pending + (size_t)srow * hidden : nullptr;
+    const float* pparts = (pending && parts > 0) ? (const float*)pending + (size_t)srow * hidden : nullptr;
+    const bool update = (pending != nullptr) && (rows == nullptr);
     float r[IT][4], wv[IT][4];
     float ss = 0.f;
 #pragma unroll
@@ -108,6 +119,14 @@ __global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const T* __
                 Vec4<T>::load(pen + i, p);
 #pragma unroll
                 for (int v = 0; v < 4; ++v) r[it][v] += p[v];
+            }
+            if (pparts) {
+                for (int q = 0; q < parts; ++q) {
+                    float p[4];
+                    Vec4<float>::load(pparts + q * part_stride + i, p);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) r[it][v] += p[v];
+                }
             }
             if (weight_f32) Vec4<float>::load((const float*)weight + i, wv[it]);
             else Vec4<bf16_t>::load((const bf16_t*)weight + i, wv[it]);
@@ -138,34 +157,38 @@ __global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const T* __
 }
 
 template <typename T>
-static void launch_add_rmsnorm(float* residual, const T* pending, const void* weight, int weight_f32, float eps, T* out,
-                               const int* rows, int out_rows, int hidden, hipStream_t stream) {
+static void launch_add_rmsnorm(float* residual, const void* pending, int parts, size_t part_stride, const void* weight,
+                               int weight_f32, float eps, T* out, const int* rows, int out_rows, int hidden, hipStream_t stream) {
     const bool aligned = hidden % 4 == 0 && ((uintptr_t)residual % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
                          ((uintptr_t)pending % 16) == 0 && ((uintptr_t)weight % 16) == 0;
     dim3 grid(out_rows);
     if (aligned && hidden <= 1024)
-        add_rmsnorm_reg_kernel<T, 1><<<grid, 256, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 1><<<grid, 256, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
     else if (aligned && hidden <= 2048)
-        add_rmsnorm_reg_kernel<T, 2><<<grid, 256, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 2><<<grid, 256, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
     else if (aligned && hidden <= 4096)
-        add_rmsnorm_reg_kernel<T, 2><<<grid, 512, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 2><<<grid, 512, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
     else if (aligned && hidden <= 8192)
-        add_rmsnorm_reg_kernel<T, 4><<<grid, 512, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 4><<<grid, 512, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
     else if (aligned && hidden <= 16384)
-        add_rmsnorm_reg_kernel<T, 4><<<grid, 1024, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 4><<<grid, 1024, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
     else
-        add_rmsnorm_kernel<T><<<grid, hidden >= 2048 ? 512 : 256, 0, stream>>>(residual, pending, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_kernel<T><<<grid, hidden >= 2048 ? 512 : 256, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
 }
 
-extern "C" int tl_add_rmsnorm(void* residual, const void* pending, const void* weight, int weight_f32,
-                              float eps, void* out, const void* rows, int out_rows, int hidden,
+// parts == 0: `pending` is [rows, hidden] of the activation type (or null); parts > 0: `pending` is
+// float [parts, part_rows, hidden], slabs of partial sums to be added up.
+extern "C" int tl_add_rmsnorm(void* residual, const void* pending, int parts, int part_rows, const void* weight,
+                              int weight_f32, float eps, void* out, const void* rows, int out_rows, int hidden,
                               int act_dtype, hipStream_t stream) {
+    TL_REQUIRE(parts >= 0 && parts <= 64, "add_rmsnorm: %d partial slabs", parts);
+    const size_t part_stride = (size_t)part_rows * hidden;
     TL_REQUIRE(out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d hidden=%d", out_rows, hidden);
     if (out_rows == 0) return TL_OK;
     if (act_dtype == TL_DT_F32)
-        launch_add_rmsnorm<float>((float*)residual, (const float*)pending, weight, weight_f32, eps, (float*)out, (const int*)rows, out_rows, hidden, stream);
+        launch_add_rmsnorm<float>((float*)residual, pending, parts, part_stride, weight, weight_f32, eps, (float*)out, (const int*)rows, out_rows, hidden, stream);
     else if (act_dtype == TL_DT_BF16)
-        launch_add_rmsnorm<bf16_t>((float*)residual, (const bf16_t*)pending, weight, weight_f32, eps, (bf16_t*)out, (const int*)rows, out_rows, hidden, stream);
+        launch_add_rmsnorm<bf16_t>((float*)residual, pending, parts, part_stride, weight, weight_f32, eps, (bf16_t*)out, (const int*)rows, out_rows, hidden, stream);
     else TL_REQUIRE(false, "add_rmsnorm: unknown dtype %d", act_dtype);
     TL_CHECK_LAUNCH("add_rmsnorm");
     return TL_OK;

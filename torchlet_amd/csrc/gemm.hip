@@ -129,8 +129,19 @@ template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false
 __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                               const void* __restrict__ bias, int bias_f32,
                                                               TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-                                                              int out_cols = 0) {
+                                                              int out_cols = 0, int k_per_split = 0) {
     static_assert(!SW || (R == 4 && KS > 1), "the fused gate needs four strips per work-group");
+    // Split K (k_per_split > 0, a multiple of 64): blockIdx.y owns the columns
+    // [y * k_per_split, ...) of x and w and writes its own [M, ldo] slab of partial sums to out
+    // (float, no bias); whoever reads them adds the slabs up.
+    const int ldw = K;
+    if (k_per_split > 0) {
+        const int kb = blockIdx.y * k_per_split;
+        x += kb;
+        w += kb;
+        out += (size_t)blockIdx.y * M * ldo;
+        K = min(K - kb, k_per_split);
+    }
     extern __shared__ __attribute__((aligned(16))) float skinny_lds[];
     float* red = skinny_lds;                                             // KS * R * MT * 256 floats
     bf16_t* xs = (bf16_t*)(skinny_lds + KS * R * MT * 256);             // XL: M rows of K + 8 elements
@@ -142,7 +153,7 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
     const bf16_t* xrow[MT];
     int xoff[MT];
 #pragma unroll
-    for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + li, N - 1) * K;
+    for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + li, N - 1) * ldw;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         xrow[t] = x + (size_t)min(t * 16 + li, M - 1) * ldx;
@@ -301,7 +312,7 @@ static void launch_skinny_t(const void* x, const void* w, const void* bias, int 
         auto kernel = gemm_skinny_kernel<R, MT, KS, TOut, SW, true>;
         static hipError_t allowed = allow_lds(kernel, 96 * 1024);
         if (allowed == hipSuccess) {
-            kernel<<<grid, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols);
+            kernel<<<grid, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0);
             return;
         }
     }
@@ -757,5 +768,39 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
         if (rc != TL_OK) return rc;
     }
     TL_CHECK_LAUNCH("gemm_swiglu");
+    return TL_OK;
+}
+
+// out[P, M, N] (float) = partial sums of x w^T over P ranges of K, for a narrow matrix with a
+// long K (the down projection of a decode step): R = 4 strips per work-group share every x
+// fetch, and P work-groups per strip group keep all compute units busy.  Returns P through
+// `parts` (the caller sizes `out` for tl_gemm_partials_max()).
+extern "C" int tl_gemm_partials_max() { return 8; }
+
+extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int* parts,
+                                hipStream_t stream) {
+    TL_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0 && ldx >= K, "gemm_partials: bad sizes M=%d N=%d K=%d", M, N, K);
+    TL_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
+               "gemm_partials: needs K and the row stride of x to be multiples of 8 and 16-byte aligned operands");
+    const int steps = (K + 63) / 64;
+    int P = steps / 32;                                  // at least 32 steps (2048 columns) per part
+    if (P < 1) P = 1;
+    if (P > 8) P = 8;
+    const int k_per = ((steps + P - 1) / P) * 64;
+    P = (K + k_per - 1) / k_per;
+    *parts = P;
+    dim3 grid((N + 63) / 64, P), block(8 * 64);
+    const size_t red_bytes = (size_t)8 * 4 * (M <= 16 ? 1 : (M <= 32 ? 2 : 4)) * 1024;
+    if (M <= 16)
+        gemm_skinny_kernel<4, 1, 8, float, false, false><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
+    else if (M <= 32)
+        gemm_skinny_kernel<4, 2, 8, float, false, false><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
+    else {
+        auto kernel = gemm_skinny_kernel<4, 4, 8, float, false, false>;
+        static hipError_t allowed = allow_lds(kernel, 128 * 1024);
+        TL_REQUIRE(allowed == hipSuccess, "gemm_partials: cannot get %zu bytes of shared memory", red_bytes);
+        kernel<<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
+    }
+    TL_CHECK_LAUNCH("gemm_partials");
     return TL_OK;
 }

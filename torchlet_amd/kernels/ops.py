@@ -114,21 +114,46 @@ def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: to
                 out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
     """``r = residual (+ pending)``; ``out = r * rsqrt(mean(r^2) + eps) * weight``.
 
-    Without ``rows`` every row is processed and ``r`` is written back into ``residual``;
-    with ``rows`` (int32 source rows) only those are read and ``residual`` is untouched."""
+    ``pending`` is ``[T, H]`` of the activation dtype, or float32 ``[P, T, H]``: slabs of partial
+    sums (from :func:`linear_partials`) that are added up here.  Without ``rows`` every row is
+    processed and ``r`` is written back into ``residual``; with ``rows`` (int32 source rows) only
+    those are read and ``residual`` is untouched."""
     T, H = residual.shape
     n = T if rows is None else rows.numel()
     if residual.dtype != torch.float32 or not residual.is_contiguous():
         raise KernelError("add_rmsnorm: the residual must be contiguous float32")
-    if pending is not None and (pending.shape != residual.shape or pending.dtype != out.dtype or not pending.is_contiguous()):
-        raise KernelError(f"add_rmsnorm: pending {pending.dtype} {tuple(pending.shape)} does not match residual/out")
+    parts = 0
+    if pending is not None:
+        if pending.dim() == 3:
+            parts = pending.shape[0]
+            if pending.dtype != torch.float32 or pending.shape[1:] != residual.shape or not pending.is_contiguous():
+                raise KernelError(f"add_rmsnorm: partial sums {pending.dtype} {tuple(pending.shape)} are not float32 [P, {T}, {H}]")
+        elif pending.shape != residual.shape or pending.dtype != out.dtype or not pending.is_contiguous():
+            raise KernelError(f"add_rmsnorm: pending {pending.dtype} {tuple(pending.shape)} does not match residual/out")
     if out.shape != (n, H) or not out.is_contiguous():
         raise KernelError(f"add_rmsnorm: out must be contiguous [{n}, {H}], got {tuple(out.shape)}")
     _i32(rows, "add_rmsnorm rows")
     wf = _vec(weight, H, "add_rmsnorm weight")
     lib = _lib("elementwise")
-    _check(lib, lib.tl_add_rmsnorm(_ptr(residual), _ptr(pending), _ptr(weight), c_int(wf), c_float(eps), _ptr(out),
-                                   _ptr(rows), c_int(n), c_int(H), c_int(_dt(out, "add_rmsnorm")), _stream()))
+    _check(lib, lib.tl_add_rmsnorm(_ptr(residual), _ptr(pending), c_int(parts), c_int(T), _ptr(weight), c_int(wf),
+                                   c_float(eps), _ptr(out), _ptr(rows), c_int(n), c_int(H),
+                                   c_int(_dt(out, "add_rmsnorm")), _stream()))
+
+
+def linear_partials(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``x @ weight.T`` as float32 slabs ``[P, M, N]`` of partial sums over P ranges of K (bfloat16
+    operands, M <= 64, K a multiple of 8): for a narrow matrix with a long K, where splitting K
+    over work-groups is what fills the GPU.  The slabs are summed by :func:`add_rmsnorm`."""
+    M, K = x.shape
+    N = weight.shape[0]
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or weight.shape[1] != K or not weight.is_contiguous() or x.stride(1) != 1:
+        raise KernelError("linear_partials: bfloat16 operands and fitting shapes only")
+    lib = _lib("gemm")
+    out = torch.empty((lib.tl_gemm_partials_max(), M, N), dtype=torch.float32, device=x.device)
+    parts = c_int(0)
+    _check(lib, lib.tl_gemm_partials(_ptr(x), _ptr(weight), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(x.stride(0)),
+                                     ctypes.byref(parts), _stream()))
+    return out[: parts.value]
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor,

@@ -98,7 +98,8 @@ class Stream:
     """The hidden state between parts: a 32-bit residual ``[T, hidden]`` and the output
     of the last branch that is still to be added to it (``pending``, or ``None``).
     The next norm adds ``pending`` in 32-bit while it normalises, which saves one pass
-    over the residual per branch."""
+    over the residual per branch.  ``pending`` is ``[T, hidden]`` in the activation dtype, or
+    float32 ``[P, T, hidden]``: P slabs of partial sums that the norm adds up as well."""
 
     __slots__ = ("residual", "pending")
 

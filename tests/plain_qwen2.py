@@ -51,7 +51,7 @@ def rope_angles(positions: torch.Tensor, head_dim: int, theta: float) -> torch.T
     The inverse frequencies and the product are taken in float32, as the reference's
     table is (v00_full_recompute/layer/rope.py:29-35), then widened.
     """
-    j = torch.arange(0, head_dim, 2, dtype=torch.float32)
+    j = torch.arange(0, head_dim, 2, dtype=torch.float32, device=positions.device)
     inv_freq = 1.0 / (theta ** (j / head_dim))
     return torch.outer(positions.to(torch.float32), inv_freq)
 
@@ -86,7 +86,7 @@ def attention_weights(q: torch.Tensor, k: torch.Tensor, window: int | None = Non
     """
     t = q.shape[-2]
     scores = q @ k.transpose(-1, -2)
-    idx = torch.arange(t)
+    idx = torch.arange(t, device=q.device)
     hidden = idx[None, :] > idx[:, None]
     if window is not None:
         hidden = hidden | (idx[None, :] <= idx[:, None] - window)
@@ -104,6 +104,7 @@ def gqa_attention(
     theta: float,
     positions: torch.Tensor,
     window: int | None = None,
+    stored=lambda t: t,
 ) -> torch.Tensor:
     """Grouped-query attention of one request, ``h [T, hidden] -> [T, hidden]``.
 
@@ -111,42 +112,47 @@ def gqa_attention(
     rotation of q and k, K/V repeated ``num_heads/num_kv_heads`` times so that query
     head ``i`` reads KV head ``i // group``, causal softmax, output projection without
     bias.  Reference: v00_full_recompute/layer/gqa.py:43-91.
+
+    ``stored`` is applied to every tensor that an implementation in separate steps would
+    write to memory between them (projections, rotated heads, the mixed heads, the output);
+    a test passes a rounding there to see how much such roundings alone can move the result.
     """
     t = h.shape[0]
-    q = linear(h, w["q_proj.weight"], w.get("q_proj.bias"))
-    k = linear(h, w["k_proj.weight"], w.get("k_proj.bias"))
-    v = linear(h, w["v_proj.weight"], w.get("v_proj.bias"))
+    q = stored(linear(h, w["q_proj.weight"], w.get("q_proj.bias")))
+    k = stored(linear(h, w["k_proj.weight"], w.get("k_proj.bias")))
+    v = stored(linear(h, w["v_proj.weight"], w.get("v_proj.bias")))
     q = q.view(t, num_heads, head_dim).transpose(0, 1)
     k = k.view(t, num_kv_heads, head_dim).transpose(0, 1)
     v = v.view(t, num_kv_heads, head_dim).transpose(0, 1)
-    q = rope_apply(q, positions, theta)
-    k = rope_apply(k, positions, theta)
+    q = stored(rope_apply(q, positions, theta))
+    k = stored(rope_apply(k, positions, theta))
     group = num_heads // num_kv_heads
     k = k.repeat_interleave(group, dim=0)
     v = v.repeat_interleave(group, dim=0)
     weights = attention_weights(q, k, window)
-    ctx = (weights @ v).transpose(0, 1).contiguous().view(t, num_heads * head_dim)
-    return linear(ctx, w["o_proj.weight"])
+    ctx = stored((weights @ v).transpose(0, 1).contiguous().view(t, num_heads * head_dim))
+    return stored(linear(ctx, w["o_proj.weight"]))
 
 
-def swiglu_ffn(h: torch.Tensor, w: dict[str, torch.Tensor]) -> torch.Tensor:
+def swiglu_ffn(h: torch.Tensor, w: dict[str, torch.Tensor], stored=lambda t: t) -> torch.Tensor:
     """``down(silu(gate(h)) * up(h))``, no biases.
 
-    Reference: v00_full_recompute/layer/ffn_swiglu.py:8-14.
+    Reference: v00_full_recompute/layer/ffn_swiglu.py:8-14.  ``stored``: see :func:`gqa_attention`.
     """
     gate = linear(h, w["gate_proj.weight"])
     up = linear(h, w["up_proj.weight"])
-    return linear(torch.nn.functional.silu(gate) * up, w["down_proj.weight"])
+    return stored(linear(stored(torch.nn.functional.silu(gate) * up), w["down_proj.weight"]))
 
 
-def block(x: torch.Tensor, w: dict[str, torch.Tensor], cfg: "PlainConfig", layer: int, positions: torch.Tensor) -> torch.Tensor:
+def block(x: torch.Tensor, w: dict[str, torch.Tensor], cfg: "PlainConfig", layer: int, positions: torch.Tensor,
+          stored=lambda t: t) -> torch.Tensor:
     """Pre-norm residual block: ``x += attn(norm1(x)); x += ffn(norm2(x))``.
 
     Reference: v00_full_recompute/layer/transformer_block.py:34-37.
     """
     attn_w = _sub(w, "self_attn.")
     x = x + gqa_attention(
-        rms_norm(x, w["input_layernorm.weight"], cfg.eps),
+        stored(rms_norm(x, w["input_layernorm.weight"], cfg.eps)),
         attn_w,
         num_heads=cfg.num_heads,
         num_kv_heads=cfg.num_kv_heads,
@@ -154,8 +160,9 @@ def block(x: torch.Tensor, w: dict[str, torch.Tensor], cfg: "PlainConfig", layer
         theta=cfg.theta,
         positions=positions,
         window=cfg.window_of(layer),
+        stored=stored,
     )
-    x = x + swiglu_ffn(rms_norm(x, w["post_attention_layernorm.weight"], cfg.eps), _sub(w, "mlp."))
+    x = x + swiglu_ffn(stored(rms_norm(x, w["post_attention_layernorm.weight"], cfg.eps)), _sub(w, "mlp."), stored)
     return x
 
 
@@ -215,19 +222,21 @@ def load_folder(folder: str | Path, dtype: torch.dtype = torch.float64):
     return cfg, weights
 
 
-def forward(cfg: PlainConfig, weights: dict[str, torch.Tensor], token_ids: list[int], first_position: int = 0) -> torch.Tensor:
+def forward(cfg: PlainConfig, weights: dict[str, torch.Tensor], token_ids: list[int], first_position: int = 0,
+            stored=lambda t: t) -> torch.Tensor:
     """Logits ``[T, vocab]`` of one whole request.
 
     embedding, ``layers`` blocks, final norm, LM head without bias (the embedding
     matrix itself when tied).  Reference: v00_full_recompute/model/qwen2_5.py:55-82.
     ``first_position`` shifts every position by a constant (used by an invariance test).
     """
-    ids = torch.tensor(token_ids, dtype=torch.long)
-    positions = torch.arange(len(token_ids)) + first_position
+    device = weights["model.embed_tokens.weight"].device
+    ids = torch.tensor(token_ids, dtype=torch.long, device=device)
+    positions = torch.arange(len(token_ids), device=device) + first_position
     x = weights["model.embed_tokens.weight"][ids]
     for i in range(cfg.layers):
-        x = block(x, _sub(weights, f"model.layers.{i}."), cfg, i, positions)
-    x = rms_norm(x, weights["model.norm.weight"], cfg.eps)
+        x = block(x, _sub(weights, f"model.layers.{i}."), cfg, i, positions, stored)
+    x = stored(rms_norm(x, weights["model.norm.weight"], cfg.eps))
     head = weights["model.embed_tokens.weight"] if cfg.tied else weights["lm_head.weight"]
     return linear(x, head)
 

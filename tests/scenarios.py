@@ -110,10 +110,9 @@ def expected_logits(folder, requests):
     return {r: plain_qwen2.forward(cfg, weights, t) for r, t in requests.items()}
 
 
-def check(steps, outputs, expected, tol, what=""):
-    """``outputs[step]``: array ``[wanted, vocab]``.  Every row is compared with the plain
-    implementation's logits of its request at its absolute position; the first mismatch
-    is reported with its place."""
+def _rows(steps, outputs, expected, what=""):
+    """Every wanted row of a replay beside the plain implementation's logits of its request
+    at its absolute position: ``(got, ref, place)``."""
     pos: dict[str, int] = {}
     for s in steps:
         rows = outputs.get(s["step"])
@@ -122,14 +121,28 @@ def check(steps, outputs, expected, tol, what=""):
             base = pos.get(e["id"], 0)
             for w in e["want"]:
                 got = torch.from_numpy(np.asarray(rows[k], dtype=np.float32)).double()
-                ref = expected[e["id"]][base + w]
-                if not torch.allclose(got, ref, **tol):
-                    err = float((got - ref).abs().max())
-                    raise AssertionError(
-                        f"{what}: step {s['step']} request {e['id']} position {base + w} "
-                        f"(portion starts at {base}, place {w} of {len(e['tokens'])}): max abs error {err:.3e}")
+                yield got, expected[e["id"]][base + w], (f"step {s['step']} request {e['id']} position {base + w} "
+                                                        f"(portion starts at {base}, place {w} of {len(e['tokens'])})")
                 k += 1
             pos[e["id"]] = base + len(e["tokens"])
         assert rows is None or k == len(rows), f"{what}: step {s['step']} returned {len(rows)} rows, {k} wanted"
         for r in s["end"]:
             pos.pop(r, None)
+
+
+def check(steps, outputs, expected, tol, what=""):
+    """``outputs[step]``: array ``[wanted, vocab]``.  Every row is compared with the plain
+    implementation's logits of its request at its absolute position; the first mismatch
+    is reported with its place."""
+    for got, ref, place in _rows(steps, outputs, expected, what):
+        if not torch.allclose(got, ref, **tol):
+            raise AssertionError(f"{what}: {place}: max abs error {float((got - ref).abs().max()):.3e}")
+
+
+def rms_error(steps, outputs, expected) -> float:
+    """Root mean square of the error over every wanted logit of a replay."""
+    total, count = 0.0, 0
+    for got, ref, _ in _rows(steps, outputs, expected):
+        total += float((got - ref).pow(2).sum())
+        count += ref.numel()
+    return (total / max(count, 1)) ** 0.5

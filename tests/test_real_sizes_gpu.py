@@ -1,0 +1,113 @@
+"""The engine at the layer widths of the 7B, 14B and 32B checkpoints (all heads, groups,
+intermediate sizes and the whole vocabulary, one or two layers, random weights) against the
+plain implementation, under every way of cutting the requests into steps.
+
+The plain implementation runs on the GPU here, in 64-bit, through library routines only; it
+shares no code with the engine.  The 32-bit bound is set from the plain implementation
+itself: its own 32-bit evaluation differs from the 64-bit one by rounding that depends on
+the order of summation only, and an engine that sums the same terms in another order may
+differ by a small multiple of that and no more.  The bfloat16 bound comes from the plain
+implementation as well: evaluated in 64-bit, but with every tensor that separate kernels hand
+to each other through memory (normalised activations, projections, rotated heads, mixed heads,
+branch outputs) rounded to bfloat16, it moves away from the unrounded result by what such
+roundings alone do.  The engine rounds at these places or at fewer (the residual, the norms and
+the softmax stay in 32-bit), in another order of summation, so its error has the same law; the
+bound is twice the largest such move, over all logits of all requests, and the root mean
+square of the engine's error, an average over tens of millions of logits and so a sharp
+figure, may exceed that of the moves by a quarter at most."""
+import pytest
+import torch
+
+import plain_qwen2 as plain
+import scenarios
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = {
+    "7B": dict(num_hidden_layers=2, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
+               intermediate_size=18944, rms_norm_eps=1e-6),
+    "14B": dict(num_hidden_layers=1, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,
+                intermediate_size=13824, rms_norm_eps=1e-5),
+    "32B": dict(num_hidden_layers=1, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,
+                intermediate_size=27648, rms_norm_eps=1e-5),
+}
+COMMON = dict(architectures=["Qwen2ForCausalLM"], vocab_size=152064, max_position_embeddings=4096, rope_theta=1e6,
+              attention_bias=True, tie_word_embeddings=False)
+LENGTHS = [150, 70, 200, 40, 97]
+PAGE = 16
+NOISE_FACTOR = 8.0
+
+
+@pytest.fixture(scope="module", params=list(SHAPES))
+def sized(request):
+    from torchlet_amd.registry import ARCHITECTURES
+    from torchlet_amd.weights.random_init import random_tensors
+    d = dict(COMMON, **SHAPES[request.param])
+    config = ARCHITECTURES["Qwen2ForCausalLM"].from_dict(d)
+    seed = 2 + list(SHAPES).index(request.param)
+    tensors = random_tensors(config, seed=seed, dtype=torch.bfloat16, device="cuda")
+    requests = scenarios.make_requests(d["vocab_size"], LENGTHS, seed=5)
+    cfg = plain.PlainConfig(d)
+    w64 = {k: v.double() for k, v in tensors.items()}
+    expected = {r: plain.forward(cfg, w64, t).cpu() for r, t in requests.items()}
+    del w64
+    w32 = {k: v.float() for k, v in tensors.items()}
+    noise = max(float((plain.forward(cfg, w32, t).cpu().double() - expected[r]).abs().max()) for r, t in requests.items())
+    del w32
+    w64 = {k: v.double() for k, v in tensors.items()}
+    rounded = lambda t: t.to(torch.bfloat16).double()
+    moved = {r: plain.forward(cfg, w64, t, stored=rounded).cpu() - expected[r] for r, t in requests.items()}
+    noise16 = max(float(m.abs().max()) for m in moved.values())
+    rms16 = float(torch.cat([m.flatten() for m in moved.values()]).pow(2).mean().sqrt())
+    del w64, moved
+    torch.cuda.empty_cache()
+    print(f"{request.param}: 32-bit noise {noise:.3e}, bfloat16 roundings move the logits by {noise16:.3e} at most, {rms16:.3e} rms", flush=True)
+    yield request.param, config, tensors, requests, expected, (noise, noise16, rms16)
+    del tensors
+    torch.cuda.empty_cache()
+
+
+def _replay(model, steps, max_tokens):
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import make_runner
+    runner = make_runner(model, page_size=PAGE, num_pages=-(-max_tokens // PAGE) + 1, max_requests=4)
+    out = {}
+    for s in steps:
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        if logits is not None:
+            out[s["step"]] = logits.cpu().numpy()
+        for r in s["end"]:
+            runner.release(r)
+    runner.cache.check()
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_every_split_at_checkpoint_widths(sized, dtype):
+    from torchlet_amd.engine.loading import build_model
+    name, config, tensors, requests, expected, (noise, noise16, rms16) = sized
+    rms = float(torch.cat([e.flatten() for e in expected.values()]).pow(2).mean().sqrt())
+    assert 0 < noise < 1e-3 * rms, f"the plain implementation's own 32-bit rounding ({noise:.2e}) should be far below the logits' size ({rms:.2e})"
+    if dtype == "float32":
+        tol = dict(atol=NOISE_FACTOR * noise, rtol=2e-5)
+    else:
+        assert noise16 < 0.1 * rms, f"bfloat16 roundings alone move the logits by {noise16:.2e} at a size of {rms:.2e}: too coarse a yardstick"
+        tol = dict(atol=2 * noise16, rtol=0.0)
+    model = build_model(config, dtype, tensors=tensors)
+    modes = {
+        "whole": scenarios.whole(requests),
+        "tail_singles": scenarios.tail_singles(requests),
+        "portions": scenarios.portions(requests),
+        "mixed": scenarios.mixed(requests, seed=3),
+    }
+    for mode, steps in modes.items():
+        steps = scenarios.number(steps)
+        print(f"{name} {dtype} {mode}: {len(steps)} steps", flush=True)
+        out = _replay(model, steps, scenarios.max_tokens_needed(steps, unit=PAGE))
+        scenarios.check(steps, out, expected, tol, what=f"{name} {dtype} {mode}")
+        if dtype == "bfloat16":
+            err = scenarios.rms_error(steps, out, expected)
+            print(f"    rms error {err:.3e}", flush=True)
+            assert err <= 1.25 * rms16, f"{name} {mode}: rms error {err:.3e}, bfloat16 roundings alone give {rms16:.3e}"
+    del model
+    torch.cuda.empty_cache()

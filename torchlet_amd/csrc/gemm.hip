@@ -115,6 +115,21 @@ union Frag16 {          // 16 bytes: eight bfloat16 as the MFMA wants them, or o
     bf16x8_t v;
 };
 
+__device__ __forceinline__ void lds_barrier() {
+    // waits for this wave's shared-memory traffic only: weight fetches stay in flight across it
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// Register sets of weights a wave of the skinny kernel keeps in flight: as many K steps as fit
+// beside the accumulators (a step takes 8 registers per strip and 8 per tile of activation rows).
+template <int R, int MT, int KS>
+constexpr int skinny_depth() {
+    const int per_step = 8 * R + 8 * MT;
+    const int budget = KS >= 16 ? 64 : 128;       // 1024 threads leave 128 registers a lane
+    const int d = budget / per_step;
+    return d < 2 ? 2 : (d > 8 ? 8 : d);
+}
+
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + expf(-g)) * u; }
 
 // SW (gate/up product with the SwiGLU gate applied to the accumulators): w holds blocks of 64
@@ -125,7 +140,9 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + 
 // every operand load of x becomes a trip to L2 that competes with the weight stream (measured:
 // 5.6 TB/s at M = 1, 4.6 at M = 8, 3.7 at M = 16 without it).  With XL the work-group copies
 // its M rows of x into shared memory once, coalesced, and reads the operands from there.
-template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false>
+// D: how many K steps of weights a wave keeps in flight (a ring of D register sets).  Short
+// rows (a few steps per wave) want them all in flight at once, or every step costs a trip to memory.
+template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false, int D = 2>
 __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                               const void* __restrict__ bias, int bias_f32,
                                                               TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
@@ -159,14 +176,6 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
         xrow[t] = x + (size_t)min(t * 16 + li, M - 1) * ldx;
         xoff[t] = min(t * 16 + li, M - 1) * (K + 8);
     }
-    if (XL) {
-        const int pieces = K / 8;                     // 16-byte pieces per row
-        for (int i = threadIdx.x; i < M * pieces; i += KS * 64) {
-            const int row = i / pieces, pc = i % pieces;
-            *(uint4*)(&xs[row * (K + 8) + pc * 8]) = *(const uint4*)(x + (size_t)row * ldx + pc * 8);
-        }
-        __syncthreads();
-    }
 #define SK_LOADB(t, k) (XL ? *(const uint4*)(&xs[xoff[t] + (k)]) : *(const uint4*)(xrow[t] + (k)))
 
     f32x4_t acc[R][MT];
@@ -176,36 +185,59 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
         for (int t = 0; t < MT; ++t) acc[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     const int full = K / 64;                   // steps that lie wholly inside K
-    Frag16 a0[R], a1[R], b0[MT], b1[MT];
-    int s = wave;
-    if (s < full) {
-        const int k = 64 * s + SK_KOFF(lg);
-#pragma unroll
-        for (int r = 0; r < R; ++r) { a0[r].u = SK_LOAD(wrow[r] + k); a1[r].u = SK_LOAD(wrow[r] + k + SK_SECOND); }
-#pragma unroll
-        for (int t = 0; t < MT; ++t) { b0[t].u = SK_LOADB(t, k); b1[t].u = SK_LOADB(t, k + SK_SECOND); }
+    // this wave's steps are s = wave + i * KS, i = 0 .. mine - 1; slot d of the ring holds step i = d (mod D)
+    const int mine = full > wave ? (full - wave + KS - 1) / KS : 0;
+    Frag16 wa0[D][R], wa1[D][R], wb0[D][MT], wb1[D][MT];
+#define SK_ISSUE(d, i)                                                                              \
+    {                                                                                               \
+        const int k_ = 64 * (wave + (i) * KS) + SK_KOFF(lg);                                        \
+        _Pragma("unroll") for (int r = 0; r < R; ++r) {                                             \
+            wa0[d][r].u = SK_LOAD(wrow[r] + k_);                                                    \
+            wa1[d][r].u = SK_LOAD(wrow[r] + k_ + SK_SECOND);                                        \
+        }                                                                                           \
+        if (!XL) {                                                                                  \
+            _Pragma("unroll") for (int t = 0; t < MT; ++t) {                                        \
+                wb0[d][t].u = SK_LOAD(xrow[t] + k_);                                                \
+                wb1[d][t].u = SK_LOAD(xrow[t] + k_ + SK_SECOND);                                    \
+            }                                                                                       \
+        }                                                                                           \
     }
-    for (; s < full; s += KS) {
-        // fetch the next step (the last one fetches itself again: no branch in the loop)
-        Frag16 na0[R], na1[R], nb0[MT], nb1[MT];
-        const int sn = (s + KS < full) ? s + KS : s;
-        const int kn = 64 * sn + SK_KOFF(lg);
 #pragma unroll
-        for (int r = 0; r < R; ++r) { na0[r].u = SK_LOAD(wrow[r] + kn); na1[r].u = SK_LOAD(wrow[r] + kn + SK_SECOND); }
+    for (int d = 0; d < D; ++d)
+        if (d < mine) SK_ISSUE(d, d)
+    if (XL) {                                  // the weights are on their way while x is copied
+        const int pieces = K / 8;                     // 16-byte pieces per row
+        for (int i = threadIdx.x; i < M * pieces; i += KS * 64) {
+            const int row = i / pieces, pc = i % pieces;
+            *(uint4*)(&xs[row * (K + 8) + pc * 8]) = *(const uint4*)(x + (size_t)row * ldx + pc * 8);
+        }
+        lds_barrier();
+    }
+    for (int i = 0; i < mine; i += D) {
 #pragma unroll
-        for (int t = 0; t < MT; ++t) { nb0[t].u = SK_LOADB(t, kn); nb1[t].u = SK_LOADB(t, kn + SK_SECOND); }
+        for (int d = 0; d < D; ++d) {
+            if (i + d < mine) {
+                if (XL) {
+                    const int k = 64 * (wave + (i + d) * KS) + SK_KOFF(lg);
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+                    for (int t = 0; t < MT; ++t) {
+                        wb0[d][t].u = *(const uint4*)(&xs[xoff[t] + k]);
+                        wb1[d][t].u = *(const uint4*)(&xs[xoff[t] + k + SK_SECOND]);
+                    }
+                }
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[r].v, b0[t].v, acc[r][t], 0, 0, 0);
-                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[r].v, b1[t].v, acc[r][t], 0, 0, 0);
+                for (int r = 0; r < R; ++r)
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) {
+                        acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa0[d][r].v, wb0[d][t].v, acc[r][t], 0, 0, 0);
+                        acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa1[d][r].v, wb1[d][t].v, acc[r][t], 0, 0, 0);
+                    }
+                if (i + d + D < mine) SK_ISSUE(d, i + d + D)
             }
-#pragma unroll
-        for (int r = 0; r < R; ++r) { a0[r] = na0[r]; a1[r] = na1[r]; }
-#pragma unroll
-        for (int t = 0; t < MT; ++t) { b0[t] = nb0[t]; b1[t] = nb1[t]; }
+        }
     }
+#undef SK_ISSUE
+    Frag16 a0[R], a1[R], b0[MT], b1[MT];
     // the tail step (K % 64 != 0) belongs to the wave whose turn it is; pieces beyond K count as zero
     if ((K & 63) && (full % KS) == wave) {
         const int k = 64 * full + SK_KOFF(lg);
@@ -300,8 +332,8 @@ static hipError_t allow_lds(Kernel kernel, size_t bytes) {
 #define SKINNY_XL_MAX_BYTES (60 * 1024)      // x may take this much shared memory: with the reduction buffer two
                                              // work-groups still fit the 160 KB of a compute unit
 
-template <int R, int MT, int KS, typename TOut, bool SW>
-static void launch_skinny_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+template <int R, int MT, int KS, typename TOut, bool SW, int D>
+static void launch_skinny_d(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                             int ldx, int ldo, int out_cols, hipStream_t stream) {
     dim3 grid((N + 16 * R - 1) / (16 * R)), block(KS * 64);
     const size_t red_bytes = (size_t)KS * R * MT * 1024;
@@ -309,14 +341,27 @@ static void launch_skinny_t(const void* x, const void* w, const void* bias, int 
     // (not with few waves per work-group: the copy of x then takes longer than it saves; measured on the
     // fused gate/up kernel, 87 us with against 64 us without at M = 8)
     if (M > 1 && KS >= 8 && x_bytes <= SKINNY_XL_MAX_BYTES) {
-        auto kernel = gemm_skinny_kernel<R, MT, KS, TOut, SW, true>;
+        auto kernel = gemm_skinny_kernel<R, MT, KS, TOut, SW, true, D>;
         static hipError_t allowed = allow_lds(kernel, 96 * 1024);
         if (allowed == hipSuccess) {
             kernel<<<grid, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0);
             return;
         }
     }
-    gemm_skinny_kernel<R, MT, KS, TOut, SW, false><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols);
+    gemm_skinny_kernel<R, MT, KS, TOut, SW, false, D><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0);
+}
+
+// A wave with many K steps ahead of it (a long K: the down projection) keeps as many in flight as
+// its registers hold; with a few steps (K of a hidden size) two are as good and start sooner
+// (measured at 3584 x 18944, one row: 33 -> 28 us with eight in flight; at 4608 x 3584: 11 -> 12.6 us).
+template <int R, int MT, int KS, typename TOut, bool SW>
+static void launch_skinny_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                            int ldx, int ldo, int out_cols, hipStream_t stream) {
+    constexpr int deep = skinny_depth<R, MT, KS>();
+    if (deep > 2 && K / 64 / KS >= 16)
+        launch_skinny_d<R, MT, KS, TOut, SW, deep>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    else
+        launch_skinny_d<R, MT, KS, TOut, SW, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
 }
 
 template <int R, int MT, int KS>
@@ -337,11 +382,6 @@ static void launch_skinny(const void* x, const void* w, const void* bias, int bi
 // the weight stream never stops for a strip's epilogue.  Needs K <= 64 * KS * DS.
 // SW: the matrix is the interleaved gate/up matrix (see gemm_skinny_kernel); a work item is a
 // (gate strip, up strip) pair, processed as two strips whose sums the same wave combines.
-__device__ __forceinline__ void lds_barrier() {
-    // waits for this wave's shared-memory traffic only: weight fetches stay in flight across it
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
 template <int KS, int DS, typename TOut, bool SW>
 __global__ __launch_bounds__(KS * 64) void gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                               const void* __restrict__ bias, int bias_f32,
@@ -792,11 +832,11 @@ extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, 
     dim3 grid((N + 63) / 64, P), block(8 * 64);
     const size_t red_bytes = (size_t)8 * 4 * (M <= 16 ? 1 : (M <= 32 ? 2 : 4)) * 1024;
     if (M <= 16)
-        gemm_skinny_kernel<4, 1, 8, float, false, false><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
+        gemm_skinny_kernel<4, 1, 8, float, false, false, skinny_depth<4, 1, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
     else if (M <= 32)
-        gemm_skinny_kernel<4, 2, 8, float, false, false><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
+        gemm_skinny_kernel<4, 2, 8, float, false, false, skinny_depth<4, 2, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
     else {
-        auto kernel = gemm_skinny_kernel<4, 4, 8, float, false, false>;
+        auto kernel = gemm_skinny_kernel<4, 4, 8, float, false, false, skinny_depth<4, 4, 8>()>;
         static hipError_t allowed = allow_lds(kernel, 128 * 1024);
         TL_REQUIRE(allowed == hipSuccess, "gemm_partials: cannot get %zu bytes of shared memory", red_bytes);
         kernel<<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);

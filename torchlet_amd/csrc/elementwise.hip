@@ -195,7 +195,7 @@ extern "C" int tl_add_rmsnorm(void* residual, const void* pending, int parts, in
 }
 
 // ------------------------------------------------------------------ RoPE + cache write
-// One block per token.  Row layout of `qkv`: [q heads | k heads | v heads], each head
+// One wave per token and head.  Row layout of `qkv`: [q heads | k heads | v heads], each head
 // `head_dim` wide, row stride `row_stride` elements.
 //   * rotate (inv_freq != null): the first `rot_heads` heads (q, then k) are rotated in
 //     place with the split-half pairing (j, j + head_dim/2) by angle = float(pos) * inv_freq[j].
@@ -203,60 +203,54 @@ extern "C" int tl_add_rmsnorm(void* residual, const void* pending, int parts, in
 //     block_table[token_req[t]][pos / page] at offset pos % page.  The key plane is
 //     [pages, kv_heads, page, head_dim]; the value plane holds each page transposed,
 //     [pages, kv_heads, head_dim, page], the layout the attention kernels read.
+#define ROPE_HEADS_PER_GROUP 4          // one wave per head, four heads per work-group
 template <typename T>
-__global__ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, int kv_heads,
-                                        int head_dim, int rot_heads, const int* __restrict__ positions,
-                                        const float* __restrict__ inv_freq, const int* __restrict__ token_req,
-                                        const int* __restrict__ block_table, int bt_stride,
-                                        T* __restrict__ k_plane, T* __restrict__ v_plane, int page_size) {
+__global__ __launch_bounds__(ROPE_HEADS_PER_GROUP * TL_WAVE)
+void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, int kv_heads,
+                             int head_dim, int rot_heads, const int* __restrict__ positions,
+                             const float* __restrict__ inv_freq, const int* __restrict__ token_req,
+                             const int* __restrict__ block_table, int bt_stride,
+                             T* __restrict__ k_plane, T* __restrict__ v_plane, int page_size) {
+    // A wave owns one head of one token: a query head (rotated in place), a key head (rotated in
+    // place and written to its page) or a value head (written to its page, transposed).  Each wave
+    // takes the cosines and sines of its own pairs, so no wave waits for another.
     const int t = blockIdx.x;
+    const int head = blockIdx.y * ROPE_HEADS_PER_GROUP + threadIdx.x / TL_WAVE;
+    const int lane = threadIdx.x % TL_WAVE;
+    const int heads = q_heads + kv_heads + (k_plane ? kv_heads : 0);
+    if (head >= heads) return;
     const int pos = positions[t];
-    T* row = qkv + (size_t)t * row_stride;
     const int half = head_dim / 2;
-    T* kdst = nullptr;
-    T* vdst = nullptr;
-    if (k_plane) {
+    T* x = qkv + (size_t)t * row_stride + (size_t)head * head_dim;
+    T* dst = nullptr;                      // this head's place in the cache, if it has one
+    if (k_plane && head >= q_heads) {
         const int page = block_table[(size_t)token_req[t] * bt_stride + pos / page_size];
-        const size_t base = ((size_t)page * kv_heads) * page_size * head_dim;
-        kdst = k_plane + base + (size_t)(pos % page_size) * head_dim;
-        vdst = v_plane + base + (pos % page_size);
+        const int kvh = (head - q_heads) % kv_heads;
+        const size_t base = ((size_t)page * kv_heads + kvh) * page_size * head_dim;
+        dst = head < q_heads + kv_heads ? k_plane + base + (size_t)(pos % page_size) * head_dim
+                                        : v_plane + base + (pos % page_size);
     }
-    const size_t head_step = (size_t)page_size * head_dim;  // between kv heads inside a page
-    // cosine and sine of the token's angles, once per frequency (every head shares them)
-    __shared__ float cs[2][128];
-    if (inv_freq) {
-        for (int j = threadIdx.x; j < half; j += blockDim.x) {
-            const float angle = (float)pos * inv_freq[j];
-            cs[0][j] = cosf(angle);
-            cs[1][j] = sinf(angle);
-        }
-        __syncthreads();
+    if (head >= q_heads + kv_heads) {      // value head: [head_dim, page] inside the page
+        for (int d = lane; d < head_dim; d += TL_WAVE) dst[(size_t)d * page_size] = x[d];
+        return;
     }
-    const int pairs = (q_heads + kv_heads) * half;
-    for (int idx = threadIdx.x; idx < pairs; idx += blockDim.x) {
-        const int head = idx / half, j = idx % half;
-        T* x = row + (size_t)head * head_dim;
+    const bool rotate = inv_freq && head < rot_heads;
+    if (!rotate && !dst) return;
+    for (int j = lane; j < half; j += TL_WAVE) {
         float x1 = to_float(x[j]), x2 = to_float(x[j + half]);
-        if (inv_freq && head < rot_heads) {
-            const float c = cs[0][j], s = cs[1][j];
-            const float y1 = x1 * c - x2 * s;
-            const float y2 = x2 * c + x1 * s;
+        if (rotate) {
+            const float angle = (float)pos * inv_freq[j];
+            const float c = cosf(angle), sn = sinf(angle);
+            const float y1 = x1 * c - x2 * sn;
+            const float y2 = x2 * c + x1 * sn;
             x1 = y1;
             x2 = y2;
             x[j] = from_float<T>(x1);
             x[j + half] = from_float<T>(x2);
         }
-        if (kdst && head >= q_heads) {
-            T* d = kdst + (size_t)(head - q_heads) * head_step;
-            d[j] = from_float<T>(x1);
-            d[j + half] = from_float<T>(x2);
-        }
-    }
-    if (vdst) {
-        const T* v = row + (size_t)(q_heads + kv_heads) * head_dim;
-        for (int idx = threadIdx.x; idx < kv_heads * head_dim; idx += blockDim.x) {
-            const int head = idx / head_dim, d = idx % head_dim;
-            vdst[(size_t)head * head_step + (size_t)d * page_size] = v[idx];
+        if (dst) {
+            dst[j] = from_float<T>(x1);
+            dst[j + half] = from_float<T>(x2);
         }
     }
 }
@@ -275,7 +269,8 @@ extern "C" int tl_rope_cache_write(void* qkv, int row_stride, int tokens, int q_
     TL_REQUIRE(row_stride >= (q_heads + (k_plane ? 2 * kv_heads : kv_heads)) * head_dim,
                "rope_cache_write: row stride %d too small", row_stride);
     if (tokens == 0) return TL_OK;
-    dim3 grid(tokens), block(256);
+    const int heads = q_heads + kv_heads + (k_plane ? kv_heads : 0);
+    dim3 grid(tokens, (heads + ROPE_HEADS_PER_GROUP - 1) / ROPE_HEADS_PER_GROUP), block(ROPE_HEADS_PER_GROUP * TL_WAVE);
     if (act_dtype == TL_DT_F32)
         rope_cache_write_kernel<float><<<grid, block, 0, stream>>>((float*)qkv, row_stride, q_heads, kv_heads, head_dim, rot_heads,
             (const int*)positions, (const float*)inv_freq, (const int*)token_req, (const int*)block_table, bt_stride,

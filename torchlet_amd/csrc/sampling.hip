@@ -1,5 +1,5 @@
 // Sampling from logits: greedy (arg max, lowest index on ties) and temperature sampling
-// by the Gumbel-max rule, one block per row.
+// by the Gumbel-max rule, in two stages: many work-groups scan a row, one wave picks.
 //
 // Temperature t > 0: the token is argmax_i(logit_i / t + g_i) with g_i = -log(-log(u_i)),
 // which is an exact draw from softmax(logits / t).  u_i comes from a counter-based hash
@@ -20,46 +20,86 @@ __device__ __forceinline__ float gumbel(uint32_t key, uint32_t i) {
     return -logf(-logf(u));
 }
 
-__global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ logits, int vocab, int ld,
-                                                      const float* __restrict__ temperature,
-                                                      const int* __restrict__ keys, int* __restrict__ out) {
-    __shared__ float bv[16];
-    __shared__ int bi[16];
-    const int row = blockIdx.x;
-    const float* x = logits + (size_t)row * ld;
-    const float t = temperature ? temperature[row] : 0.f;
-    const uint32_t key = keys ? (uint32_t)keys[row] : 0u;
-    float best = -INFINITY;
-    int besti = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-        float v = x[i];
-        if (t > 0.f) v = v / t + gumbel(key, (uint32_t)i);
-        if (v > best) { best = v; besti = i; }        // strided scan: earlier i wins ties
-    }
+// One row's candidate: the larger value wins, the lower index on ties.
+__device__ __forceinline__ void keep_better(float& best, int& besti, float v, int i) {
+    if (v > best || (v == best && i < besti)) { best = v; besti = i; }
+}
+
+__device__ __forceinline__ void wave_best(float& best, int& besti) {
 #pragma unroll
     for (int o = TL_WAVE / 2; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, TL_WAVE);
         const int oi = __shfl_xor(besti, o, TL_WAVE);
-        if (ov > best || (ov == best && oi < besti)) { best = ov; besti = oi; }
+        keep_better(best, besti, ov, oi);
     }
+}
+
+// Stage 1: work-group (chunk, row) scans columns [chunk * per, (chunk + 1) * per) of its row and
+// leaves its candidate in part_v / part_i [row, chunk].  A row of a large vocabulary is spread
+// over many work-groups, so the scan is as wide as the machine and not as long as the row.
+#define SAMPLE_THREADS 256
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_scan_kernel(const float* __restrict__ logits, int vocab, int ld, int per,
+                                                                     const float* __restrict__ temperature,
+                                                                     const int* __restrict__ keys,
+                                                                     float* __restrict__ part_v, int* __restrict__ part_i) {
+    __shared__ float bv[SAMPLE_THREADS / TL_WAVE];
+    __shared__ int bi[SAMPLE_THREADS / TL_WAVE];
+    const int chunk = blockIdx.x, row = blockIdx.y;
+    const float* x = logits + (size_t)row * ld;
+    const float t = temperature ? temperature[row] : 0.f;
+    const uint32_t key = keys ? (uint32_t)keys[row] : 0u;
+    const int end = min(vocab, (chunk + 1) * per);
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    for (int i = chunk * per + threadIdx.x; i < end; i += SAMPLE_THREADS) {
+        float v = x[i];
+        if (t > 0.f) v = v / t + gumbel(key, (uint32_t)i);
+        if (v > best) { best = v; besti = i; }        // strided scan: earlier i wins ties
+    }
+    wave_best(best, besti);
     const int wave = threadIdx.x / TL_WAVE, lane = threadIdx.x % TL_WAVE;
     if (lane == 0) { bv[wave] = best; bi[wave] = besti; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        const int nw = (blockDim.x + TL_WAVE - 1) / TL_WAVE;
-        for (int w = 1; w < nw; ++w)
-            if (bv[w] > best || (bv[w] == best && bi[w] < besti)) { best = bv[w]; besti = bi[w]; }
-        out[row] = besti < vocab ? besti : 0;
+        for (int w = 1; w < SAMPLE_THREADS / TL_WAVE; ++w) keep_better(best, besti, bv[w], bi[w]);
+        part_v[(size_t)row * gridDim.x + chunk] = best;
+        part_i[(size_t)row * gridDim.x + chunk] = besti;
     }
 }
 
+// Stage 2: one wave per row picks among the chunks' candidates.
+__global__ __launch_bounds__(TL_WAVE) void sample_pick_kernel(const float* __restrict__ part_v, const int* __restrict__ part_i,
+                                                              int chunks, int vocab, int* __restrict__ out) {
+    const int row = blockIdx.x;
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    for (int c = threadIdx.x; c < chunks; c += TL_WAVE)
+        keep_better(best, besti, part_v[(size_t)row * chunks + c], part_i[(size_t)row * chunks + c]);
+    wave_best(best, besti);
+    if (threadIdx.x == 0) out[row] = besti < vocab ? besti : 0;
+}
+
+// Chunks a row of `vocab` columns is scanned in: about a thousand columns each, 128 at most.
+extern "C" int tl_sample_chunks(int vocab) {
+    const int c = (vocab + 1023) / 1024;
+    return c < 1 ? 1 : (c > 128 ? 128 : c);
+}
+
 // temperature: float[rows] or null (all greedy); keys: int32[rows] bit patterns or null.
+// scratch: rows * tl_sample_chunks(vocab) * 8 bytes, 4-byte aligned.
 extern "C" int tl_sample(const void* logits, int rows, int vocab, int ld, const void* temperature,
-                         const void* keys, void* out, hipStream_t stream) {
+                         const void* keys, void* out, void* scratch, hipStream_t stream) {
     TL_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "sample: bad sizes rows=%d vocab=%d ld=%d", rows, vocab, ld);
+    TL_REQUIRE(scratch != nullptr || rows == 0, "sample: no scratch buffer");
     if (rows == 0) return TL_OK;
-    sample_kernel<<<dim3(rows), dim3(1024), 0, stream>>>((const float*)logits, vocab, ld, (const float*)temperature,
-                                                         (const int*)keys, (int*)out);
-    TL_CHECK_LAUNCH("sample");
+    const int chunks = tl_sample_chunks(vocab);
+    const int per = (vocab + chunks - 1) / chunks;
+    float* part_v = (float*)scratch;
+    int* part_i = (int*)scratch + (size_t)rows * chunks;
+    sample_scan_kernel<<<dim3(chunks, rows), dim3(SAMPLE_THREADS), 0, stream>>>((const float*)logits, vocab, ld, per,
+        (const float*)temperature, (const int*)keys, part_v, part_i);
+    TL_CHECK_LAUNCH("sample_scan");
+    sample_pick_kernel<<<dim3(rows), dim3(TL_WAVE), 0, stream>>>(part_v, part_i, chunks, vocab, (int*)out);
+    TL_CHECK_LAUNCH("sample_pick");
     return TL_OK;
 }

@@ -379,5 +379,6 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor | None, keys: torch.T
     _i32(keys, "sample keys", N)
     _i32(out, "sample out", N)
     lib = _lib("sampling")
+    scratch = torch.empty((2, N, lib.tl_sample_chunks(c_int(V))), dtype=torch.int32, device=logits.device)
     _check(lib, lib.tl_sample(_ptr(logits), c_int(N), c_int(V), c_int(logits.stride(0)), _ptr(temperature), _ptr(keys),
-                              _ptr(out), _stream()))
+                              _ptr(out), _ptr(scratch), _stream()))

@@ -195,6 +195,28 @@ def test_linear_many_rows_on_matrix_cores(ops, out_dtype, tile, M, N, K):
     torch.testing.assert_close(out2.double(), ref - b.double(), **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("tile", [(64, 64), (64, 256), (128, 128), (128, 256), (256, 128), (256, 256)])
+@pytest.mark.parametrize("M,N,K", [(65, 129, 64), (300, 520, 192), (1000, 257, 1024), (33, 48, 3584), (40, 4608, 128), (513, 700, 320)])
+def test_linear_many_rows_fetched_straight_into_shared_memory(ops, out_dtype, tile, M, N, K):
+    """Every tile shape of the direct-load matrix-core kernel, with tails in M and N, one slab to
+    many (fewer slabs than pipeline stages too), a bias, a strided x."""
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).cuda()
+    b = torch.randn(N, generator=g).to(torch.bfloat16).cuda()
+    ref = x.double() @ w.double().T + b.double()
+    out = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
+    ops.linear_direct_variant(x, w, b, out, *tile)
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    torch.testing.assert_close(out.double(), ref, **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
+    wide = torch.zeros(M, K + 40, dtype=torch.bfloat16, device="cuda")
+    wide[:, 16:16 + K] = x
+    out2 = torch.empty_like(out)
+    ops.linear_direct_variant(wide[:, 16:16 + K], w, None, out2, *tile)
+    torch.testing.assert_close(out2.double(), ref - b.double(), **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 32, 33, 64, 65, 300])
 @pytest.mark.parametrize("I,K", [(128, 64), (200, 96), (112, 80), (18944, 256), (32768 + 40, 64)])
 def test_linear_swiglu_fused(ops, M, I, K):

@@ -724,6 +724,230 @@ static int launch_mfma_tile(const void* x, const void* w, const void* bias, int 
     return launch_mfma_tile_t<BM, BN, WGM, WGN, bf16_t, false, TK>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
 }
 
+// =====================================================================================
+// The same product with the operands fetched straight into shared memory (K a multiple of 64).
+//
+// global_load_lds_dwordx4 moves 16 bytes per lane from memory into shared memory without passing
+// through registers: one instruction of a wave fills 1 KB, eight rows of a 64-element slab.  A slab
+// row is 128 bytes with no padding; piece c (16 bytes) of row r lies in slot c ^ ((r >> 1) & 7), so
+// that the sixteen rows a quarter-wave reads for one MFMA operand fall on all 64 banks (measured:
+// no bank conflicts).  The lane that fills slot s of row r therefore fetches piece s ^ ((r >> 1) & 7)
+// of that row from memory.  STAGES slabs are in flight or in use: the slab STAGES - 1 ahead is
+// requested at the top of a step into the buffer that the previous step has finished with, and a
+// step ends with a wait for this wave's requests of the next slab and one barrier.
+// The requests are issued as assembly: the compiler orders every later shared-memory read behind
+// a direct load it knows of (a full wait per slab), so the kernel keeps that order itself.
+__device__ __forceinline__ void load_to_lds(const void* gptr, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW = false>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                      const void* __restrict__ bias, int bias_f32,
+                                                                      TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
+                                                                      int out_cols) {
+    static_assert(!SW || (BN / WGN) % 64 == 0, "the fused gate needs whole 64-row blocks per wave");
+    constexpr int TK = 64;
+    constexpr int NW = WGM * WGN;
+    constexpr int WM = BM / WGM, WN = BN / WGN;          // wave tile
+    constexpr int FM = WM / 32, FN = WN / 32;            // 32x32 blocks per wave
+    constexpr int ROWS = BM + BN;
+    constexpr int LOADS = ROWS / 8 / NW;                 // load instructions per wave and slab (8 rows each)
+    static_assert(ROWS % (8 * NW) == 0, "slab rows must divide over the waves");
+    static_assert(LOADS * (STAGES - 2) < 64, "outstanding loads must fit the counter");
+    extern __shared__ __attribute__((aligned(16))) bf16_t lds_raw[];   // [STAGES][ROWS][64]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    // tile order as in gemm_mfma_tile_kernel: each XCD walks 8 x 8 blocks of tiles out of its own L2
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    int lid;
+    {
+        const int total = gridDim.x, xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
+        lid = xcd * (total / 8) + min(xcd, total % 8) + idx;
+    }
+    int tm, tn;
+    {
+        const int per_group = 8 * tiles_n;
+        const int first_m = (lid / per_group) * 8;
+        const int rows = min(tiles_m - first_m, 8);
+        tm = first_m + (lid % per_group) % rows;
+        tn = (lid % per_group) / rows;
+    }
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // instruction j of this wave fills rows 8 (wave + j NW) .. + 8 of the stacked [x rows; w rows] slab
+    const bf16_t* src[LOADS];
+    int ldst[LOADS];
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) {
+        const int base_row = 8 * (wave + j * NW);
+        const int row = base_row + (lane >> 3);
+        const int c = (lane & 7) ^ ((row >> 1) & 7);
+        if (row < BM) src[j] = x + (size_t)min(m0 + row, M - 1) * ldx + c * 8;
+        else src[j] = w + (size_t)min(n0 + row - BM, N - 1) * K + c * 8;
+        ldst[j] = __builtin_amdgcn_readfirstlane(base_row * TK * 2);
+    }
+    const unsigned lds_base = (unsigned)(uintptr_t)((void __attribute__((address_space(3)))*)lds_raw);
+
+    f32x16_t acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    const int slabs = K / TK;
+#pragma unroll
+    for (int st = 0; st < STAGES - 1; ++st) {
+        const int k0 = min(st, slabs - 1) * TK;
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j) load_to_lds(src[j] + k0, lds_base + st * ROWS * TK * 2 + ldst[j]);
+    }
+    wait_direct_loads<(STAGES - 2) * LOADS>();
+    __syncthreads();
+
+    const int fr = lane & 31, fh = lane >> 5;
+    int arow[FM], brow[FN], akey[FM], bkey[FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) { arow[i] = wm * WM + i * 32 + fr; akey[i] = (arow[i] >> 1) & 7; }
+#pragma unroll
+    for (int j = 0; j < FN; ++j) { brow[j] = BM + wn * WN + j * 32 + fr; bkey[j] = (brow[j] >> 1) & 7; }
+
+    for (int sl = 0; sl < slabs; ++sl) {
+        {   // past the end the last slab is requested again (nobody reads it): the count of requests
+            // in flight stays the same in every step, which the wait below relies on
+            const int k0 = min(sl + STAGES - 1, slabs - 1) * TK;
+            const unsigned nb = lds_base + ((sl + STAGES - 1) % STAGES) * ROWS * TK * 2;
+#pragma unroll
+            for (int j = 0; j < LOADS; ++j) load_to_lds(src[j] + k0, nb + ldst[j]);
+        }
+        const bf16_t* cb = lds_raw + (sl % STAGES) * ROWS * TK;
+        Frag16 af[2][FM], bfr[2][FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i) af[0][i].u = *(const uint4*)(cb + arow[i] * TK + ((fh ^ akey[i]) * 8));
+#pragma unroll
+        for (int j = 0; j < FN; ++j) bfr[0][j].u = *(const uint4*)(cb + brow[j] * TK + ((fh ^ bkey[j]) * 8));
+#pragma unroll
+        for (int kk = 0; kk < TK / 16; ++kk) {
+            if (kk + 1 < TK / 16) {
+                const int c = 2 * (kk + 1) + fh;
+#pragma unroll
+                for (int i = 0; i < FM; ++i) af[(kk + 1) & 1][i].u = *(const uint4*)(cb + arow[i] * TK + ((c ^ akey[i]) * 8));
+#pragma unroll
+                for (int j = 0; j < FN; ++j) bfr[(kk + 1) & 1][j].u = *(const uint4*)(cb + brow[j] * TK + ((c ^ bkey[j]) * 8));
+            }
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i].v, bfr[kk & 1][j].v, acc[i][j], 0, 0, 0);
+            if (kk + 1 < TK / 16) {      // one operand read of the next step between the products of this one
+#pragma unroll
+                for (int q = 0; q < FM + FN; ++q) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                if (FM * FN > FM + FN) __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - (FM + FN), 0);
+            }
+        }
+        wait_direct_loads<(STAGES - 2) * LOADS>();
+        __syncthreads();
+    }
+    wait_direct_loads<0>();
+
+    // block result: lane holds column (lane % 32), rows 8 * (v / 4) + 4 * (lane / 32) + v % 4
+    if (SW) {   // even blocks hold gate columns, the next block the up columns of the same outputs
+#pragma unroll
+        for (int j = 0; j + 1 < FN; j += 2) {
+            const int col = (n0 + wn * WN + j * 32) / 2 + (lane & 31);
+            if (col >= out_cols) continue;
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                    if (m < M) out[(size_t)m * ldo + col] = from_float<TOut>(silu_mul(acc[i][j][v], acc[i][j + 1][v]));
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+        const int n = n0 + wn * WN + j * 32 + (lane & 31);
+        if (n >= N) continue;
+        const float b = bias ? load_vec(bias, bias_f32, n) : 0.f;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                if (m < M) out[(size_t)m * ldo + n] = from_float<TOut>(acc[i][j][v] + b);
+            }
+        }
+    }
+}
+
+// Tile shapes of the direct-load kernel and which one a product gets.  Estimate per shape: the
+// tiles are dealt to 256 compute units, each works through ceil(tiles / 256) of them one after
+// the other at the rate the shape reaches on a full machine (measured at Qwen2.5-7B sizes,
+// TFLOP/s: 64x64 700, 64x256 800, 128x128 900, 128x256 950, 256x128 1000, 256x256 1100), plus
+// about 2 us per tile for filling the pipeline and storing the result.
+enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_256x256, DL_TILES };
+static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 256};
+static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256};
+static const double DL_RATE[DL_TILES] = {700e12, 800e12, 900e12, 950e12, 1000e12, 1100e12};
+
+static DlTile pick_dl_tile(int M, int N, int K, bool sw) {
+    DlTile best = DL_128x128;
+    double best_t = 1e30;
+    for (int t = 0; t < DL_TILES; ++t) {
+        if (sw && t == DL_64x64) continue;               // a wave of the fused gate needs 64 weight rows
+        const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
+        const double per_tile = 2.0 * DL_BM[t] * DL_BN[t] * K / (DL_RATE[t] / 256) + 2e-6;
+        const double est = (double)((tiles + 255) / 256) * per_tile;
+        if (est < best_t) { best_t = est; best = (DlTile)t; }
+    }
+    return best;
+}
+
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW>
+static int launch_dl_tile_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                            int ldx, int ldo, int out_cols, hipStream_t stream) {
+    constexpr size_t lds = (size_t)STAGES * (BM + BN) * 64 * sizeof(bf16_t);
+    auto kernel = gemm_dl_tile_kernel<BM, BN, WGM, WGN, STAGES, TOut, SW>;
+    static hipError_t allowed = allow_lds(kernel, lds);
+    if (allowed != hipSuccess) {
+        tl_set_error("gemm_dl_tile: cannot get %zu bytes of shared memory: %s", lds, hipGetErrorString(allowed));
+        return TL_ERR_HIP;
+    }
+    dim3 grid(((M + BM - 1) / BM) * ((N + BN - 1) / BN)), block(64 * WGM * WGN);
+    kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols);
+    return TL_OK;
+}
+
+template <typename TOut, bool SW>
+static int launch_dl_tile(DlTile tile, const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                          int ldx, int ldo, int out_cols, hipStream_t stream) {
+    switch (tile) {
+    case DL_64x64:
+        if constexpr (!SW) return launch_dl_tile_t<64, 64, 2, 2, 4, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+        else break;
+    case DL_64x256: return launch_dl_tile_t<64, 256, 1, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    case DL_128x128: return launch_dl_tile_t<128, 128, 2, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    case DL_128x256: return launch_dl_tile_t<128, 256, 2, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    case DL_256x128: return launch_dl_tile_t<256, 128, 4, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    case DL_256x256: return launch_dl_tile_t<256, 256, 4, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    default: break;
+    }
+    tl_set_error("gemm_dl_tile: no instance of tile %d", (int)tile);
+    return TL_ERR_ARG;
+}
+
 // One named tile shape of the many-rows kernel (tests cover each; tuning times them).
 extern "C" int tl_gemm_tile_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
                                     int M, int N, int K, int ldx, int ldo, int out_f32, int BM, int BN, int TK, hipStream_t stream) {
@@ -743,6 +967,22 @@ extern "C" int tl_gemm_tile_variant(const void* x, const void* w, const void* bi
     return TL_OK;
 }
 
+// One named tile shape of the direct-load kernel (tests cover each; tuning times them).
+extern "C" int tl_gemm_direct_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
+                                      int M, int N, int K, int ldx, int ldo, int out_f32, int BM, int BN, hipStream_t stream) {
+    TL_REQUIRE(M > 0 && K % 64 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
+               "gemm_direct: needs M > 0, K a multiple of 64 and 16-byte aligned rows");
+    int tile = -1;
+    for (int t = 0; t < DL_TILES; ++t)
+        if (DL_BM[t] == BM && DL_BN[t] == BN) tile = t;
+    TL_REQUIRE(tile >= 0, "gemm_direct: no tile of %d x %d", BM, BN);
+    const int rc = out_f32 ? launch_dl_tile<float, false>((DlTile)tile, x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream)
+                           : launch_dl_tile<bf16_t, false>((DlTile)tile, x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
+    if (rc != TL_OK) return rc;
+    TL_CHECK_LAUNCH("gemm_dl_tile");
+    return TL_OK;
+}
+
 static bool skinny_fits(const void* x, const void* w, int M, int K, int ldx) {
     return M <= 64 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
 }
@@ -750,6 +990,8 @@ static bool skinny_fits(const void* x, const void* w, int M, int K, int ldx) {
 // out = x w^T (+ bias) in the engine's dtype: picks the kernel for the shape.
 //   bfloat16, aligned, M <= 64  -> gemm_skinny (matrix cores, weight streaming), except that
 //                                  33..64 rows against a wide matrix go to the tile kernel
+//   bfloat16, aligned, M > 32, K a multiple of 64 -> gemm_dl_tile (matrix cores, operands straight
+//                                  into shared memory)
 //   bfloat16, aligned, M > 64   -> gemm_mfma_tile (matrix cores, shared-memory tiles)
 //   everything else             -> gemm_tile (true 32-bit arithmetic)
 extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_f32, void* out,
@@ -757,6 +999,13 @@ extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_
     TL_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldo >= N, "gemm: bad sizes M=%d N=%d K=%d ldx=%d ldo=%d", M, N, K, ldx, ldo);
     if (M == 0) return TL_OK;
     const bool aligned = K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
+    if (dtype == TL_DT_BF16 && aligned && K % 64 == 0 && M > 32) {
+        int rc = out_f32 ? launch_dl_tile<float, false>(pick_dl_tile(M, N, K, false), x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream)
+                         : launch_dl_tile<bf16_t, false>(pick_dl_tile(M, N, K, false), x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
+        if (rc != TL_OK) return rc;
+        TL_CHECK_LAUNCH("gemm_dl_tile");
+        return TL_OK;
+    }
     if (dtype == TL_DT_BF16 && aligned && (M > 64 || (M > 32 && N >= 16384))) {
         int rc;
         switch (pick_tile(M, N)) {
@@ -797,6 +1046,9 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
     if (M <= 32) {
         if (M <= 16) launch_skinny_t<4, 1, 4, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
         else launch_skinny_t<4, 2, 4, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
+    } else if (K % 64 == 0) {
+        const int rc = launch_dl_tile<bf16_t, true>(pick_dl_tile(M, N, K, true), xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
+        if (rc != TL_OK) return rc;
     } else {
         int rc;
         switch (pick_tile(M, N)) {

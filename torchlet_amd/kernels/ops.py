@@ -215,6 +215,23 @@ def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int, sla
                                          c_int(1 if out.dtype == torch.float32 else 0), c_int(tile_m), c_int(tile_n), c_int(slab), _stream()))
 
 
+DIRECT_TILES = ((64, 64), (64, 256), (128, 128), (128, 256), (256, 128), (256, 256))
+
+
+def linear_direct_variant(x, weight, bias, out, tile_m: int, tile_n: int) -> None:
+    """One named tile shape of the many-rows kernel that fetches its operands straight into
+    shared memory (K a multiple of 64; for tests and tuning)."""
+    M, K = x.shape
+    N = weight.shape[0]
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or out.shape != (M, N) or not weight.is_contiguous():
+        raise KernelError("linear_direct_variant: bfloat16 operands and fitting shapes only")
+    bf = _vec(bias, N, "linear bias")
+    lib = _lib("gemm")
+    _check(lib, lib.tl_gemm_direct_variant(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N),
+                                           c_int(K), c_int(x.stride(0)), c_int(out.stride(0)),
+                                           c_int(1 if out.dtype == torch.float32 else 0), c_int(tile_m), c_int(tile_n), _stream()))
+
+
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """The layout :func:`linear_swiglu` wants: blocks of 64 rows, 32 rows of ``gate`` then the
     32 rows of ``up`` with the same indices; the last block is padded with zero rows."""

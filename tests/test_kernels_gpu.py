@@ -403,6 +403,58 @@ def test_paged_attention_prompt_portions(ops, nh, nkv, hd, page, window):
         torch.testing.assert_close(got[a:b], ref, **tol)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page,window", [
+    (28, 4, 128, 16, 0), (20, 1, 64, 16, 0), (40, 8, 128, 8, 0), (4, 4, 64, 32, 0), (130, 1, 64, 16, 0),
+    (14, 2, 128, 64, 40), (4, 4, 64, 32, 29), (6, 2, 128, 24, 100),
+])
+def test_paged_attention_prompt_tiles_of_128_rows(ops, nh, nkv, hd, page, window):
+    """The 128-row kernel for prompt portions: whole prompts, portions on top of a cached context
+    (also one that starts inside a page and inside a step of 64 keys), a single token, groups of
+    1, 3, 5, 7, 20 and 130 heads.  Places of the pages that hold no key yet are filled with NaN:
+    nothing of them may reach a result."""
+    assert ops.prompt_attention_fits(torch.bfloat16, hd, page)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(15)
+    lens, ctxs = [150, 37, 70, 1, 64, 300], [0, 150, 43, 99, 64, 5]
+    R, T = len(lens), sum(lens)
+    totals = [a + b for a, b in zip(lens, ctxs)]
+    max_blocks = (max(totals) + page - 1) // page + 1
+    pages = R * max_blocks + 1
+    bt = (torch.randperm(pages - 1, generator=g)[: R * max_blocks] + 1).view(R, max_blocks).int()
+    q = torch.randn(T, nh * hd, generator=g).to(dtype)
+    kp = torch.full((pages, nkv, page, hd), float("nan"), dtype=dtype)
+    vp = torch.full((pages, nkv, hd, page), float("nan"), dtype=dtype)
+    ks, vs = [], []
+    for r in range(R):
+        k = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
+        v = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
+        k[min(3, totals[r] - 1)] *= 3.0
+        for p in range(totals[r]):
+            kp[bt[r, p // page], :, p % page] = k[p]
+            vp[bt[r, p // page], :, :, p % page] = v[p]
+        ks.append(k); vs.append(v)
+    indptr = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    tq = ops.prompt_attention_tile_tokens(nh, nkv)
+    tile_req, tile_tok0 = [], []
+    for r, n in enumerate(lens):
+        for t0 in range(0, n, tq):
+            tile_req.append(r); tile_tok0.append(t0)
+    out = torch.full((T, nh * hd), float("nan"), dtype=dtype, device="cuda")
+    wide = torch.zeros(T, nh * hd + 32, dtype=dtype, device="cuda")
+    wide[:, : nh * hd] = q.cuda()
+    ops.paged_attention_prompt(wide[:, : nh * hd], out, kp.cuda(), vp.cuda(), bt.cuda(), indptr.cuda(),
+                               torch.tensor(ctxs, dtype=torch.int32).cuda(), torch.tensor(tile_req, dtype=torch.int32).cuda(),
+                               torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq, nh, nkv, hd, page, window,
+                               1.0 / math.sqrt(hd))
+    got = out.cpu().double().view(T, nh, hd)
+    for r in range(R):
+        a, b = int(indptr[r]), int(indptr[r + 1])
+        ref = _attention_ref(q[a:b].double().view(-1, nh, hd), ks[r].double(), vs[r].double(), window)
+        tol = _tol(dtype)
+        tol = dict(rtol=tol["rtol"], atol=tol["atol"] + 2 ** -9 * float(vs[r].abs().max()))
+        torch.testing.assert_close(got[a:b], ref, **tol)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,I", [(3, 200), (17, 1001)])
 def test_swiglu(ops, dtype, T, I):

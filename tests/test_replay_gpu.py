@@ -16,7 +16,8 @@ import tiny_models
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
 
-LENGTHS = {"A": [70, 33, 97, 5, 120, 64], "B": [40, 129, 9, 64, 200, 1 + 32], "C": [150, 61, 33, 90, 47, 128]}
+LENGTHS = {"A": [70, 33, 97, 5, 120, 64], "B": [40, 129, 9, 64, 200, 1 + 32], "C": [150, 61, 33, 90, 47, 128],
+           "D": [260, 77, 140, 33, 200, 64]}
 TOL = {"float32": scenarios.FP32_TOL, "bfloat16": scenarios.BF16_TOL}
 
 
@@ -52,7 +53,7 @@ def expected(model_folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 @pytest.mark.parametrize("mode", ["whole", "tail_singles", "portions", "mixed"])
 def test_split(model_folders, expected, name, dtype, mode):
     reqs, exp = expected(name)

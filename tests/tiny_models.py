@@ -1,8 +1,10 @@
 """Tiny random-weight model folders for the tests.
 
-Three configurations of the one architecture that differ in every size and option:
+Four configurations of the one architecture that differ in every size and option:
 A and B are the two tiny workloads the benchmark contract names; C adds what they leave
-out (no QKV bias, one KV head per query head, a window on the later layers).
+out (no QKV bias, one KV head per query head, a window on the later layers); D has heads of
+64 (the size from which the 128-row prompt attention kernel is built), groups of three, a
+window wider than a step of keys and pages of 8.
 """
 import json
 from pathlib import Path
@@ -27,9 +29,15 @@ CONFIGS = {
         attention_bias=False, tie_word_embeddings=False,
         use_sliding_window=True, sliding_window=20, max_window_layers=1,
     ),
+    "D": dict(
+        architectures=["Qwen2ForCausalLM"], vocab_size=190, hidden_size=72, num_hidden_layers=2,
+        num_attention_heads=6, num_key_value_heads=2, head_dim=64, intermediate_size=104,
+        max_position_embeddings=400, rope_theta=30000.0, rms_norm_eps=2e-6, tie_word_embeddings=True,
+        use_sliding_window=True, sliding_window=70, max_window_layers=1,
+    ),
 }
-SEEDS = {"A": 0, "B": 1, "C": 5}
-PAGE_SIZES = {"A": 16, "B": 8, "C": 16}
+SEEDS = {"A": 0, "B": 1, "C": 5, "D": 8}
+PAGE_SIZES = {"A": 16, "B": 8, "C": 16, "D": 8}
 
 
 def write(name: str, root: Path, dtype=torch.bfloat16) -> Path:

@@ -735,6 +735,303 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
     out[r * AT_HD + d] = from_float<T>(num / denom);
 }
 
+// =====================================================================================
+// Prompt portions, 128 rows per work-group (bfloat16, head size 64 or 128, pages of a multiple
+// of 8 tokens).
+//
+// Four waves of 32 rows share steps of 64 keys.  Keys and transposed values of a step go from
+// the pages straight into shared memory (global_load_lds_dwordx4, two buffers: the next step is
+// on its way while this one is multiplied), in 16-byte pieces whose slot within a row is
+// exclusive-ored with the row number, so that the operand reads of sixteen neighbouring rows
+// fall on all banks.  Both products run transposed on v_mfma_f32_32x32x16_bf16:
+//   S^T[key, row] = K[key, :] . Q[row, :]      A = 32 keys x 16 d from shared memory, B = Q (registers)
+//   O^T[d, row]  += V^T[d, key] . P^T[key, row] A = 32 d x 16 keys from shared memory, B = P (registers)
+// so a lane owns ONE query row (its column, lane % 32): maximum, sum and the rescaling of the
+// accumulator are lane-local but for one exchange with lane ^ 32.  Which key an A row of the
+// first product carries is free; row 8 q + 4 h + v carries key 16 (q / 2) + 8 h + 4 (q % 2) + v of
+// its block of 32, which makes the eight probabilities a lane holds for a 16-key chunk exactly
+// the B operand of the second product, with no exchange between lanes.
+#if AT_HD == 64 || AT_HD == 128
+#define ATQ_ROWS 128
+#define ATQ_KEYS 64
+#define ATQ_KBYTES (ATQ_KEYS * AT_HD * 2)
+#define ATQ_STAGE (2 * ATQ_KBYTES)                 // keys, then values
+#define ATQ_SMEM (2 * ATQ_STAGE + ATM_BT_MAX * 4)
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+// 16 bytes per lane from memory straight into shared memory at lds_addr + 16 * lane.  Issued as
+// assembly: the compiler would make every later shared-memory read wait for a direct load it
+// knows of; the kernel waits itself (vmcnt) before the barrier that publishes a step.
+__device__ __forceinline__ void attn_load_to_lds(const void* gptr, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+
+__device__ __forceinline__ int atq_key_slot(int piece, int key) {        // slot of a 16-byte piece in its key row
+    return AT_HD == 128 ? (piece ^ (key & 15)) : (piece ^ ((key >> 1) & 7));
+}
+
+__global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char atq_smem[];
+    int* bt_s = (int*)(atq_smem + 2 * ATQ_STAGE);
+    const unsigned lds_base = (unsigned)(uintptr_t)((void __attribute__((address_space(3)))*)atq_smem);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lr = lane & 31, h = lane >> 5;
+
+    const int tile = gridDim.x - 1 - blockIdx.x;            // late tiles see the most keys: they start first
+    const int group = a.heads / a.kv_heads;
+    const int chunks_h = (group + a.gcap - 1) / a.gcap;
+    const int kvh = blockIdx.y / chunks_h;
+    const int g0 = (blockIdx.y % chunks_h) * a.gcap;
+    const int gcount = min(a.gcap, group - g0);
+
+    const int req = a.tile_req[tile];
+    const int tok0 = a.tile_tok0[tile];
+    const int first = a.req_indptr[req];
+    const int n_new = a.req_indptr[req + 1] - first;
+    const int ctx = a.ctx_lens[req];
+    const int ntok = min(a.tq, n_new - tok0);
+
+    const int row = wave * 32 + lr;
+    const int r_tok = row / a.gcap, r_g = row % a.gcap;
+    const bool row_ok = r_tok < ntok && r_g < gcount;
+    const int r_pos = ctx + tok0 + r_tok;
+    const int r_lo = a.window > 0 ? r_pos - a.window + 1 : 0;
+    const int r_head = kvh * group + g0 + r_g;
+    const int r_token = first + tok0 + r_tok;
+
+    // the wave's rows: smallest and largest position, largest window start (uniform)
+    const int w_tok_lo = min((wave * 32) / a.gcap, ntok - 1), w_tok_hi = min((wave * 32 + 31) / a.gcap, ntok - 1);
+    const bool wave_has_rows = (wave * 32) / a.gcap < ntok;
+    const int w_pos_min = ctx + tok0 + w_tok_lo, w_pos_max = ctx + tok0 + w_tok_hi;
+    const int w_lo_min = a.window > 0 ? max(0, w_pos_min - a.window + 1) : 0;
+    const int w_lo_max = a.window > 0 ? max(0, w_pos_max - a.window + 1) : 0;
+
+    // my row's query, B operand of the first product: d = 16 c + 8 h .. + 8
+    FragK qf[AT_HD / 16];
+    {
+        const bf16_t* q = (const bf16_t*)a.q + (size_t)r_token * a.q_stride + (size_t)r_head * AT_HD;
+#pragma unroll
+        for (int c = 0; c < AT_HD / 16; ++c) qf[c].u = row_ok ? *(const uint4*)(q + 16 * c + 8 * h) : make_uint4(0, 0, 0, 0);
+    }
+
+    const int key_hi = ctx + tok0 + ntok;
+    const int key_lo = a.window > 0 ? max(0, ctx + tok0 - a.window + 1) : 0;
+    const int st_first = key_lo / ATQ_KEYS, st_last = (key_hi + ATQ_KEYS - 1) / ATQ_KEYS;
+
+    const bf16_t* kp = (const bf16_t*)a.k_plane;
+    const bf16_t* vp = (const bf16_t*)a.v_plane;
+    const int page = a.page;
+    const size_t kv_stride = (size_t)a.kv_heads * page * AT_HD;
+    const int kvh_off = kvh * page * AT_HD;
+    const int* bt_g = a.block_table + (size_t)req * a.bt_stride;
+    const int blk0 = (st_first * ATQ_KEYS) / page;
+    const int blk_n = (key_hi - 1) / page - blk0 + 1;
+    const bool bt_local = blk_n <= ATM_BT_MAX;
+    if (bt_local) {
+        for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
+        __syncthreads();
+    }
+#define ATQ_PAGE_OF(blk) (bt_local ? bt_s[(blk) - blk0] : bt_g[(blk)])
+
+    // requests of one step: K rows of AT_HD * 2 bytes, then V^T rows of 128 bytes (64 keys)
+    constexpr int KPI = 1024 / (AT_HD * 2);                 // keys per load instruction (4 or 8)
+    constexpr int KPP = AT_HD / 8;                          // pieces per key row (16 or 8)
+    constexpr int K_INSTR = ATQ_KBYTES / 1024 / 4;          // per wave
+    auto request_step = [&](int st, int buf) {
+        const int kbase = st * ATQ_KEYS;
+        const unsigned sb = lds_base + buf * ATQ_STAGE;
+#pragma unroll
+        for (int j = 0; j < K_INSTR; ++j) {
+            const int ii = __builtin_amdgcn_readfirstlane(wave + 4 * j);
+            const int kl = KPI * ii + lane / KPP;            // key within the step
+            const int piece = atq_key_slot(lane % KPP, kl);  // exclusive-or is its own inverse
+            int blk, off;
+            split_key(min(kbase + kl, key_hi - 1), page, a.page_shift, blk, off);
+            attn_load_to_lds(kp + ((size_t)ATQ_PAGE_OF(blk) * kv_stride + kvh_off + off * AT_HD + piece * 8), sb + ii * 1024);
+        }
+#pragma unroll
+        for (int j = 0; j < K_INSTR; ++j) {
+            const int ii = __builtin_amdgcn_readfirstlane(wave + 4 * j);
+            const int d = 8 * ii + (lane >> 3);
+            const int piece = (lane & 7) ^ ((d >> 1) & 7);   // keys 8 piece .. + 8 of the step
+            int blk, off;
+            split_key(min(kbase + 8 * piece, (key_hi - 1) & ~7), page, a.page_shift, blk, off);
+            attn_load_to_lds(vp + ((size_t)ATQ_PAGE_OF(blk) * kv_stride + kvh_off + (size_t)d * page + off), sb + ATQ_KBYTES + ii * 1024);
+        }
+    };
+
+    const float scale2 = a.scale * 1.44269504088896341f;
+    float m = -INFINITY, l = 0.f;
+    f32x16_t acc[AT_HD / 32];
+#pragma unroll
+    for (int b = 0; b < AT_HD / 32; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+
+    // key (within its block of 32) that A row lr of the first product carries
+    const int krow = 16 * (lr >> 4) + 8 * ((lr >> 2) & 1) + 4 * ((lr >> 3) & 1) + (lr & 3);
+
+    if (st_first < st_last) request_step(st_first, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int st = st_first; st < st_last; ++st) {
+        const int buf = (st - st_first) & 1;
+        if (st + 1 < st_last) request_step(st + 1, buf ^ 1);
+        const int kbase = st * ATQ_KEYS;
+        unsigned char* kb_s = atq_smem + buf * ATQ_STAGE;
+        unsigned char* vb_s = kb_s + ATQ_KBYTES;
+        if (kbase + ATQ_KEYS > key_hi) {
+            // the last step holds keys that are not written yet: whatever lies in their places in
+            // the pages must not reach the second product (0 * Inf), so their values become zero
+            for (int i = threadIdx.x; i < AT_HD * 8; i += 256) {
+                const int d = i >> 3, piece = i & 7;
+                const int k0 = kbase + 8 * piece;
+                if (k0 + 8 > key_hi) {
+                    FragK f;
+                    uint4* ptr = (uint4*)(vb_s + d * 128 + ((piece ^ ((d >> 1) & 7)) * 16));
+                    f.u = *ptr;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (k0 + e >= key_hi) f.v[e] = (__bf16)0.f;
+                    *ptr = f.u;
+                }
+            }
+            __syncthreads();
+        }
+        if (wave_has_rows && kbase <= w_pos_max && kbase + ATQ_KEYS > w_lo_min) {
+            // ---- scores of two blocks of 32 keys
+            f32x16_t sc[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) sc[kb][v] = 0.f;
+                const int kl = 32 * kb + krow;
+#pragma unroll
+                for (int c = 0; c < AT_HD / 16; ++c) {
+                    FragK kf;
+                    kf.u = *(const uint4*)(kb_s + kl * (AT_HD * 2) + atq_key_slot(2 * c + h, kl) * 16);
+                    sc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[c].v, sc[kb], 0, 0, 0);
+                }
+            }
+            // ---- mask, maximum, probabilities.  Element (kb, 4 q + v) of this lane is key
+            // kbase + 32 kb + 16 (q / 2) + 8 h + 4 (q % 2) + v of row lr.
+            float mloc = -INFINITY;
+            if (kbase + ATQ_KEYS - 1 <= w_pos_min && kbase >= w_lo_max) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        sc[kb][v] *= scale2;
+                        mloc = fmaxf(mloc, sc[kb][v]);
+                    }
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int q = e >> 2, v = e & 3;
+                        const int key = kbase + 32 * kb + 16 * (q >> 1) + 8 * h + 4 * (q & 1) + v;
+                        const bool seen = row_ok && key <= r_pos && key >= r_lo;
+                        sc[kb][e] = seen ? sc[kb][e] * scale2 : -INFINITY;
+                        mloc = fmaxf(mloc, sc[kb][e]);
+                    }
+            }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TL_WAVE));
+            const float m_new = fmaxf(m, mloc);
+            const float alpha = (m == -INFINITY) ? 0.f : fast_exp2(m - m_new);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;     // nothing seen yet: every score is -inf
+            FragK pf[4];
+            float psum = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float p = fast_exp2(sc[kb][e] - m_use);
+                    psum += p;
+                    pf[2 * kb + (e >> 3)].v[e & 7] = (__bf16)p;
+                }
+            l = l * alpha + psum;
+            const bool moved = __any(m_new != m);
+            m = m_new;
+            if (moved) {
+#pragma unroll
+                for (int b = 0; b < AT_HD / 32; ++b) acc[b] *= alpha;
+            }
+            // ---- values
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4)
+#pragma unroll
+                for (int b = 0; b < AT_HD / 32; ++b) {
+                    const int d = 32 * b + lr;
+                    FragK vf;
+                    vf.u = *(const uint4*)(vb_s + d * 128 + (((2 * c4 + h) ^ ((d >> 1) & 7)) * 16));
+                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[c4].v, acc[b], 0, 0, 0);
+                }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+#undef ATQ_PAGE_OF
+    l += __shfl_xor(l, 32, TL_WAVE);
+    if (!row_ok) return;
+    // lane holds d = 32 b + 8 q + 4 h + v of its row
+    bf16_t* o = (bf16_t*)a.out + (size_t)r_token * a.heads * AT_HD + (size_t)r_head * AT_HD;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int b = 0; b < AT_HD / 32; ++b)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            union { uint2 u; uint16_t e[4]; } pk;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(acc[b][4 * q + v] * inv).bits;
+            *(uint2*)(o + 32 * b + 8 * q + 4 * h) = pk.u;
+        }
+}
+#endif
+
+// The 128-row prompt kernel: tiles of `tq` tokens with tq * min(group, 128) <= 128.  Returns an
+// error where it is not built (head sizes other than 64 and 128, pages not a multiple of 8).
+extern "C" int tl_paged_attention_prompt_rows() {
+#if AT_HD == 64 || AT_HD == 128
+    return ATQ_ROWS;
+#else
+    return 0;
+#endif
+}
+
+extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out, const void* k_plane, const void* v_plane,
+                                         const void* block_table, int bt_stride, const void* req_indptr, const void* ctx_lens,
+                                         const void* tile_req, const void* tile_tok0, int tiles, int tq,
+                                         int heads, int kv_heads, int page, int window, float scale, hipStream_t stream) {
+#if AT_HD == 64 || AT_HD == 128
+    TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
+    TL_REQUIRE(page > 0 && page % 8 == 0 && bt_stride > 0 && tq > 0 && window >= 0, "attention_prompt: pages of a multiple of 8 tokens, not %d", page);
+    const int group = heads / kv_heads;
+    const int gcap = group < ATQ_ROWS ? group : ATQ_ROWS;
+    TL_REQUIRE(tq * gcap <= ATQ_ROWS, "attention_prompt: tile of %d tokens x %d heads exceeds %d rows", tq, gcap, ATQ_ROWS);
+    TL_REQUIRE(q_stride >= heads * AT_HD && q_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0 &&
+               ((uintptr_t)k_plane % 16) == 0 && ((uintptr_t)v_plane % 16) == 0, "attention_prompt: operands not aligned");
+    if (tiles == 0) return TL_OK;
+    AttnArgs a;
+    a.q = q; a.out = out; a.k_plane = k_plane; a.v_plane = v_plane;
+    a.block_table = (const int*)block_table; a.req_indptr = (const int*)req_indptr; a.ctx_lens = (const int*)ctx_lens;
+    a.tile_req = (const int*)tile_req; a.tile_tok0 = (const int*)tile_tok0;
+    a.part_o = nullptr; a.part_ml = nullptr;
+    a.q_stride = q_stride; a.bt_stride = bt_stride; a.heads = heads; a.kv_heads = kv_heads; a.page = page;
+    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = 1; a.scale = scale;
+    a.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz(page) : -1;
+    const int chunks = (group + gcap - 1) / gcap;
+    static hipError_t allowed = hipFuncSetAttribute((const void*)paged_attention_prompt_kernel,
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, ATQ_SMEM);
+    TL_REQUIRE(allowed == hipSuccess, "attention_prompt: cannot get %d bytes of shared memory", ATQ_SMEM);
+    paged_attention_prompt_kernel<<<dim3(tiles, kv_heads * chunks), dim3(256), ATQ_SMEM, stream>>>(a);
+    TL_CHECK_LAUNCH("paged_attention_prompt");
+    return TL_OK;
+#else
+    TL_REQUIRE(false, "attention_prompt: built for head sizes 64 and 128, this library is for %d", AT_HD);
+#endif
+}
+
 extern "C" int tl_attention_head_dim() { return AT_HD; }
 
 // Scratch the caller must provide when splits > 1:

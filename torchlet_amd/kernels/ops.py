@@ -375,6 +375,48 @@ def paged_attention_prefill(q: torch.Tensor, out: torch.Tensor, k_plane: torch.T
                                                c_int(window), c_float(scale), _stream()))
 
 
+PROMPT_ATTENTION_ROWS = 128      # rows a work-group of the 128-row prompt kernel owns
+PROMPT_ATTENTION_HEAD_DIMS = (64, 128)
+
+
+def prompt_attention_fits(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
+    """Whether :func:`paged_attention_prompt` is built for this case."""
+    return dtype == torch.bfloat16 and head_dim in PROMPT_ATTENTION_HEAD_DIMS and page_size % 8 == 0
+
+
+def prompt_attention_tile_tokens(num_heads: int, num_kv_heads: int) -> int:
+    group = num_heads // num_kv_heads
+    return max(1, PROMPT_ATTENTION_ROWS // min(group, PROMPT_ATTENTION_ROWS))
+
+
+def paged_attention_prompt(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v_plane: torch.Tensor,
+                           block_table: torch.Tensor, req_indptr: torch.Tensor, ctx_lens: torch.Tensor,
+                           tile_req: torch.Tensor, tile_tok0: torch.Tensor, num_tiles: int, tile_tokens: int,
+                           num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
+                           scale: float) -> None:
+    """The attention of :func:`paged_attention` for prompt portions in tiles of 128 rows
+    (``tile_tokens`` tokens times the heads of a group): bfloat16, head size 64 or 128, pages
+    of a multiple of 8 tokens; keys and values go straight into shared memory once per
+    work-group.  Writes the rows of its tiles only."""
+    T = q.shape[0]
+    if not prompt_attention_fits(q.dtype, head_dim, page_size):
+        raise KernelError("paged_attention_prompt: bfloat16, head size 64 or 128 and pages of a multiple of 8 tokens only")
+    if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelError("paged_attention_prompt: q/out shapes or dtypes do not fit")
+    _check_planes("paged_attention_prompt", k_plane, v_plane, q.dtype, num_kv_heads, page_size, head_dim)
+    for name, t in (("block_table", block_table), ("req_indptr", req_indptr), ("ctx_lens", ctx_lens),
+                    ("tile_req", tile_req), ("tile_tok0", tile_tok0)):
+        _i32(t, name)
+    if tile_req.numel() < num_tiles or tile_tok0.numel() < num_tiles:
+        raise KernelError("paged_attention_prompt: tile arrays shorter than the number of tiles")
+    lib = _lib(f"attention_hd{head_dim}")
+    _check(lib, lib.tl_paged_attention_prompt(_ptr(q), c_int(q.stride(0)), _ptr(out), _ptr(k_plane), _ptr(v_plane),
+                                              _ptr(block_table), c_int(block_table.stride(0)), _ptr(req_indptr),
+                                              _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles),
+                                              c_int(tile_tokens), c_int(num_heads), c_int(num_kv_heads), c_int(page_size),
+                                              c_int(window), c_float(scale), _stream()))
+
+
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     """``out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]``."""
     T, I2 = gate_up.shape

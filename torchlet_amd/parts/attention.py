@@ -21,9 +21,11 @@ from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedNeed, WeightSpec
 
 _TARGET_WORKGROUPS = 512     # enough work-groups to fill 256 compute units twice
 _MIN_KEYS_PER_SPLIT = 256
-_PORTION_MIN_TOKENS = 16     # requests that bring at least this many tokens go to the prompt-portion kernel ...
-_PORTION_MIN_CONTEXT = 4096  # ... in steps whose longest sequence has at least this many tokens (measured on
-                             # MI355X: the shared-memory kernel wins from about 4k keys on, 13 % at 8k)
+_PORTION_MIN_TOKENS = 16     # requests that bring at least this many tokens go to a prompt-portion kernel: the
+                             # 128-row one where it is built (head size 64 or 128, pages of a multiple of 8
+                             # tokens; measured on MI355X at 28/4 heads of 128: 2048 new tokens 222 -> 110 us,
+                             # 8192 new tokens 2.9 -> 0.84 ms), else the 64-row one ...
+_PORTION_MIN_CONTEXT = 4096  # ... which pays only in steps whose longest sequence has at least this many tokens
 
 
 @MIXERS.register("gqa_attention")
@@ -50,6 +52,7 @@ class GQAttention(Mixer):
         self.position = POSITION_ENCODINGS.build(spec.position, dtype, device) if spec.position is not None else None
         self.tile_tokens = ops.attention_tile_tokens(self.heads, self.kv_heads)
         self.portion_tile_tokens = ops.prefill_attention_tile_tokens(self.heads, self.kv_heads)
+        self.prompt_tile_tokens = ops.prompt_attention_tile_tokens(self.heads, self.kv_heads)
         self.w_qkv: torch.Tensor | None = None
         self.b_qkv: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
@@ -122,15 +125,18 @@ class GQAttention(Mixer):
         out = torch.empty((T, self.q_width), dtype=self.dtype, device=h.device)
         q = qkv[:, : self.q_width]
         common = (self.heads, self.kv_heads, self.head_dim, cache.page_size, self.window or 0, self.scale)
+        rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size)
+                   and ctx.max_new_tokens >= _PORTION_MIN_TOKENS)
         portions = (self.dtype == torch.bfloat16 and self.head_dim <= ops.PREFILL_ATTENTION_MAX_HEAD_DIM
                     and cache.page_size % 4 == 0 and ctx.max_new_tokens >= _PORTION_MIN_TOKENS
                     and ctx.max_total_len >= _PORTION_MIN_CONTEXT)
-        if portions:
-            # prompt portions: 64-row tiles with keys and values through shared memory; the other
-            # requests of the step (decode tokens, short portions): 16-row tiles, keys split over waves
-            short, long = ctx.tiles_by_length(self.tile_tokens, self.portion_tile_tokens, _PORTION_MIN_TOKENS)
-            ops.paged_attention_prefill(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
-                                        long[0], long[1], long[2], self.portion_tile_tokens, *common)
+        if rows128 or portions:
+            # prompt portions: tiles of 128 (or 64) rows with keys and values through shared memory; the
+            # other requests of the step (decode tokens, short portions): 16-row tiles, keys split over waves
+            tq = self.prompt_tile_tokens if rows128 else self.portion_tile_tokens
+            kernel = ops.paged_attention_prompt if rows128 else ops.paged_attention_prefill
+            short, long = ctx.tiles_by_length(self.tile_tokens, tq, _PORTION_MIN_TOKENS)
+            kernel(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens, long[0], long[1], long[2], tq, *common)
             if short[2]:     # one split: the merge of several would run over the rows of the long requests too
                 ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
                                     short[0], short[1], short[2], self.tile_tokens, *common, 1)

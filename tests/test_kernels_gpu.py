@@ -354,6 +354,51 @@ def test_paged_attention(ops, dtype, general, nh, nkv, hd, page, window, splits)
         torch.testing.assert_close(got[a:b], ref, **tol)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_of_some_requests_leaves_the_other_rows_alone(ops, dtype):
+    """Tiles of two of four requests, keys split over work-groups: with the tokens of those
+    requests listed, the merge of the parts writes their rows only."""
+    nh, nkv, hd, page, splits = 6, 2, 32, 8, 3
+    g = torch.Generator().manual_seed(9)
+    lens, ctxs = [5, 1, 40, 1], [60, 150, 0, 90]
+    chosen = [1, 3]
+    R, T = len(lens), sum(lens)
+    totals = [a + b for a, b in zip(lens, ctxs)]
+    max_blocks = (max(totals) + page - 1) // page + 1
+    pages = R * max_blocks + 1
+    bt = (torch.randperm(pages - 1, generator=g)[: R * max_blocks] + 1).view(R, max_blocks).int()
+    q = torch.randn(T, nh * hd, generator=g).to(dtype)
+    kp = torch.randn(pages, nkv, page, hd, generator=g).to(dtype)
+    vp = torch.randn(pages, nkv, hd, page, generator=g).to(dtype)
+    ks, vs = [], []
+    for r in range(R):
+        k = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
+        v = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
+        for p in range(totals[r]):
+            kp[bt[r, p // page], :, p % page] = k[p]
+            vp[bt[r, p // page], :, :, p % page] = v[p]
+        ks.append(k); vs.append(v)
+    indptr = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    tq = ops.attention_tile_tokens(nh, nkv)
+    tile_req = [r for r in chosen for _ in range(0, lens[r], tq)]
+    tile_tok0 = [t0 for r in chosen for t0 in range(0, lens[r], tq)]
+    tokens = [t for r in chosen for t in range(int(indptr[r]), int(indptr[r + 1]))]
+    out = torch.full((T, nh * hd), 7.0, dtype=dtype, device="cuda")
+    ops.paged_attention(q.cuda(), out, kp.cuda(), vp.cuda(), bt.cuda(), indptr.cuda(),
+                        torch.tensor(ctxs, dtype=torch.int32).cuda(), torch.tensor(tile_req, dtype=torch.int32).cuda(),
+                        torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq, nh, nkv, hd, page, 0,
+                        1.0 / math.sqrt(hd), splits, merge_tokens=(torch.tensor(tokens, dtype=torch.int32).cuda(), len(tokens)))
+    got = out.cpu().double().view(T, nh, hd)
+    for r in range(R):
+        a, b = int(indptr[r]), int(indptr[r + 1])
+        if r in chosen:
+            ref = _attention_ref(q[a:b].double().view(-1, nh, hd), ks[r].double(), vs[r].double(), 0)
+            tol = _tol(dtype)
+            torch.testing.assert_close(got[a:b], ref, rtol=tol["rtol"], atol=tol["atol"] + 2 ** -9 * float(vs[r].abs().max()))
+        else:
+            assert bool((got[a:b] == 7.0).all()), f"rows of request {r} were written"
+
+
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [
     (4, 2, 16, 16, 0), (3, 1, 32, 8, 0), (28, 4, 128, 16, 0), (6, 6, 48, 4, 0), (20, 1, 64, 16, 0),
     (4, 2, 16, 16, 13), (8, 2, 80, 32, 29), (14, 2, 128, 64, 40), (5, 5, 112, 12, 70),

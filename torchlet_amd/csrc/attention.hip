@@ -699,10 +699,11 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(AttnArgs a
 
 // out[row] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s over the parts of a row.
 // The parts are read eight at a time with all loads issued before the first use.
+// Rows are (token, head) pairs: all of them, or those of the tokens listed in `tokens`.
 template <typename T>
 __global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                       T* __restrict__ out, int splits) {
-    const size_t r = blockIdx.x;
+                                       T* __restrict__ out, int splits, const int* __restrict__ tokens, int heads) {
+    const size_t r = tokens ? (size_t)tokens[blockIdx.x / heads] * heads + blockIdx.x % heads : blockIdx.x;
     const float2* ml = (const float2*)(part_ml + r * splits * 2);
     const float* po = part_o + r * splits * AT_HD;
     const int d = threadIdx.x;                     // blockDim.x == AT_HD
@@ -1040,7 +1041,8 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
                                   const void* block_table, int bt_stride, const void* req_indptr, const void* ctx_lens,
                                   const void* tile_req, const void* tile_tok0, int tiles, int tokens, int tq,
                                   int heads, int kv_heads, int page, int window, float scale, int splits,
-                                  void* part_o, void* part_ml, int dtype, int general, hipStream_t stream) {
+                                  void* part_o, void* part_ml, const void* merge_tokens, int merge_count, int dtype, int general,
+                                  hipStream_t stream) {
     TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
     TL_REQUIRE(page > 0 && bt_stride > 0 && tq > 0 && splits > 0 && window >= 0, "attention: bad page/table/tile sizes");
     TL_REQUIRE(splits == 1 || (part_o && part_ml), "attention: splits > 1 needs scratch");
@@ -1067,9 +1069,12 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
     else TL_REQUIRE(false, "attention: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("paged_attention");
     if (splits > 1) {
-        dim3 mgrid((unsigned)((size_t)tokens * heads)), mblock(AT_HD);
-        if (dtype == TL_DT_F32) attention_merge_kernel<float><<<mgrid, mblock, 0, stream>>>((const float*)part_o, (const float*)part_ml, (float*)out, splits);
-        else attention_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, splits);
+        // merge_tokens: the tokens whose rows the tiles cover, when these are not all tokens of the step
+        const size_t rows = (size_t)(merge_tokens ? merge_count : tokens) * heads;
+        if (rows == 0) return TL_OK;
+        dim3 mgrid((unsigned)rows), mblock(AT_HD);
+        if (dtype == TL_DT_F32) attention_merge_kernel<float><<<mgrid, mblock, 0, stream>>>((const float*)part_o, (const float*)part_ml, (float*)out, splits, (const int*)merge_tokens, heads);
+        else attention_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, splits, (const int*)merge_tokens, heads);
         TL_CHECK_LAUNCH("attention_merge");
     }
     return TL_OK;

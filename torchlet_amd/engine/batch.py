@@ -49,6 +49,7 @@ class StepContext:
         self.decode_only = bool(R and self.max_new_tokens == 1)
         self.device = device
         self._host_new_lens = new_lens
+        self._host_ctx_lens = ctx_np
         self._tiles: dict[int, tuple] = {}
 
         fields = {
@@ -115,15 +116,23 @@ class StepContext:
 
     def tiles_by_length(self, tq_short: int, tq_long: int, threshold: int):
         """Two tile lists: requests that bring fewer than ``threshold`` tokens in tiles of
-        ``tq_short`` tokens, the others in tiles of ``tq_long``."""
+        ``tq_short`` tokens, the others in tiles of ``tq_long``.  The first list comes with the
+        indices of its requests' tokens and the largest sequence length among them:
+        ``((tile_req, tile_tok0, tiles, tokens, number of tokens, longest), (tile_req, tile_tok0, tiles))``."""
         key = (tq_short, tq_long, threshold)
         t = self._tiles.get(key)
         if t is None:
             long = self._host_new_lens >= threshold
             sr, s0 = self._build_tiles(tq_short, ~long)
             lr, l0 = self._build_tiles(tq_long, long)
-            v = self._upload({"sr": sr, "s0": s0, "lr": lr, "l0": l0})
-            t = self._tiles[key] = ((v["sr"], v["s0"], len(sr)), (v["lr"], v["l0"], len(lr)))
+            starts = np.zeros(self.num_requests + 1, dtype=np.int64)
+            np.cumsum(self._host_new_lens, out=starts[1:])
+            short_tokens = np.concatenate([np.arange(starts[r], starts[r + 1]) for r in np.nonzero(~long)[0]] or
+                                          [np.zeros(0, dtype=np.int64)]).astype(np.int32)
+            longest = int((self._host_new_lens + self._host_ctx_lens)[~long].max()) if (~long).any() else 0
+            v = self._upload({"sr": sr, "s0": s0, "lr": lr, "l0": l0, "st": short_tokens})
+            t = self._tiles[key] = ((v["sr"], v["s0"], len(sr), v["st"], len(short_tokens), longest),
+                                    (v["lr"], v["l0"], len(lr)))
         return t
 
 

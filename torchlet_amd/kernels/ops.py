@@ -309,14 +309,16 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
                     block_table: torch.Tensor, req_indptr: torch.Tensor, ctx_lens: torch.Tensor,
                     tile_req: torch.Tensor, tile_tok0: torch.Tensor, num_tiles: int, tile_tokens: int,
                     num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
-                    scale: float, splits: int = 1, general: bool = False) -> None:
+                    scale: float, splits: int = 1, general: bool = False, merge_tokens=None) -> None:
     """Causal attention of the step's tokens over their requests' cached keys.
 
     ``q [T, >= heads*hd]`` (row-strided view), ``out [T, heads*hd]``, ``k_plane [pages,
     kv_heads, page, hd]``, ``v_plane [pages, kv_heads, hd, page]``, ``block_table [R,
     max_blocks]`` int32; the new token ``i`` of request ``r`` sits at position
     ``ctx_lens[r] + i``.  ``window`` 0: all keys.  bfloat16 with pages of a multiple of 4
-    tokens runs on the matrix cores; ``general=True`` forces the general kernel."""
+    tokens runs on the matrix cores; ``general=True`` forces the general kernel.  When the
+    tiles cover only some of the step's tokens and ``splits > 1``, ``merge_tokens = (int32
+    indices of those tokens, their number)`` keeps the merge of the parts to their rows."""
     T = q.shape[0]
     if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
         raise KernelError("paged_attention: q/out shapes or dtypes do not fit")
@@ -326,6 +328,8 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
         _i32(t, name)
     if tile_req.numel() < num_tiles or tile_tok0.numel() < num_tiles:
         raise KernelError("paged_attention: tile arrays shorter than the number of tiles")
+    if merge_tokens is not None:
+        _i32(merge_tokens[0], "merge_tokens", merge_tokens[1])
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty((T * num_heads * splits, head_dim), dtype=torch.float32, device=q.device)
@@ -336,6 +340,8 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
                                        _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles), c_int(T), c_int(tile_tokens),
                                        c_int(num_heads), c_int(num_kv_heads), c_int(page_size), c_int(window),
                                        c_float(scale), c_int(splits), _ptr(part_o), _ptr(part_ml),
+                                       _ptr(merge_tokens[0]) if merge_tokens is not None else c_void_p(None),
+                                       c_int(merge_tokens[1] if merge_tokens is not None else 0),
                                        c_int(_dt(q, "paged_attention")), c_int(1 if general else 0), _stream()))
 
 

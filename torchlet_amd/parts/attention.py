@@ -87,12 +87,13 @@ class GQAttention(Mixer):
         self.w_o = self._place(tensors["o_proj.weight"], "matrix")
 
     # -- the step -----------------------------------------------------------------
-    def _splits(self, ctx, tiles: int) -> int:
+    def _splits(self, ctx, tiles: int, longest: int | None = None) -> int:
         group = self.heads // self.kv_heads
         chunks = -(-group // ops.ATTENTION_ROWS)
         base = max(1, tiles * self.kv_heads * chunks)
         by_fill = -(-_TARGET_WORKGROUPS // base)
-        longest = ctx.max_total_len if self.window is None else min(ctx.max_total_len, self.window + ctx.max_new_tokens)
+        longest = ctx.max_total_len if longest is None else longest
+        longest = longest if self.window is None else min(longest, self.window + ctx.max_new_tokens)
         by_keys = max(1, longest // _MIN_KEYS_PER_SPLIT)
         return max(1, min(by_fill, by_keys, 64))
 
@@ -137,9 +138,10 @@ class GQAttention(Mixer):
             kernel = ops.paged_attention_prompt if rows128 else ops.paged_attention_prefill
             short, long = ctx.tiles_by_length(self.tile_tokens, tq, _PORTION_MIN_TOKENS)
             kernel(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens, long[0], long[1], long[2], tq, *common)
-            if short[2]:     # one split: the merge of several would run over the rows of the long requests too
+            if short[2]:     # split over their keys; the merge of the parts is kept to the rows of these requests
                 ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
-                                    short[0], short[1], short[2], self.tile_tokens, *common, 1)
+                                    short[0], short[1], short[2], self.tile_tokens, *common,
+                                    self._splits(ctx, short[2], short[5]), merge_tokens=(short[3], short[4]))
         else:
             tile_req, tile_tok0, tiles = ctx.tiles(self.tile_tokens)
             ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,

@@ -139,3 +139,10 @@ def test_errors_fail_every_unfinished_request(cpu_ops, model_folders, monkeypatc
     assert engine.runner.cache.live_requests() == [] and not engine.has_work()
     with pytest.raises(ValueError, match="outside the vocabulary"):
         engine.add_request(Request(prompt_tokens=[999]))
+
+
+def test_toy_parts_and_a_layer_run_twice_on_the_host(cpu_ops):
+    """The generality test of ``toy_parts.py`` (a routed feed-forward, a position encoding of its
+    own, a layer that runs twice and reads its first run's cache) through the host logic."""
+    import toy_parts
+    toy_parts.run_toy_mix(torch.float32, torch.device("cpu"), lambda dtype, ref: dict(atol=2e-5, rtol=1e-4))

@@ -267,3 +267,9 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path):
     finally:
         unregister_architecture("ToyDecayForCausalLM")
         MIXERS.unregister("toy_decay")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_routed_feed_forward_and_toy_position_encoding_with_a_layer_run_twice(dtype):
+    import toy_parts
+    toy_parts.run_toy_mix(dtype, torch.device("cuda"), _tol)

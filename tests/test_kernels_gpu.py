@@ -316,8 +316,10 @@ def test_paged_attention(ops, dtype, general, nh, nkv, hd, page, window, splits)
     pages = R * max_blocks + 1
     bt = (torch.randperm(pages - 1, generator=g)[: R * max_blocks] + 1).view(R, max_blocks).int()
     q = torch.randn(T, nh * hd, generator=g).to(dtype)
-    kp = torch.randn(pages, nkv, page, hd, generator=g).to(dtype)      # stale pages hold noise, not zeros
-    vp = torch.randn(pages, nkv, hd, page, generator=g).to(dtype)      # transposed inside a page
+    # places that hold no key yet are NaN (a page that another request left behind may hold anything):
+    # nothing of them may reach a result
+    kp = torch.full((pages, nkv, page, hd), float("nan"), dtype=dtype)
+    vp = torch.full((pages, nkv, hd, page), float("nan"), dtype=dtype)      # transposed inside a page
     ks, vs = [], []
     for r in range(R):
         k = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)
@@ -415,8 +417,8 @@ def test_paged_attention_prompt_portions(ops, nh, nkv, hd, page, window):
     pages = R * max_blocks + 1
     bt = (torch.randperm(pages - 1, generator=g)[: R * max_blocks] + 1).view(R, max_blocks).int()
     q = torch.randn(T, nh * hd, generator=g).to(dtype)
-    kp = torch.randn(pages, nkv, page, hd, generator=g).to(dtype)
-    vp = torch.randn(pages, nkv, hd, page, generator=g).to(dtype)
+    kp = torch.full((pages, nkv, page, hd), float("nan"), dtype=dtype)      # NaN where no key is written
+    vp = torch.full((pages, nkv, hd, page), float("nan"), dtype=dtype)
     ks, vs = [], []
     for r in range(R):
         k = torch.randn(totals[r], nkv, hd, generator=g).to(dtype)

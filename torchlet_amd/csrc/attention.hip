@@ -55,6 +55,18 @@ __device__ __forceinline__ void split_key(int key, int page, int shift, int& blk
     }
 }
 
+// Four bfloat16 values of the keys key0 .. key0 + 3 with those at or beyond key_hi set to zero.
+// A page may hold anything where no key has been written yet (another request's leftovers, even
+// Inf or NaN); a probability of zero does not stop those from reaching the sum, a zero value does.
+__device__ __forceinline__ uint2 keep_written(uint2 v, int key0, int key_hi) {
+    const int n = key_hi - key0;                  // written keys among the four
+    if (n >= 4) return v;
+    if (n <= 0) return make_uint2(0, 0);
+    if (n == 1) return make_uint2(v.x & 0xffffu, 0);
+    if (n == 2) return make_uint2(v.x, 0);
+    return make_uint2(v.x, v.y & 0xffffu);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     __shared__ float qs[AT_ROWS][AT_HD + 1];
@@ -335,6 +347,12 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
             VA[t] = oka ? *(const uint2*)(va + 16 * t * page) : make_uint2(0, 0);                            \
             VB[t] = okb ? *(const uint2*)(vb + 16 * t * page) : make_uint2(0, 0);                            \
         }                                                                                                    \
+        if (kb_ + 32 > key_hi) {          /* the last chunk: keys that are not written yet */                 \
+            _Pragma("unroll") for (int t = 0; t < ATM_DT; ++t) {                                             \
+                VA[t] = keep_written(VA[t], ka, key_hi);                                                     \
+                VB[t] = keep_written(VB[t], kb, key_hi);                                                     \
+            }                                                                                                \
+        }                                                                                                    \
     }
 
     const size_t kv_stride = (size_t)a.kv_heads * page * AT_HD;     /* elements per page, all KV heads */
@@ -575,7 +593,7 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(AttnArgs a
             if (tid + 256 * i < ATP_VPIECES && key4 < key_hi) {                                            \
                 int blk, off;                                                                              \
                 split_key(key4, page, a.page_shift, blk, off);                                             \
-                VS_[i] = *(const uint2*)(vp + ((size_t)ATP_PAGE_OF(blk) * kv_stride + kvh_off + vd[i] * page + off)); \
+                VS_[i] = keep_written(*(const uint2*)(vp + ((size_t)ATP_PAGE_OF(blk) * kv_stride + kvh_off + vd[i] * page + off)), key4, key_hi); \
             }                                                                                              \
         }                                                                                                  \
     }

@@ -21,12 +21,15 @@ LENGTHS = {"A": [70, 33, 97, 5, 120, 64], "B": [40, 129, 9, 64, 200, 1 + 32], "C
 TOL = {"float32": scenarios.FP32_TOL, "bfloat16": scenarios.BF16_TOL}
 
 
-def _run_in_process(folder, dtype, steps, page_size, max_tokens, max_requests=4):
+def _run_in_process(folder, dtype, steps, page_size, max_tokens, max_requests=4, poison=False):
     from torchlet_amd.engine.batch import StepEntry
     from torchlet_amd.engine.loading import load_model, make_runner
 
     _, model = load_model(folder, dtype)
     runner = make_runner(model, page_size=page_size, num_pages=-(-max_tokens // page_size) + 1, max_requests=max_requests)
+    if poison:      # every page but the sentinel (page 0), which nothing ever writes and released entries point to
+        for group in runner.cache.groups:
+            group.tensor[:, :, 1:].fill_(float("nan"))          # [runs, planes, pages, heads, page, head size]
     out = {}
     for s in steps:
         logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
@@ -36,6 +39,9 @@ def _run_in_process(folder, dtype, steps, page_size, max_tokens, max_requests=4)
             runner.release(r)
     runner.cache.check()
     assert runner.cache.live_requests() == []
+    if poison:
+        for group in runner.cache.groups:
+            assert not bool(group.tensor[:, :, 0].any()), "the sentinel page was written"
     return out
 
 
@@ -109,6 +115,17 @@ def test_decode_steps_replayed_as_graphs(model_folders, expected, name, dtype):
             runner.release(r)
     assert runner.graph_replays >= 20 and len(runner._graphs) >= 2
     scenarios.check(steps, out, exp, TOL[dtype], f"graphs/{name}/{dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_pages_that_hold_nan_where_nothing_is_written_yet(model_folders, expected, name, dtype):
+    """The pool starts out full of NaN instead of zeros, as if earlier requests had left the worst
+    behind: no kernel may let a place that its request has not written reach a result."""
+    reqs, exp = expected(name)
+    steps = scenarios.number(scenarios.mixed(reqs))
+    out = _run_in_process(model_folders[name], dtype, steps, tiny_models.PAGE_SIZES[name], scenarios.max_tokens_needed(steps), poison=True)
+    scenarios.check(steps, out, exp, TOL[dtype], f"poisoned pool/{name}/{dtype}")
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])

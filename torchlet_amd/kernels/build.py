@@ -31,7 +31,7 @@ FLAGS = [
 HEADERS = ["common.h"]
 
 # head sizes compiled by build_all(): what the tests, the smoke run and the benchmark use
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
 
 
 class BuildError(RuntimeError):

@@ -157,23 +157,6 @@ def test_linear_few_rows_on_matrix_cores(ops, out_dtype, M, N, K):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("M", [1, 7, 16])
-@pytest.mark.parametrize("N,K", [(16384, 64), (16400, 200), (40000, 1000), (20011, 3584), (16384, 4096)])
-def test_linear_streaming_kernel(ops, out_dtype, M, N, K):
-    """The persistent weight-streaming kernel: every depth of K steps per wave, tails in N and K,
-    strips that do not divide evenly over the work-groups."""
-    g = torch.Generator().manual_seed(M + N)
-    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
-    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).cuda()
-    b = torch.randn(N, generator=g).to(torch.bfloat16).cuda()
-    ref = x.double() @ w.double().T + b.double()
-    out = torch.full((M, N), float("nan"), dtype=out_dtype, device="cuda")
-    ops.linear_stream_variant(x, w, b, out)
-    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
-    torch.testing.assert_close(out.double(), ref, **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
-
-
-@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("tile", [(128, 128, 32), (128, 128, 64), (256, 128, 32), (256, 128, 64), (128, 256, 32), (128, 256, 64),
                                   (64, 128, 32), (64, 128, 64), (256, 256, 32), (256, 256, 64)])
 @pytest.mark.parametrize("M,N,K", [(65, 129, 64), (300, 520, 200), (1000, 257, 1000), (2, 48, 3584)])

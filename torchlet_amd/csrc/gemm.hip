@@ -371,134 +371,6 @@ static void launch_skinny(const void* x, const void* w, const void* bias, int bi
     else launch_skinny_t<R, MT, KS, bf16_t, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
 }
 
-// =====================================================================================
-// The same product for up to 16 rows against a matrix with many strips (gate/up, LM head):
-// one work-group per compute unit that walks a range of strips.
-//
-// Every wave keeps its share of x (the K steps s = wave, wave + KS, ...) in registers for the
-// whole kernel, so after the first strip only weights are read; the weights of strip i + 1
-// are fetched while strip i is multiplied, reduced and stored, and the reduction of a strip
-// (through shared memory, two buffers) is done by one wave in turn while the others go on:
-// the weight stream never stops for a strip's epilogue.  Needs K <= 64 * KS * DS.
-// SW: the matrix is the interleaved gate/up matrix (see gemm_skinny_kernel); a work item is a
-// (gate strip, up strip) pair, processed as two strips whose sums the same wave combines.
-template <int KS, int DS, typename TOut, bool SW>
-__global__ __launch_bounds__(KS * 64) void gemm_stream_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                              const void* __restrict__ bias, int bias_f32,
-                                                              TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-                                                              int out_cols, int items, int items_per_group) {
-    __shared__ float red[2][KS * 256];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int li = lane & 15, lg = lane >> 4;
-
-    // my K steps and which 8-element pieces of them lie inside K
-    int koff[DS];
-    bool v0[DS], v1[DS];
-    Frag16 xb0[DS], xb1[DS];
-    const bf16_t* xrow = x + (size_t)min(li, M - 1) * ldx;
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-#pragma unroll
-    for (int d = 0; d < DS; ++d) {
-        koff[d] = 64 * (wave + d * KS) + 16 * lg;
-        v0[d] = koff[d] + 8 <= K;
-        v1[d] = koff[d] + 16 <= K;
-        xb0[d].u = v0[d] ? *(const uint4*)(xrow + koff[d]) : zero;
-        xb1[d].u = v1[d] ? *(const uint4*)(xrow + koff[d] + 8) : zero;
-    }
-
-    const int first = blockIdx.x * items_per_group;
-    const int last = min(first + items_per_group, items);
-    // first weight row of a work item's strip
-    auto strip_row = [&](int item) -> int {
-        if (!SW) return 16 * item;
-        const int pair = item >> 1, sub = item & 1;
-        return 16 * (4 * (pair >> 1) + (pair & 1) + 2 * sub);
-    };
-    Frag16 a0[DS], a1[DS], n0[DS], n1[DS];
-#define ST_FETCH(A0, A1, item)                                                                  \
-    {                                                                                           \
-        const bf16_t* wr = w + (size_t)min(strip_row(item) + li, N - 1) * K;                    \
-        _Pragma("unroll") for (int d = 0; d < DS; ++d) {                                        \
-            A0[d].u = v0[d] ? *(const uint4*)(wr + koff[d]) : zero;                             \
-            A1[d].u = v1[d] ? *(const uint4*)(wr + koff[d] + 8) : zero;                         \
-        }                                                                                       \
-    }
-    if (first < last) ST_FETCH(a0, a1, first)
-    f32x4_t gate_sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    for (int item = first; item < last; ++item) {
-        if (item + 1 < last) ST_FETCH(n0, n1, item + 1)
-        f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int d = 0; d < DS; ++d) {
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[d].v, xb0[d].v, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[d].v, xb1[d].v, acc, 0, 0, 0);
-        }
-        const int buf = (item - first) & 1;
-        *(f32x4_t*)(&red[buf][(wave * 64 + lane) * 4]) = acc;
-        lds_barrier();
-        const int unit = SW ? (item >> 1) : item;
-        if (wave == unit % KS) {
-            f32x4_t sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int wv = 0; wv < KS; ++wv) sum += *(const f32x4_t*)(&red[buf][(wv * 64 + lane) * 4]);
-            // D[i][j]: i = 4 * lg + v (weight row of the strip), j = li (activation row)
-            if (SW) {
-                if ((item & 1) == 0) {
-                    gate_sum = sum;
-                } else if (li < M) {
-                    const int col = 16 * unit + 4 * lg;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v)
-                        if (col + v < out_cols) out[(size_t)li * ldo + col + v] = from_float<TOut>(silu_mul(gate_sum[v], sum[v]));
-                }
-            } else if (li < M) {
-                const int n = 16 * item + 4 * lg;
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    if (n + v < N) {
-                        float val = sum[v];
-                        if (bias) val += load_vec(bias, bias_f32, n + v);
-                        out[(size_t)li * ldo + n + v] = from_float<TOut>(val);
-                    }
-            }
-        }
-#pragma unroll
-        for (int d = 0; d < DS; ++d) { a0[d] = n0[d]; a1[d] = n1[d]; }
-    }
-#undef ST_FETCH
-}
-
-// Launches gemm_stream_kernel if the shape fits it (M <= 16, K <= 4096, at least 1024 strips);
-// returns false otherwise.
-template <typename TOut, bool SW>
-static bool launch_stream(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
-                          int ldx, int ldo, int out_cols, hipStream_t stream) {
-    const int strips = (N + 15) / 16;
-    if (M > 16 || K > 4096 || strips < 1024) return false;
-    const int units = SW ? strips / 4 * 2 : strips;          // SW: N is a multiple of 64 rows
-    const int groups = units < 512 ? units : 512;             // two work-groups' worth per compute unit, walked in order
-    const int per_group = (units + groups - 1) / groups * (SW ? 2 : 1);
-    const int items = SW ? units * 2 : units;
-    const int grid = (items + per_group - 1) / per_group;
-    const int ds = ((K + 63) / 64 + 15) / 16;
-#define TL_STREAM_CASE(d) \
-    if (ds == d) gemm_stream_kernel<16, d, TOut, SW><<<dim3(grid), dim3(1024), 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, items, per_group);
-    TL_STREAM_CASE(1) TL_STREAM_CASE(2) TL_STREAM_CASE(3) TL_STREAM_CASE(4)
-#undef TL_STREAM_CASE
-    return true;
-}
-
-// The streaming kernel by itself (tests and tuning).
-extern "C" int tl_gemm_stream_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
-                                      int M, int N, int K, int ldx, int ldo, int out_f32, hipStream_t stream) {
-    TL_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_stream: needs K, ldx multiples of 8");
-    const bool ok = out_f32 ? launch_stream<float, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream)
-                            : launch_stream<bf16_t, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
-    TL_REQUIRE(ok, "gemm_stream: shape M=%d N=%d K=%d does not fit (M <= 16, K <= 4096, N >= 16384)", M, N, K);
-    TL_CHECK_LAUNCH("gemm_stream");
-    return TL_OK;
-}
-
 template <int MT>
 static void pick_skinny(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                         int ldx, int ldo, int out_f32, hipStream_t stream) {

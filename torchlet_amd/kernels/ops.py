@@ -191,17 +191,6 @@ def linear_few_rows_variant(x, weight, bias, out, strips_per_wave: int, waves_al
                                            c_int(waves_along_k), _stream()))
 
 
-def linear_stream_variant(x, weight, bias, out) -> None:
-    """The persistent weight-streaming kernel by itself (M <= 16, K <= 4096, N >= 16384)."""
-    M, K = x.shape
-    N = weight.shape[0]
-    bf = _vec(bias, N, "linear bias")
-    lib = _lib("gemm")
-    _check(lib, lib.tl_gemm_stream_variant(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N),
-                                           c_int(K), c_int(x.stride(0)), c_int(out.stride(0)),
-                                           c_int(1 if out.dtype == torch.float32 else 0), _stream()))
-
-
 def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int, slab: int = 32) -> None:
     """One named tile shape of the many-rows matrix-core kernel (for tests and tuning)."""
     M, K = x.shape

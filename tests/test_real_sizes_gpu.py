@@ -1,4 +1,4 @@
-"""The engine at the layer widths of the 7B, 14B and 32B checkpoints (all heads, groups,
+"""The engine at the layer widths of the 0.5B to 32B checkpoints (all heads, groups,
 intermediate sizes and the whole vocabulary, one or two layers, random weights) against the
 plain implementation, under every way of cutting the requests into steps.
 
@@ -24,6 +24,12 @@ import scenarios
 pytestmark = pytest.mark.gpu
 
 SHAPES = {
+    "0.5B": dict(num_hidden_layers=3, hidden_size=896, num_attention_heads=14, num_key_value_heads=2,
+                 intermediate_size=4864, rms_norm_eps=1e-6, vocab_size=151936, tie_word_embeddings=True),
+    "1.5B": dict(num_hidden_layers=2, hidden_size=1536, num_attention_heads=12, num_key_value_heads=2,
+                 intermediate_size=8960, rms_norm_eps=1e-6, vocab_size=151936, tie_word_embeddings=True),
+    "3B": dict(num_hidden_layers=2, hidden_size=2048, num_attention_heads=16, num_key_value_heads=2,
+               intermediate_size=11008, rms_norm_eps=1e-6, vocab_size=151936, tie_word_embeddings=True),
     "7B": dict(num_hidden_layers=2, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4,
                intermediate_size=18944, rms_norm_eps=1e-6),
     "14B": dict(num_hidden_layers=1, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,

@@ -435,14 +435,14 @@ def test_paged_attention_prompt_portions(ops, nh, nkv, hd, page, window):
 
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [
     (28, 4, 128, 16, 0), (20, 1, 64, 16, 0), (40, 8, 128, 8, 0), (4, 4, 64, 32, 0), (130, 1, 64, 16, 0),
-    (14, 2, 128, 64, 40), (4, 4, 64, 32, 29), (6, 2, 128, 24, 100),
+    (14, 2, 128, 64, 40), (4, 4, 64, 32, 29), (6, 2, 128, 8, 100),
 ])
 def test_paged_attention_prompt_tiles_of_128_rows(ops, nh, nkv, hd, page, window):
     """The 128-row kernel for prompt portions: whole prompts, portions on top of a cached context
     (also one that starts inside a page and inside a step of 64 keys), a single token, groups of
     1, 3, 5, 7, 20 and 130 heads.  Places of the pages that hold no key yet are filled with NaN:
     nothing of them may reach a result."""
-    assert ops.prompt_attention_fits(torch.bfloat16, hd, page)
+    assert ops.prompt_attention_fits(torch.bfloat16, hd, page) and not ops.prompt_attention_fits(torch.bfloat16, hd, 24)
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(15)
     lens, ctxs = [150, 37, 70, 1, 64, 300], [0, 150, 43, 99, 64, 5]

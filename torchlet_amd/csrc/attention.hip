@@ -755,12 +755,13 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
 }
 
 // =====================================================================================
-// Prompt portions, 128 rows per work-group (bfloat16, head size 64 or 128, pages of a multiple
-// of 8 tokens).
+// Prompt portions, 128 rows per work-group (bfloat16, head size 64 or 128, pages of 8, 16, 32, ...
+// tokens, block tables of up to ATM_BT_MAX entries).
 //
-// Four waves of 32 rows share steps of 64 keys.  Keys and transposed values of a step go from
-// the pages straight into shared memory (global_load_lds_dwordx4, two buffers: the next step is
-// on its way while this one is multiplied), in 16-byte pieces whose slot within a row is
+// Four waves of 32 rows share steps of 32 keys.  Keys and transposed values of a step go from
+// the pages straight into shared memory (global_load_lds_dwordx4, four buffers: three steps are
+// on their way while one is multiplied; with two buffers of 64 keys the kernel spent half its
+// time waiting for the next step's keys), in 16-byte pieces whose slot within a row is
 // exclusive-ored with the row number, so that the operand reads of sixteen neighbouring rows
 // fall on all banks.  Both products run transposed on v_mfma_f32_32x32x16_bf16:
 //   S^T[key, row] = K[key, :] . Q[row, :]      A = 32 keys x 16 d from shared memory, B = Q (registers)
@@ -772,10 +773,18 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
 // the B operand of the second product, with no exchange between lanes.
 #if AT_HD == 64 || AT_HD == 128
 #define ATQ_ROWS 128
-#define ATQ_KEYS 64
+#ifndef ATQ_KEYS
+#define ATQ_KEYS 32                 // keys per step: 32 or 64
+#endif
+#ifndef ATQ_STAGES
+#define ATQ_STAGES 4               // steps in shared memory: this one and those on their way
+#endif
+#define ATQ_KB (ATQ_KEYS / 32)      // blocks of 32 keys per step
+#define ATQ_VROW (ATQ_KEYS * 2)     // bytes of a transposed value row (one d, the step's keys)
+#define ATQ_VPP (ATQ_KEYS / 8)      // 16-byte pieces in it
 #define ATQ_KBYTES (ATQ_KEYS * AT_HD * 2)
 #define ATQ_STAGE (2 * ATQ_KBYTES)                 // keys, then values
-#define ATQ_SMEM (2 * ATQ_STAGE + ATM_BT_MAX * 4)
+#define ATQ_SMEM (ATQ_STAGES * ATQ_STAGE + ATM_BT_MAX * 4)
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 // 16 bytes per lane from memory straight into shared memory at lds_addr + 16 * lane.  Issued as
@@ -788,10 +797,13 @@ __device__ __forceinline__ void attn_load_to_lds(const void* gptr, unsigned lds_
 __device__ __forceinline__ int atq_key_slot(int piece, int key) {        // slot of a 16-byte piece in its key row
     return AT_HD == 128 ? (piece ^ (key & 15)) : (piece ^ ((key >> 1) & 7));
 }
+__device__ __forceinline__ int atq_value_slot(int piece, int d) {        // ... in its transposed value row
+    return ATQ_KEYS == 64 ? (piece ^ ((d >> 1) & 7)) : (piece ^ ((d >> 2) & 3));
+}
 
 __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char atq_smem[];
-    int* bt_s = (int*)(atq_smem + 2 * ATQ_STAGE);
+    int* bt_s = (int*)(atq_smem + ATQ_STAGES * ATQ_STAGE);
     const unsigned lds_base = (unsigned)(uintptr_t)((void __attribute__((address_space(3)))*)atq_smem);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lr = lane & 31, h = lane >> 5;
@@ -842,40 +854,49 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     const int page = a.page;
     const size_t kv_stride = (size_t)a.kv_heads * page * AT_HD;
     const int kvh_off = kvh * page * AT_HD;
+    // the request's block-table row goes to shared memory (the host checked that it fits); pages are a
+    // power of two, so a key's block and place in it are a shift and a mask
     const int* bt_g = a.block_table + (size_t)req * a.bt_stride;
-    const int blk0 = (st_first * ATQ_KEYS) / page;
-    const int blk_n = (key_hi - 1) / page - blk0 + 1;
-    const bool bt_local = blk_n <= ATM_BT_MAX;
-    if (bt_local) {
-        for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
-        __syncthreads();
-    }
-#define ATQ_PAGE_OF(blk) (bt_local ? bt_s[(blk) - blk0] : bt_g[(blk)])
+    const int shift = a.page_shift, pmask = page - 1;
+    const int blk0 = (st_first * ATQ_KEYS) >> shift;
+    const int blk_n = ((key_hi - 1) >> shift) - blk0 + 1;
+    for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
+    __syncthreads();
 
-    // requests of one step: K rows of AT_HD * 2 bytes, then V^T rows of 128 bytes (64 keys)
+    // requests of one step: K rows of AT_HD * 2 bytes, then V^T rows of ATQ_VROW bytes
     constexpr int KPI = 1024 / (AT_HD * 2);                 // keys per load instruction (4 or 8)
     constexpr int KPP = AT_HD / 8;                          // pieces per key row (16 or 8)
     constexpr int K_INSTR = ATQ_KBYTES / 1024 / 4;          // per wave
+    constexpr int VDI = 1024 / ATQ_VROW;                    // value rows (d) per load instruction (8 or 16)
+    static_assert(K_INSTR >= 1 && 2 * K_INSTR * (ATQ_STAGES - 2) < 64, "loads per wave and step");
+    // what does not change from step to step, per load instruction of this lane
+    int k_local[K_INSTR], k_piece[K_INSTR], v_key[K_INSTR], v_row[K_INSTR];
+    unsigned k_dst[K_INSTR];
+#pragma unroll
+    for (int j = 0; j < K_INSTR; ++j) {
+        const int ii = wave + 4 * j;
+        k_local[j] = KPI * ii + lane / KPP;
+        k_piece[j] = atq_key_slot(lane % KPP, k_local[j]) * 8;       // exclusive-or is its own inverse
+        const int d = VDI * ii + lane / ATQ_VPP;
+        v_key[j] = 8 * atq_value_slot(lane % ATQ_VPP, d);            // first of the piece's eight keys
+        v_row[j] = kvh_off + d * page;
+        k_dst[j] = __builtin_amdgcn_readfirstlane(ii * 1024);
+    }
+    const int key_last8 = (key_hi - 1) & ~7;
     auto request_step = [&](int st, int buf) {
         const int kbase = st * ATQ_KEYS;
         const unsigned sb = lds_base + buf * ATQ_STAGE;
 #pragma unroll
         for (int j = 0; j < K_INSTR; ++j) {
-            const int ii = __builtin_amdgcn_readfirstlane(wave + 4 * j);
-            const int kl = KPI * ii + lane / KPP;            // key within the step
-            const int piece = atq_key_slot(lane % KPP, kl);  // exclusive-or is its own inverse
-            int blk, off;
-            split_key(min(kbase + kl, key_hi - 1), page, a.page_shift, blk, off);
-            attn_load_to_lds(kp + ((size_t)ATQ_PAGE_OF(blk) * kv_stride + kvh_off + off * AT_HD + piece * 8), sb + ii * 1024);
+            const int key = min(kbase + k_local[j], key_hi - 1);
+            const int pg = bt_s[(key >> shift) - blk0];
+            attn_load_to_lds(kp + ((size_t)pg * kv_stride + kvh_off + (key & pmask) * AT_HD + k_piece[j]), sb + k_dst[j]);
         }
 #pragma unroll
         for (int j = 0; j < K_INSTR; ++j) {
-            const int ii = __builtin_amdgcn_readfirstlane(wave + 4 * j);
-            const int d = 8 * ii + (lane >> 3);
-            const int piece = (lane & 7) ^ ((d >> 1) & 7);   // keys 8 piece .. + 8 of the step
-            int blk, off;
-            split_key(min(kbase + 8 * piece, (key_hi - 1) & ~7), page, a.page_shift, blk, off);
-            attn_load_to_lds(vp + ((size_t)ATQ_PAGE_OF(blk) * kv_stride + kvh_off + (size_t)d * page + off), sb + ATQ_KBYTES + ii * 1024);
+            const int key = min(kbase + v_key[j], key_last8);
+            const int pg = bt_s[(key >> shift) - blk0];
+            attn_load_to_lds(vp + ((size_t)pg * kv_stride + v_row[j] + (key & pmask)), sb + ATQ_KBYTES + k_dst[j]);
         }
     };
 
@@ -890,24 +911,27 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     // key (within its block of 32) that A row lr of the first product carries
     const int krow = 16 * (lr >> 4) + 8 * ((lr >> 2) & 1) + 4 * ((lr >> 3) & 1) + (lr & 3);
 
-    if (st_first < st_last) request_step(st_first, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // Steps st .. st + ATQ_STAGES - 2 are requested ahead; past the end the last step is requested
+    // again (nobody reads it), so that the number of requests in flight is the same at every wait.
+#pragma unroll
+    for (int i = 0; i < ATQ_STAGES - 1; ++i) request_step(min(st_first + i, st_last - 1), i);
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * K_INSTR * (ATQ_STAGES - 2)) : "memory");
     __syncthreads();
     for (int st = st_first; st < st_last; ++st) {
-        const int buf = (st - st_first) & 1;
-        if (st + 1 < st_last) request_step(st + 1, buf ^ 1);
+        const int buf = (st - st_first) % ATQ_STAGES;
+        request_step(min(st + ATQ_STAGES - 1, st_last - 1), (st - st_first + ATQ_STAGES - 1) % ATQ_STAGES);
         const int kbase = st * ATQ_KEYS;
         unsigned char* kb_s = atq_smem + buf * ATQ_STAGE;
         unsigned char* vb_s = kb_s + ATQ_KBYTES;
         if (kbase + ATQ_KEYS > key_hi) {
             // the last step holds keys that are not written yet: whatever lies in their places in
             // the pages must not reach the second product (0 * Inf), so their values become zero
-            for (int i = threadIdx.x; i < AT_HD * 8; i += 256) {
-                const int d = i >> 3, piece = i & 7;
+            for (int i = threadIdx.x; i < AT_HD * ATQ_VPP; i += 256) {
+                const int d = i / ATQ_VPP, piece = i % ATQ_VPP;
                 const int k0 = kbase + 8 * piece;
                 if (k0 + 8 > key_hi) {
                     FragK f;
-                    uint4* ptr = (uint4*)(vb_s + d * 128 + ((piece ^ ((d >> 1) & 7)) * 16));
+                    uint4* ptr = (uint4*)(vb_s + d * ATQ_VROW + atq_value_slot(piece, d) * 16);
                     f.u = *ptr;
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
@@ -919,9 +943,9 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
         }
         if (wave_has_rows && kbase <= w_pos_max && kbase + ATQ_KEYS > w_lo_min) {
             // ---- scores of two blocks of 32 keys
-            f32x16_t sc[2];
+            f32x16_t sc[ATQ_KB];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+            for (int kb = 0; kb < ATQ_KB; ++kb) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) sc[kb][v] = 0.f;
                 const int kl = 32 * kb + krow;
@@ -937,7 +961,7 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
             float mloc = -INFINITY;
             if (kbase + ATQ_KEYS - 1 <= w_pos_min && kbase >= w_lo_max) {
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < ATQ_KB; ++kb)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         sc[kb][v] *= scale2;
@@ -945,7 +969,7 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
                     }
             } else {
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < ATQ_KB; ++kb)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
                         const int q = e >> 2, v = e & 3;
@@ -959,10 +983,10 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
             const float m_new = fmaxf(m, mloc);
             const float alpha = (m == -INFINITY) ? 0.f : fast_exp2(m - m_new);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;     // nothing seen yet: every score is -inf
-            FragK pf[4];
+            FragK pf[2 * ATQ_KB];
             float psum = 0.f;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < ATQ_KB; ++kb)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const float p = fast_exp2(sc[kb][e] - m_use);
@@ -978,19 +1002,19 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
             }
             // ---- values
 #pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4)
+            for (int c4 = 0; c4 < 2 * ATQ_KB; ++c4)
 #pragma unroll
                 for (int b = 0; b < AT_HD / 32; ++b) {
                     const int d = 32 * b + lr;
                     FragK vf;
-                    vf.u = *(const uint4*)(vb_s + d * 128 + (((2 * c4 + h) ^ ((d >> 1) & 7)) * 16));
+                    vf.u = *(const uint4*)(vb_s + d * ATQ_VROW + atq_value_slot(2 * c4 + h, d) * 16);
                     acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[c4].v, acc[b], 0, 0, 0);
                 }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * K_INSTR * (ATQ_STAGES - 2)) : "memory");
         __syncthreads();
     }
-#undef ATQ_PAGE_OF
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     l += __shfl_xor(l, 32, TL_WAVE);
     if (!row_ok) return;
     // lane holds d = 32 b + 8 q + 4 h + v of its row
@@ -1009,7 +1033,8 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
 #endif
 
 // The 128-row prompt kernel: tiles of `tq` tokens with tq * min(group, 128) <= 128.  Returns an
-// error where it is not built (head sizes other than 64 and 128, pages not a multiple of 8).
+// error where it is not built (head sizes other than 64 and 128, pages that are no power of two from 8 up,
+// block tables wider than tl_paged_attention_prompt_blocks()).
 extern "C" int tl_paged_attention_prompt_rows() {
 #if AT_HD == 64 || AT_HD == 128
     return ATQ_ROWS;
@@ -1018,13 +1043,16 @@ extern "C" int tl_paged_attention_prompt_rows() {
 #endif
 }
 
+extern "C" int tl_paged_attention_prompt_blocks() { return ATM_BT_MAX; }
+
 extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out, const void* k_plane, const void* v_plane,
                                          const void* block_table, int bt_stride, const void* req_indptr, const void* ctx_lens,
                                          const void* tile_req, const void* tile_tok0, int tiles, int tq,
                                          int heads, int kv_heads, int page, int window, float scale, hipStream_t stream) {
 #if AT_HD == 64 || AT_HD == 128
     TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
-    TL_REQUIRE(page > 0 && page % 8 == 0 && bt_stride > 0 && tq > 0 && window >= 0, "attention_prompt: pages of a multiple of 8 tokens, not %d", page);
+    TL_REQUIRE(page >= 8 && (page & (page - 1)) == 0 && tq > 0 && window >= 0, "attention_prompt: pages of 8, 16, 32, ... tokens, not %d", page);
+    TL_REQUIRE(bt_stride > 0 && bt_stride <= ATM_BT_MAX, "attention_prompt: block tables of up to %d entries, not %d", ATM_BT_MAX, bt_stride);
     const int group = heads / kv_heads;
     const int gcap = group < ATQ_ROWS ? group : ATQ_ROWS;
     TL_REQUIRE(tq * gcap <= ATQ_ROWS, "attention_prompt: tile of %d tokens x %d heads exceeds %d rows", tq, gcap, ATQ_ROWS);

@@ -374,9 +374,14 @@ PROMPT_ATTENTION_ROWS = 128      # rows a work-group of the 128-row prompt kerne
 PROMPT_ATTENTION_HEAD_DIMS = (64, 128)
 
 
-def prompt_attention_fits(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
-    """Whether :func:`paged_attention_prompt` is built for this case."""
-    return dtype == torch.bfloat16 and head_dim in PROMPT_ATTENTION_HEAD_DIMS and page_size % 8 == 0
+PROMPT_ATTENTION_MAX_BLOCKS = 2048     # block-table entries a work-group keeps in shared memory
+
+
+def prompt_attention_fits(dtype: torch.dtype, head_dim: int, page_size: int, max_blocks: int = 0) -> bool:
+    """Whether :func:`paged_attention_prompt` is built for this case: bfloat16, head size 64 or
+    128, pages of 8, 16, 32, ... tokens, block tables of up to 2048 entries."""
+    return (dtype == torch.bfloat16 and head_dim in PROMPT_ATTENTION_HEAD_DIMS and page_size >= 8
+            and page_size & (page_size - 1) == 0 and max_blocks <= PROMPT_ATTENTION_MAX_BLOCKS)
 
 
 def prompt_attention_tile_tokens(num_heads: int, num_kv_heads: int) -> int:
@@ -394,8 +399,9 @@ def paged_attention_prompt(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Te
     of a multiple of 8 tokens; keys and values go straight into shared memory once per
     work-group.  Writes the rows of its tiles only."""
     T = q.shape[0]
-    if not prompt_attention_fits(q.dtype, head_dim, page_size):
-        raise KernelError("paged_attention_prompt: bfloat16, head size 64 or 128 and pages of a multiple of 8 tokens only")
+    if not prompt_attention_fits(q.dtype, head_dim, page_size, block_table.shape[1]):
+        raise KernelError("paged_attention_prompt: bfloat16, head size 64 or 128, pages of 8, 16, 32, ... tokens and block "
+                          f"tables of up to {PROMPT_ATTENTION_MAX_BLOCKS} entries only")
     if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
         raise KernelError("paged_attention_prompt: q/out shapes or dtypes do not fit")
     _check_planes("paged_attention_prompt", k_plane, v_plane, q.dtype, num_kv_heads, page_size, head_dim)

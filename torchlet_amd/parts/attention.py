@@ -22,7 +22,7 @@ from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedNeed, WeightSpec
 _TARGET_WORKGROUPS = 512     # enough work-groups to fill 256 compute units twice
 _MIN_KEYS_PER_SPLIT = 256
 _PORTION_MIN_TOKENS = 16     # requests that bring at least this many tokens go to a prompt-portion kernel: the
-                             # 128-row one where it is built (head size 64 or 128, pages of a multiple of 8
+                             # 128-row one where it is built (head size 64 or 128, pages of 8, 16, 32, ...
                              # tokens; measured on MI355X at 28/4 heads of 128: 2048 new tokens 222 -> 110 us,
                              # 8192 new tokens 2.9 -> 0.84 ms), else the 64-row one ...
 _PORTION_MIN_CONTEXT = 4096  # ... which pays only in steps whose longest sequence has at least this many tokens
@@ -126,7 +126,7 @@ class GQAttention(Mixer):
         out = torch.empty((T, self.q_width), dtype=self.dtype, device=h.device)
         q = qkv[:, : self.q_width]
         common = (self.heads, self.kv_heads, self.head_dim, cache.page_size, self.window or 0, self.scale)
-        rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size)
+        rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size, table.shape[1])
                    and ctx.max_new_tokens >= _PORTION_MIN_TOKENS)
         portions = (self.dtype == torch.bfloat16 and self.head_dim <= ops.PREFILL_ATTENTION_MAX_HEAD_DIM
                     and cache.page_size % 4 == 0 and ctx.max_new_tokens >= _PORTION_MIN_TOKENS

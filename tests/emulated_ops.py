@@ -47,16 +47,25 @@ def linear(x, weight, bias, out, general=False):
     out.copy_(y.to(out.dtype))
 
 
+def linear_rope_cache_write(*args, **kwargs):
+    return False          # not fused here: the caller runs the product and the rotation one after the other
+
+
 def rope_cache_write(qkv, q_heads, kv_heads, head_dim, rot_heads, positions, inv_freq,
-                     token_req=None, block_table=None, k_plane=None, v_plane=None, page_size=0):
+                     token_req=None, block_table=None, k_plane=None, v_plane=None, page_size=0, pairs=False):
     T = qkv.shape[0]
     x = qkv[:, : (q_heads + kv_heads) * head_dim].float().view(T, q_heads + kv_heads, head_dim)
     if inv_freq is not None:
         ang = positions.float()[:, None] * inv_freq[None, :]
         c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
         half = head_dim // 2
-        x1, x2 = x[:, :rot_heads, :half], x[:, :rot_heads, half:]
-        x = torch.cat((torch.cat((x1 * c - x2 * s, x2 * c + x1 * s), -1), x[:, rot_heads:]), 1)
+        if pairs:
+            x1, x2 = x[:, :rot_heads, 0::2], x[:, :rot_heads, 1::2]
+            turned = torch.stack((x1 * c - x2 * s, x2 * c + x1 * s), -1).reshape(T, rot_heads, head_dim)
+        else:
+            x1, x2 = x[:, :rot_heads, :half], x[:, :rot_heads, half:]
+            turned = torch.cat((x1 * c - x2 * s, x2 * c + x1 * s), -1)
+        x = torch.cat((turned, x[:, rot_heads:]), 1)
         qkv[:, : (q_heads + kv_heads) * head_dim] = x.reshape(T, -1).to(qkv.dtype)
     if k_plane is not None:
         k = qkv[:, q_heads * head_dim: (q_heads + kv_heads) * head_dim].view(T, kv_heads, head_dim)

@@ -264,6 +264,91 @@ def test_rope_cache_write(ops, dtype, nh, nkv, hd, page, theta):
     assert float(d_kp[0].abs().sum()) == 0.0                # page 0 is never written
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,page,theta", [(4, 2, 16, 16, 1e4), (28, 4, 128, 16, 1e6), (5, 5, 48, 4, 5e5)])
+def test_rope_cache_write_in_the_pair_layout(ops, dtype, nh, nkv, hd, page, theta):
+    """With the dimensions of every head reordered so that the two that a frequency turns are
+    neighbours, the kernel's pair mode gives the reordered result of the usual rotation."""
+    g = torch.Generator().manual_seed(6)
+    lens, ctxs = [5, 1, 11], [0, 37, 6]
+    T = sum(lens)
+    max_blocks = (max(a + b for a, b in zip(lens, ctxs)) + page - 1) // page
+    pages = 3 * max_blocks + 2
+    qkv = torch.randn(T, (nh + 2 * nkv) * hd, generator=g).to(dtype)
+    positions = torch.cat([torch.arange(c, c + n) for n, c in zip(lens, ctxs)]).int()
+    token_req = torch.cat([torch.full((n,), r) for r, n in enumerate(lens)]).int()
+    bt = (torch.randperm(pages - 1, generator=g)[: 3 * max_blocks] + 1).view(3, max_blocks).int()
+    inv_freq = 1.0 / (theta ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))
+    order = torch.cat((ops.pair_layout_rows(nh + nkv, hd), (nh + nkv) * hd + torch.arange(nkv * hd)))    # values keep their order
+    outs = []
+    for pairs, src in ((False, qkv), (True, qkv[:, order].contiguous())):
+        d_qkv = src.cuda()
+        d_kp = torch.zeros(pages, nkv, page, hd, dtype=dtype, device="cuda")
+        d_vp = torch.zeros(pages, nkv, hd, page, dtype=dtype, device="cuda")
+        ops.rope_cache_write(d_qkv, nh, nkv, hd, nh + nkv, positions.cuda(), inv_freq.cuda(), token_req.cuda(), bt.cuda(), d_kp, d_vp, page, pairs=pairs)
+        outs.append((d_qkv.cpu(), d_kp.cpu(), d_vp.cpu()))
+    (plain_qkv, plain_k, plain_v), (pair_qkv, pair_k, pair_v) = outs
+    korder = ops.pair_layout_rows(1, hd)
+    assert torch.equal(pair_qkv, plain_qkv[:, order])
+    assert torch.equal(pair_k, plain_k[..., korder])
+    assert torch.equal(pair_v, plain_v)
+
+
+@pytest.mark.parametrize("M", [1, 2, 8, 16])
+@pytest.mark.parametrize("nh,nkv,hd,page,hidden,bias", [(28, 4, 128, 16, 3584, True), (4, 2, 16, 8, 64, False), (14, 2, 64, 16, 896, True),
+                                                        (40, 8, 128, 32, 5120, True), (5, 5, 48, 16, 240, True)])
+def test_projection_with_rotation_and_cache_write_in_its_epilogue(ops, M, nh, nkv, hd, page, hidden, bias):
+    """The fused query/key/value projection of a decode step against the product, the rotation and
+    the cache write done one after the other."""
+    g = torch.Generator().manual_seed(M + nh)
+    T = M
+    ctxs = [int(c) for c in torch.randint(0, 90, (T,), generator=g)]
+    max_blocks = (max(ctxs) + 1 + page - 1) // page
+    pages = T * max_blocks + 2
+    width = (nh + 2 * nkv) * hd
+    x = torch.randn(T, hidden, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(width, hidden, generator=g) / math.sqrt(hidden)).to(torch.bfloat16).cuda()
+    b = torch.randn(width, generator=g).to(torch.bfloat16).cuda() if bias else None
+    positions = torch.tensor(ctxs, dtype=torch.int32).cuda()
+    token_req = torch.arange(T, dtype=torch.int32).cuda()
+    bt = (torch.randperm(pages - 1, generator=g)[: T * max_blocks] + 1).view(T, max_blocks).int().cuda()
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))).cuda()
+
+    def planes():
+        return (torch.zeros(pages, nkv, page, hd, dtype=torch.bfloat16, device="cuda"),
+                torch.zeros(pages, nkv, hd, page, dtype=torch.bfloat16, device="cuda"))
+    ref = torch.empty(T, width, dtype=torch.bfloat16, device="cuda")
+    ops.linear(x, w, b, ref)
+    rk, rv = planes()
+    ops.rope_cache_write(ref, nh, nkv, hd, nh + nkv, positions, inv_freq, token_req, bt, rk, rv, page, pairs=True)
+    got = torch.full((T, width), float("nan"), dtype=torch.bfloat16, device="cuda")
+    gk, gv = planes()
+    fused = ops.linear_rope_cache_write(x, w, b, got, nh, nkv, hd, positions, inv_freq, token_req, bt, gk, gv, page)
+    assert fused
+    # against the exact product and rotation: the fused kernel rounds once, to bfloat16, at the end
+    # (half an ulp, 2^-9 of the value; 2^-8 allowed), on top of the 32-bit sums' own error
+    exact = x.double().cpu() @ w.double().cpu().T + (b.double().cpu() if bias else 0.0)
+    heads = exact[:, : (nh + nkv) * hd].view(T, nh + nkv, hd)
+    ang = (positions.cpu().float()[:, None] * inv_freq.cpu()[None, :]).double()[:, None, :]
+    a, c = heads[..., 0::2], heads[..., 1::2]
+    turned = torch.stack((a * ang.cos() - c * ang.sin(), c * ang.cos() + a * ang.sin()), -1).reshape(T, nh + nkv, hd)
+    tol = dict(rtol=2 ** -8, atol=1e-5 * float(exact.abs().max()))
+    torch.testing.assert_close(got[:, : nh * hd].double().cpu(), turned[:, :nh].reshape(T, -1), **tol)
+    for t in range(T):
+        pg, off = int(bt[t, ctxs[t] // page]), ctxs[t] % page
+        torch.testing.assert_close(gk[pg, :, off].double().cpu(), turned[t, nh:], **tol)
+    # and next to the two-kernel path, which rounds twice: a whole ulp apart at most
+    loose = dict(rtol=2 ** -6, atol=2 ** -7 * float(exact.abs().max()))
+    torch.testing.assert_close(got[:, : nh * hd].float(), ref[:, : nh * hd].float(), **loose)
+    torch.testing.assert_close(gk.float(), rk.float(), **loose)
+    assert torch.equal(gv, rv)
+    assert float(gk[0].abs().sum()) == 0.0 and float(gv[0].abs().sum()) == 0.0
+    # queries alone, as a run that reads another run's cache asks for them
+    q_only = torch.empty(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+    assert ops.linear_rope_cache_write(x, w[: nh * hd], None if b is None else b[: nh * hd], q_only, nh, nkv, hd, positions, inv_freq)
+    assert torch.equal(q_only, got[:, : nh * hd])
+
+
 def _attention_ref(q, k, v, window):
     """One request: q [n, heads, hd] at positions ctx..ctx+n-1, k/v [ctx+n, kvh, hd] (float64)."""
     n, heads, hd = q.shape

@@ -198,7 +198,8 @@ extern "C" int tl_add_rmsnorm(void* residual, const void* pending, int parts, in
 // One wave per token and head.  Row layout of `qkv`: [q heads | k heads | v heads], each head
 // `head_dim` wide, row stride `row_stride` elements.
 //   * rotate (inv_freq != null): the first `rot_heads` heads (q, then k) are rotated in
-//     place with the split-half pairing (j, j + head_dim/2) by angle = float(pos) * inv_freq[j].
+//     place with the split-half pairing (j, j + head_dim/2) by angle = float(pos) * inv_freq[j];
+//     with `pairs` the two elements of frequency j are the neighbours (2j, 2j + 1) instead.
 //   * write (k_plane != null): rotated k and raw v of the token go to the page
 //     block_table[token_req[t]][pos / page] at offset pos % page.  The key plane is
 //     [pages, kv_heads, page, head_dim]; the value plane holds each page transposed,
@@ -210,7 +211,7 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
                              int head_dim, int rot_heads, const int* __restrict__ positions,
                              const float* __restrict__ inv_freq, const int* __restrict__ token_req,
                              const int* __restrict__ block_table, int bt_stride,
-                             T* __restrict__ k_plane, T* __restrict__ v_plane, int page_size) {
+                             T* __restrict__ k_plane, T* __restrict__ v_plane, int page_size, int pairs) {
     // A wave owns one head of one token: a query head (rotated in place), a key head (rotated in
     // place and written to its page) or a value head (written to its page, transposed).  Each wave
     // takes the cosines and sines of its own pairs, so no wave waits for another.
@@ -237,7 +238,10 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
     const bool rotate = inv_freq && head < rot_heads;
     if (!rotate && !dst) return;
     for (int j = lane; j < half; j += TL_WAVE) {
-        float x1 = to_float(x[j]), x2 = to_float(x[j + half]);
+        // the two elements that frequency j turns: (j, j + half), or neighbours (2j, 2j + 1) in the
+        // pair layout (a projection whose rows were reordered that way at load time)
+        const int i1 = pairs ? 2 * j : j, i2 = pairs ? 2 * j + 1 : j + half;
+        float x1 = to_float(x[i1]), x2 = to_float(x[i2]);
         if (rotate) {
             const float angle = (float)pos * inv_freq[j];
             const float c = cosf(angle), sn = sinf(angle);
@@ -245,12 +249,12 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
             const float y2 = x2 * c + x1 * sn;
             x1 = y1;
             x2 = y2;
-            x[j] = from_float<T>(x1);
-            x[j + half] = from_float<T>(x2);
+            x[i1] = from_float<T>(x1);
+            x[i2] = from_float<T>(x2);
         }
         if (dst) {
-            dst[j] = from_float<T>(x1);
-            dst[j + half] = from_float<T>(x2);
+            dst[i1] = from_float<T>(x1);
+            dst[i2] = from_float<T>(x2);
         }
     }
 }
@@ -258,7 +262,7 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
 extern "C" int tl_rope_cache_write(void* qkv, int row_stride, int tokens, int q_heads, int kv_heads,
                                    int head_dim, int rot_heads, const void* positions, const void* inv_freq,
                                    const void* token_req, const void* block_table, int bt_stride,
-                                   void* k_plane, void* v_plane, int page_size, int act_dtype,
+                                   void* k_plane, void* v_plane, int page_size, int pairs, int act_dtype,
                                    hipStream_t stream) {
     TL_REQUIRE(tokens >= 0 && q_heads >= 0 && kv_heads >= 0 && head_dim > 0 && head_dim % 2 == 0 && head_dim <= 256,
                "rope_cache_write: bad sizes tokens=%d q_heads=%d kv_heads=%d head_dim=%d (even, at most 256)", tokens, q_heads, kv_heads, head_dim);
@@ -274,11 +278,11 @@ extern "C" int tl_rope_cache_write(void* qkv, int row_stride, int tokens, int q_
     if (act_dtype == TL_DT_F32)
         rope_cache_write_kernel<float><<<grid, block, 0, stream>>>((float*)qkv, row_stride, q_heads, kv_heads, head_dim, rot_heads,
             (const int*)positions, (const float*)inv_freq, (const int*)token_req, (const int*)block_table, bt_stride,
-            (float*)k_plane, (float*)v_plane, page_size);
+            (float*)k_plane, (float*)v_plane, page_size, pairs);
     else if (act_dtype == TL_DT_BF16)
         rope_cache_write_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)qkv, row_stride, q_heads, kv_heads, head_dim, rot_heads,
             (const int*)positions, (const float*)inv_freq, (const int*)token_req, (const int*)block_table, bt_stride,
-            (bf16_t*)k_plane, (bf16_t*)v_plane, page_size);
+            (bf16_t*)k_plane, (bf16_t*)v_plane, page_size, pairs);
     else TL_REQUIRE(false, "rope_cache_write: unknown dtype %d", act_dtype);
     TL_CHECK_LAUNCH("rope_cache_write");
     return TL_OK;

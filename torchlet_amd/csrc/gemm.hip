@@ -142,12 +142,27 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + 
 // its M rows of x into shared memory once, coalesced, and reads the operands from there.
 // D: how many K steps of weights a wave keeps in flight (a ring of D register sets).  Short
 // rows (a few steps per wave) want them all in flight at once, or every step costs a trip to memory.
-template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false, int D = 2>
+// RP (the fused query/key/value projection of a decode step, R == 1 and MT == 1): the epilogue rotates
+// the query and key heads by the token's position and puts keys and values into their pages, so no
+// kernel of its own has to.  The projection's rows are in the pair layout: the two elements that
+// frequency j turns are the neighbouring output columns 2j and 2j + 1 of a head, both in one lane.
+struct RopeArgs {
+    const int* positions;      // [M]
+    const float* inv_freq;     // [head_dim / 2]
+    const int* token_req;      // [M] request of each row (null: no cache write)
+    const int* block_table;    // [requests, bt_stride]
+    bf16_t* k_plane;           // [pages, kv_heads, page, head_dim]
+    bf16_t* v_plane;           // [pages, kv_heads, head_dim, page]
+    int bt_stride, page, q_heads, kv_heads, head_dim;
+};
+
+template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false, int D = 2, bool RP = false>
 __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                               const void* __restrict__ bias, int bias_f32,
                                                               TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-                                                              int out_cols = 0, int k_per_split = 0) {
+                                                              int out_cols, int k_per_split, RopeArgs ra) {
     static_assert(!SW || (R == 4 && KS > 1), "the fused gate needs four strips per work-group");
+    static_assert(!RP || (R == 1 && MT == 1 && !SW), "the fused rotation is built for one strip and up to 16 rows");
     // Split K (k_per_split > 0, a multiple of 64): blockIdx.y owns the columns
     // [y * k_per_split, ...) of x and w and writes its own [M, ldo] slab of partial sums to out
     // (float, no bias); whoever reads them adds the slabs up.
@@ -165,6 +180,12 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
     const int n0 = blockIdx.x * (16 * R);
+    int rp_pos = 0, rp_page = 0;               // RP: this lane's row (li), fetched now, used in the epilogue
+    if (RP) {
+        const int row = min(li, M - 1);
+        rp_pos = ra.positions[row];
+        if (ra.k_plane) rp_page = ra.block_table[(size_t)ra.token_req[row] * ra.bt_stride + rp_pos / ra.page];
+    }
 
     const bf16_t* wrow[R];
     const bf16_t* xrow[MT];
@@ -309,6 +330,40 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
         }
         const int m = t * 16 + li;
         const int n = n0 + r * 16 + 4 * lg;
+        if (RP) {
+            if (m >= M || n >= N) continue;                    // N is a multiple of 16 here
+            float val[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) val[v] = sum[v] + (bias ? load_vec(bias, bias_f32, n + v) : 0.f);
+            const int head = n / ra.head_dim, dd = n - head * ra.head_dim;
+            if (head < ra.q_heads + ra.kv_heads) {
+#pragma unroll
+                for (int pr = 0; pr < 2; ++pr) {
+                    const float angle = (float)rp_pos * ra.inv_freq[dd / 2 + pr];
+                    const float c = cosf(angle), sn = sinf(angle);
+                    const float y1 = val[2 * pr] * c - val[2 * pr + 1] * sn;
+                    const float y2 = val[2 * pr + 1] * c + val[2 * pr] * sn;
+                    val[2 * pr] = y1;
+                    val[2 * pr + 1] = y2;
+                }
+            }
+            union { uint2 u; uint16_t e[4]; } pk;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(val[v]).bits;
+            if (head < ra.q_heads || !ra.k_plane) {
+                *(uint2*)((bf16_t*)out + (size_t)m * ldo + n) = pk.u;
+            } else {
+                const int kvh = (head - ra.q_heads) % ra.kv_heads, off = rp_pos % ra.page;
+                const size_t base = ((size_t)rp_page * ra.kv_heads + kvh) * ra.page * ra.head_dim;
+                if (head < ra.q_heads + ra.kv_heads) {
+                    *(uint2*)(ra.k_plane + base + (size_t)off * ra.head_dim + dd) = pk.u;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) ra.v_plane[base + (size_t)(dd + v) * ra.page + off].bits = pk.e[v];
+                }
+            }
+            continue;
+        }
         if (m < M) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
@@ -344,11 +399,11 @@ static void launch_skinny_d(const void* x, const void* w, const void* bias, int 
         auto kernel = gemm_skinny_kernel<R, MT, KS, TOut, SW, true, D>;
         static hipError_t allowed = allow_lds(kernel, 96 * 1024);
         if (allowed == hipSuccess) {
-            kernel<<<grid, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0);
+            kernel<<<grid, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{});
             return;
         }
     }
-    gemm_skinny_kernel<R, MT, KS, TOut, SW, false, D><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0);
+    gemm_skinny_kernel<R, MT, KS, TOut, SW, false, D><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{});
 }
 
 // A wave with many K steps ahead of it (a long K: the down projection) keeps as many in flight as
@@ -902,6 +957,45 @@ extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_
     return tl_gemm_general(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, dtype, out_f32, stream);
 }
 
+// The fused query/key/value projection of up to 16 rows: out[:, :q_heads * head_dim] = rotated queries,
+// rotated keys and values go to their pages (see RopeArgs; the weight rows of every query and key head
+// are in the pair layout).  Returns TL_NOT_FUSED (nothing launched) for shapes it is not built for;
+// the caller then runs the product and the rotation as two kernels.
+#define TL_NOT_FUSED 100
+template <int KS, bool XL>
+static void launch_skinny_rope(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                               int ldx, int ldo, const RopeArgs& ra, hipStream_t stream) {
+    dim3 grid((N + 15) / 16), block(KS * 64);
+    const size_t lds = (size_t)KS * 1024 + (XL ? (size_t)M * (K + 8) * 2 : 0);
+    auto kernel = gemm_skinny_kernel<1, 1, KS, bf16_t, false, XL, 2, true>;
+    if (XL) { static hipError_t allowed = allow_lds(kernel, 96 * 1024); (void)allowed; }
+    kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo, 0, 0, ra);
+}
+
+extern "C" int tl_gemm_rope(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                            int ldx, int ldo, const void* positions, const void* inv_freq, const void* token_req,
+                            const void* block_table, int bt_stride, void* k_plane, void* v_plane, int page,
+                            int q_heads, int kv_heads, int head_dim, hipStream_t stream) {
+    TL_REQUIRE(M > 0 && N > 0 && K > 0 && ldx >= K && ldo >= q_heads * head_dim, "gemm_rope: bad sizes M=%d N=%d K=%d", M, N, K);
+    TL_REQUIRE(positions && inv_freq && head_dim % 4 == 0 && q_heads >= 0 && kv_heads >= 0, "gemm_rope: needs positions, frequencies and a head size that is a multiple of 4");
+    TL_REQUIRE((k_plane == nullptr) == (v_plane == nullptr) && (!k_plane || (token_req && block_table && page > 0 && bt_stride > 0)),
+               "gemm_rope: the cache write needs both planes, the block table and the requests of the rows");
+    TL_REQUIRE(N == (q_heads + (k_plane ? 2 * kv_heads : 0)) * head_dim, "gemm_rope: %d output columns do not match the heads", N);
+    const int strips = (N + 15) / 16, ks = strips >= 1024 ? 16 : 8;
+    if (M > 16 || !skinny_fits(x, w, M, K, ldx) || N % 16 || ldo % 4 || ((uintptr_t)out % 8) || K / 64 / ks >= 16 ||
+        (k_plane && (((uintptr_t)k_plane % 8) || head_dim % 4)))
+        return TL_NOT_FUSED;
+    RopeArgs ra;
+    ra.positions = (const int*)positions; ra.inv_freq = (const float*)inv_freq; ra.token_req = (const int*)token_req;
+    ra.block_table = (const int*)block_table; ra.k_plane = (bf16_t*)k_plane; ra.v_plane = (bf16_t*)v_plane;
+    ra.bt_stride = bt_stride; ra.page = page > 0 ? page : 1; ra.q_heads = q_heads; ra.kv_heads = k_plane ? kv_heads : 0; ra.head_dim = head_dim;
+    const bool xl = M > 1 && (size_t)M * (K + 8) * 2 <= SKINNY_XL_MAX_BYTES;
+    if (ks == 8) { if (xl) launch_skinny_rope<8, true>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); else launch_skinny_rope<8, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); }
+    else { if (xl) launch_skinny_rope<16, true>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); else launch_skinny_rope<16, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); }
+    TL_CHECK_LAUNCH("gemm_rope");
+    return TL_OK;
+}
+
 // out[M, I] = silu(x g^T) * (x u^T) for bfloat16, with w = the gate and up matrices interleaved
 // in blocks of 32 rows (rows 64 b .. 64 b + 31: gate rows 32 b .., rows 64 b + 32 ..: the up rows
 // of the same columns), padded with zero rows to a multiple of 64.  The gate is applied to the
@@ -958,14 +1052,14 @@ extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, 
     dim3 grid((N + 63) / 64, P), block(8 * 64);
     const size_t red_bytes = (size_t)8 * 4 * (M <= 16 ? 1 : (M <= 32 ? 2 : 4)) * 1024;
     if (M <= 16)
-        gemm_skinny_kernel<4, 1, 8, float, false, false, skinny_depth<4, 1, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
+        gemm_skinny_kernel<4, 1, 8, float, false, false, skinny_depth<4, 1, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{});
     else if (M <= 32)
-        gemm_skinny_kernel<4, 2, 8, float, false, false, skinny_depth<4, 2, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
+        gemm_skinny_kernel<4, 2, 8, float, false, false, skinny_depth<4, 2, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{});
     else {
         auto kernel = gemm_skinny_kernel<4, 4, 8, float, false, false, skinny_depth<4, 4, 8>()>;
         static hipError_t allowed = allow_lds(kernel, 128 * 1024);
         TL_REQUIRE(allowed == hipSuccess, "gemm_partials: cannot get %zu bytes of shared memory", red_bytes);
-        kernel<<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per);
+        kernel<<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{});
     }
     TL_CHECK_LAUNCH("gemm_partials");
     return TL_OK;

@@ -252,9 +252,10 @@ def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: i
                      positions: torch.Tensor, inv_freq: torch.Tensor | None,
                      token_req: torch.Tensor | None = None, block_table: torch.Tensor | None = None,
                      k_plane: torch.Tensor | None = None, v_plane: torch.Tensor | None = None,
-                     page_size: int = 0) -> None:
+                     page_size: int = 0, pairs: bool = False) -> None:
     """Rotate the first ``rot_heads`` heads of each row of ``qkv [T, >= (q+2kv)*hd]`` in
-    place by the token's position (``inv_freq`` float32 ``[hd/2]``; ``None``: no rotation)
+    place by the token's position (``inv_freq`` float32 ``[hd/2]``; ``None``: no rotation;
+    ``pairs``: frequency j turns the neighbours ``(2j, 2j+1)`` instead of ``(j, j+hd/2)``)
     and, when planes are given, store rotated k and raw v of every token in its page:
     ``k_plane [pages, kv_heads, page, hd]``, ``v_plane [pages, kv_heads, hd, page]`` (values
     lie transposed inside a page)."""
@@ -274,7 +275,56 @@ def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: i
     _check(lib, lib.tl_rope_cache_write(_ptr(qkv), c_int(qkv.stride(0)), c_int(T), c_int(q_heads), c_int(kv_heads),
                                         c_int(head_dim), c_int(rot_heads), _ptr(positions), _ptr(inv_freq), _ptr(token_req),
                                         _ptr(block_table), c_int(bt_stride), _ptr(k_plane), _ptr(v_plane), c_int(page_size),
-                                        c_int(_dt(qkv, "rope_cache_write")), _stream()))
+                                        c_int(1 if pairs else 0), c_int(_dt(qkv, "rope_cache_write")), _stream()))
+
+
+def pair_layout_rows(num_heads: int, head_dim: int) -> torch.Tensor:
+    """Row order that turns a projection into the pair layout: within every head the rows
+    ``j`` and ``j + head_dim/2`` (the two that frequency ``j`` of the split-half rotary encoding
+    turns) become the neighbours ``2j`` and ``2j + 1``.  Scores are sums over the head's
+    dimensions, so they do not change when queries and keys are reordered alike."""
+    half = head_dim // 2
+    within = torch.stack((torch.arange(half), torch.arange(half) + half), dim=1).reshape(-1)
+    return (torch.arange(num_heads)[:, None] * head_dim + within[None, :]).reshape(-1)
+
+
+def linear_rope_cache_write(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor,
+                            q_heads: int, kv_heads: int, head_dim: int, positions: torch.Tensor, inv_freq: torch.Tensor,
+                            token_req: torch.Tensor | None = None, block_table: torch.Tensor | None = None,
+                            k_plane: torch.Tensor | None = None, v_plane: torch.Tensor | None = None,
+                            page_size: int = 0) -> bool:
+    """The query/key/value projection of a decode step with the rotation and the cache write in
+    its epilogue: ``out[:, :q_heads*hd]`` gets the rotated queries; with planes given, ``weight``
+    has ``(q_heads + 2 kv_heads) * hd`` rows and rotated keys and values go to their pages.  The
+    rows of the query and key heads are in the pair layout (:func:`pair_layout_rows`).  Built
+    for bfloat16 and up to 16 rows; returns ``False`` without doing anything for other shapes."""
+    M, K = x.shape
+    N = weight.shape[0]
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or M > 16 or M == 0:
+        return False
+    if x.stride(1) != 1 or out.stride(1) != 1 or not weight.is_contiguous() or weight.shape[1] != K or out.shape[0] != M:
+        raise KernelError("linear_rope_cache_write: shapes or strides do not fit")
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() != head_dim // 2:
+        raise KernelError("linear_rope_cache_write: inv_freq must be float32 [head_dim/2]")
+    _i32(positions, "positions", M)
+    bt_stride = 0
+    if k_plane is not None:
+        _i32(token_req, "token_req", M)
+        _i32(block_table, "block_table")
+        bt_stride = block_table.stride(0)
+        _check_planes("linear_rope_cache_write", k_plane, v_plane, x.dtype, kv_heads, page_size, head_dim)
+    if N != (q_heads + (2 * kv_heads if k_plane is not None else 0)) * head_dim or out.shape[1] < q_heads * head_dim:
+        raise KernelError("linear_rope_cache_write: the projection's rows do not match the heads")
+    bf = _vec(bias, N, "linear bias")
+    lib = _lib("gemm")
+    rc = lib.tl_gemm_rope(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N), c_int(K),
+                          c_int(x.stride(0)), c_int(out.stride(0)), _ptr(positions), _ptr(inv_freq), _ptr(token_req),
+                          _ptr(block_table), c_int(bt_stride), _ptr(k_plane), _ptr(v_plane), c_int(page_size),
+                          c_int(q_heads), c_int(kv_heads), c_int(head_dim), _stream())
+    if rc == 100:          # not built for this shape
+        return False
+    _check(lib, rc)
+    return True
 
 
 def _check_planes(what, k_plane, v_plane, dtype, kv_heads, page_size, head_dim) -> None:

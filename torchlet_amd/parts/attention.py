@@ -53,6 +53,7 @@ class GQAttention(Mixer):
         self.tile_tokens = ops.attention_tile_tokens(self.heads, self.kv_heads)
         self.portion_tile_tokens = ops.prefill_attention_tile_tokens(self.heads, self.kv_heads)
         self.prompt_tile_tokens = ops.prompt_attention_tile_tokens(self.heads, self.kv_heads)
+        self.pair_layout = False      # set when the weights are loaded
         self.w_qkv: torch.Tensor | None = None
         self.b_qkv: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
@@ -78,9 +79,17 @@ class GQAttention(Mixer):
         return specs
 
     def load_weights(self, tensors):
-        self.w_qkv = self._place(torch.cat([tensors[f"{n}_proj.weight"] for n in "qkv"], dim=0), "matrix")
+        # The bfloat16 engine keeps the rows of the query and key projections in the pair layout, in
+        # which the rotary encoding turns neighbouring dimensions: the projection of a decode step
+        # then rotates in its own epilogue.  Keys lie in the cache in that order too; scores are
+        # sums over a head's dimensions and do not notice.
+        self.pair_layout = (self.dtype == torch.bfloat16 and self.position is not None
+                            and hasattr(self.position, "fused_inv_freq"))
+        rows = {"q": ops.pair_layout_rows(self.heads, self.head_dim), "k": ops.pair_layout_rows(self.kv_heads, self.head_dim)}
+        order = lambda n, t: t[rows[n]] if self.pair_layout and n in rows else t
+        self.w_qkv = self._place(torch.cat([order(n, tensors[f"{n}_proj.weight"]) for n in "qkv"], dim=0), "matrix")
         if self.qkv_bias:
-            biases = [tensors[f"{n}_proj.bias"] for n in "qkv"]
+            biases = [order(n, tensors[f"{n}_proj.bias"]) for n in "qkv"]
             if len({b.dtype for b in biases}) > 1:
                 biases = [b.to(torch.float32) for b in biases]
             self.b_qkv = self._place(torch.cat(biases), "vector")
@@ -104,7 +113,6 @@ class GQAttention(Mixer):
         w = self.w_qkv if writes else self.w_qkv[: self.q_width]
         b = self.b_qkv if (self.b_qkv is None or writes) else self.b_qkv[: self.q_width]
         qkv = torch.empty((T, width), dtype=self.dtype, device=h.device)
-        ops.linear(h, w, b, qkv)
 
         # the cache hands out two planes of [pages, kv_heads, page, head_dim]; this mixer keeps the
         # values of a page transposed, [kv_heads, head_dim, page], as its kernels read them
@@ -113,15 +121,18 @@ class GQAttention(Mixer):
         table = ctx.block_tables[cache.group]
         kv_heads = self.kv_heads if writes else 0
         inv_freq = self.position.fused_inv_freq() if hasattr(self.position, "fused_inv_freq") else None
-        if self.position is not None and inv_freq is None:
-            q3 = qkv[:, : self.q_width].unflatten(1, (self.heads, self.head_dim))
-            k3 = qkv[:, self.q_width: self.q_width + self.kv_width].unflatten(1, (self.kv_heads, self.head_dim)) if writes else None
-            self.position.apply(q3, k3, ctx.positions)
-        if inv_freq is not None or writes:
-            ops.rope_cache_write(
-                qkv, self.heads, kv_heads, self.head_dim, self.heads + kv_heads, ctx.positions, inv_freq,
-                ctx.token_req if writes else None, table if writes else None,
-                k_plane if writes else None, v_plane if writes else None, cache.page_size if writes else 0)
+        cache_args = (ctx.token_req, table, k_plane, v_plane, cache.page_size) if writes else (None, None, None, None, 0)
+        fused = self.pair_layout and ops.linear_rope_cache_write(h, w, b, qkv, self.heads, self.kv_heads, self.head_dim,
+                                                                 ctx.positions, inv_freq, *cache_args)
+        if not fused:
+            ops.linear(h, w, b, qkv)
+            if self.position is not None and inv_freq is None:
+                q3 = qkv[:, : self.q_width].unflatten(1, (self.heads, self.head_dim))
+                k3 = qkv[:, self.q_width: self.q_width + self.kv_width].unflatten(1, (self.kv_heads, self.head_dim)) if writes else None
+                self.position.apply(q3, k3, ctx.positions)
+            if inv_freq is not None or writes:
+                ops.rope_cache_write(qkv, self.heads, kv_heads, self.head_dim, self.heads + kv_heads, ctx.positions, inv_freq,
+                                     *cache_args, pairs=self.pair_layout)
 
         out = torch.empty((T, self.q_width), dtype=self.dtype, device=h.device)
         q = qkv[:, : self.q_width]

@@ -211,7 +211,7 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
                              int head_dim, int rot_heads, const int* __restrict__ positions,
                              const float* __restrict__ inv_freq, const int* __restrict__ token_req,
                              const int* __restrict__ block_table, int bt_stride,
-                             T* __restrict__ k_plane, T* __restrict__ v_plane, int page_size, int pairs) {
+                             T* __restrict__ k_plane, T* __restrict__ v_plane, int page_size, int pairs, int pair_aligned) {
     // A wave owns one head of one token: a query head (rotated in place), a key head (rotated in
     // place and written to its page) or a value head (written to its page, transposed).  Each wave
     // takes the cosines and sines of its own pairs, so no wave waits for another.
@@ -237,6 +237,27 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
     }
     const bool rotate = inv_freq && head < rot_heads;
     if (!rotate && !dst) return;
+    if (pairs && pair_aligned) {
+        // pair layout: the two elements of a frequency are one aligned load and one aligned store
+        struct __attribute__((aligned(2 * sizeof(T)))) Two { T a, b; };
+        for (int j = lane; j < half; j += TL_WAVE) {
+            Two p = *(const Two*)(x + 2 * j);
+            float x1 = to_float(p.a), x2 = to_float(p.b);
+            if (rotate) {
+                const float angle = (float)pos * inv_freq[j];
+                const float c = cosf(angle), sn = sinf(angle);
+                const float y1 = x1 * c - x2 * sn;
+                const float y2 = x2 * c + x1 * sn;
+                x1 = y1;
+                x2 = y2;
+            }
+            p.a = from_float<T>(x1);
+            p.b = from_float<T>(x2);
+            if (rotate) *(Two*)(x + 2 * j) = p;
+            if (dst) *(Two*)(dst + 2 * j) = p;
+        }
+        return;
+    }
     for (int j = lane; j < half; j += TL_WAVE) {
         // the two elements that frequency j turns: (j, j + half), or neighbours (2j, 2j + 1) in the
         // pair layout (a projection whose rows were reordered that way at load time)
@@ -274,15 +295,17 @@ extern "C" int tl_rope_cache_write(void* qkv, int row_stride, int tokens, int q_
                "rope_cache_write: row stride %d too small", row_stride);
     if (tokens == 0) return TL_OK;
     const int heads = q_heads + kv_heads + (k_plane ? kv_heads : 0);
+    // pairs as one access: rows and planes start on a multiple of two elements (eight bytes covers both dtypes)
+    const int pair_aligned = row_stride % 2 == 0 && ((uintptr_t)qkv % 8) == 0 && ((uintptr_t)k_plane % 8) == 0;
     dim3 grid(tokens, (heads + ROPE_HEADS_PER_GROUP - 1) / ROPE_HEADS_PER_GROUP), block(ROPE_HEADS_PER_GROUP * TL_WAVE);
     if (act_dtype == TL_DT_F32)
         rope_cache_write_kernel<float><<<grid, block, 0, stream>>>((float*)qkv, row_stride, q_heads, kv_heads, head_dim, rot_heads,
             (const int*)positions, (const float*)inv_freq, (const int*)token_req, (const int*)block_table, bt_stride,
-            (float*)k_plane, (float*)v_plane, page_size, pairs);
+            (float*)k_plane, (float*)v_plane, page_size, pairs, pair_aligned);
     else if (act_dtype == TL_DT_BF16)
         rope_cache_write_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)qkv, row_stride, q_heads, kv_heads, head_dim, rot_heads,
             (const int*)positions, (const float*)inv_freq, (const int*)token_req, (const int*)block_table, bt_stride,
-            (bf16_t*)k_plane, (bf16_t*)v_plane, page_size, pairs);
+            (bf16_t*)k_plane, (bf16_t*)v_plane, page_size, pairs, pair_aligned);
     else TL_REQUIRE(false, "rope_cache_write: unknown dtype %d", act_dtype);
     TL_CHECK_LAUNCH("rope_cache_write");
     return TL_OK;

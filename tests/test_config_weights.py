@@ -183,3 +183,35 @@ def test_random_weights_law_and_reproducibility(tmp_path):
     assert set(stored) == set(a)
     assert torch.equal(stored["lm_head.weight"], a["lm_head.weight"].to(torch.bfloat16))
     assert isinstance(load_config(folder), Qwen2Config)
+
+
+def test_attention_part_fuses_its_projections_and_keeps_32_bit_biases():
+    """q, k and v become one matrix; biases stored in different dtypes are kept in 32-bit; the
+    bfloat16 engine reorders the rows of q and k (not v) into the pair layout of the rotary
+    encoding, the 32-bit engine leaves them as they are."""
+    from torchlet_amd.config import AttentionSpec, RotarySpec
+    from torchlet_amd.kernels import ops
+    from torchlet_amd.parts import MIXERS
+    heads, kvh, hd, hidden = 4, 2, 16, 24
+    spec = AttentionSpec(hidden=hidden, num_heads=heads, num_kv_heads=kvh, head_dim=hd, qkv_bias=True,
+                         position=RotarySpec(head_dim=hd, theta=1e4, max_positions=64))
+    g = torch.Generator().manual_seed(0)
+    t = {f"{n}_proj.weight": torch.randn(w * hd, hidden, generator=g).to(torch.bfloat16) for n, w in (("q", heads), ("k", kvh), ("v", kvh))}
+    t["o_proj.weight"] = torch.randn(hidden, heads * hd, generator=g).to(torch.bfloat16)
+    t["q_proj.bias"] = torch.randn(heads * hd, generator=g)                        # stored in 32-bit
+    t["k_proj.bias"] = torch.randn(kvh * hd, generator=g).to(torch.bfloat16)
+    t["v_proj.bias"] = torch.randn(kvh * hd, generator=g).to(torch.bfloat16)
+    plain_rows = torch.cat([t[f"{n}_proj.weight"] for n in "qkv"])
+    plain_bias = torch.cat([t[f"{n}_proj.bias"].float() for n in "qkv"])
+
+    wide = MIXERS.build(spec, torch.float32, torch.device("cpu"))
+    wide.load_weights(t)
+    assert not wide.pair_layout and torch.equal(wide.w_qkv, plain_rows.float()) and torch.equal(wide.b_qkv, plain_bias)
+
+    half = MIXERS.build(spec, torch.bfloat16, torch.device("cpu"))
+    half.load_weights(t)
+    assert half.pair_layout and half.b_qkv.dtype == torch.float32 and half.w_qkv.dtype == torch.bfloat16
+    order = torch.cat((ops.pair_layout_rows(heads + kvh, hd), (heads + kvh) * hd + torch.arange(kvh * hd)))
+    assert torch.equal(half.w_qkv, plain_rows[order]) and torch.equal(half.b_qkv, plain_bias[order])
+    # within a head: row 2j is the old row j, row 2j + 1 the old row j + hd/2
+    assert order[:6].tolist() == [0, 8, 1, 9, 2, 10] and order[hd:hd + 2].tolist() == [16, 24]

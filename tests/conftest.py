@@ -44,6 +44,6 @@ def cpu_ops(monkeypatch):
 
     for name in ("attention_tile_tokens", "load", "embedding", "add_rmsnorm", "linear", "rope_cache_write",
                  "paged_attention", "swiglu", "sample", "interleave_gate_up", "linear_swiglu",
-                 "prefill_attention_tile_tokens", "paged_attention_prefill", "linear_partials", "linear_rope_cache_write"):
+                 "prefill_attention_tile_tokens", "paged_attention_prefill", "linear_partials", "linear_partials_pay", "linear_rope_cache_write"):
         monkeypatch.setattr(ops, name, getattr(emulated_ops, name))
     return ops

@@ -137,6 +137,10 @@ def paged_attention_prefill(q, out, k_plane, v_plane, block_table, req_indptr, c
             tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale)
 
 
+def linear_partials_pay(M, N, K):
+    return False
+
+
 def linear_partials(x, weight):
     K = x.shape[1]
     half = (K // 2 // 8) * 8 or K

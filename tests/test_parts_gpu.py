@@ -93,11 +93,11 @@ def test_swiglu_part_alone(dtype):
 
 
 def test_swiglu_part_with_a_long_intermediate_hands_partial_sums_to_the_next_norm():
-    """17 to 64 rows over a long intermediate size: the down product comes back as slabs of
-    partial sums, which the next norm adds into the residual in 32-bit."""
+    """17 rows up over a long intermediate size and a narrow output: the down product comes back as
+    slabs of partial sums, which the next norm adds into the residual in 32-bit."""
     from torchlet_amd.config import RMSNormSpec, SwiGLUSpec
     from torchlet_amd.parts import FEED_FORWARDS, NORMS, Stream
-    hidden, inter, rows = 72, 8200, 24
+    hidden, inter, rows = 72, 8192, 24
     dev = torch.device("cuda")
     ffn = FEED_FORWARDS.build(SwiGLUSpec(hidden=hidden, intermediate=inter), torch.bfloat16, dev)
     w = {"gate_proj.weight": torch.randn(inter, hidden) * 0.2, "up_proj.weight": torch.randn(inter, hidden) * 0.2,

@@ -140,16 +140,25 @@ def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: to
                                    c_int(_dt(out, "add_rmsnorm")), _stream()))
 
 
+def linear_partials_pay(M: int, N: int, K: int) -> bool:
+    """Whether :func:`linear_partials` would split this bfloat16 product over K (17 rows up: when
+    its 64 x 64 output tiles are too few to fill the GPU and K is a multiple of 64)."""
+    if M <= 16 or K % 64:
+        return False
+    return _lib("gemm").tl_gemm_partials_parts(c_int(M), c_int(N), c_int(K)) > 1
+
+
 def linear_partials(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``x @ weight.T`` as float32 slabs ``[P, M, N]`` of partial sums over P ranges of K (bfloat16
-    operands, M <= 64, K a multiple of 8): for a narrow matrix with a long K, where splitting K
-    over work-groups is what fills the GPU.  The slabs are summed by :func:`add_rmsnorm`."""
+    operands, K a multiple of 8; more than 64 rows need a multiple of 64): for a product with too
+    few output tiles to fill the GPU, where splitting K over work-groups does.  The slabs are
+    summed by :func:`add_rmsnorm`."""
     M, K = x.shape
     N = weight.shape[0]
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or weight.shape[1] != K or not weight.is_contiguous() or x.stride(1) != 1:
         raise KernelError("linear_partials: bfloat16 operands and fitting shapes only")
     lib = _lib("gemm")
-    out = torch.empty((lib.tl_gemm_partials_max(), M, N), dtype=torch.float32, device=x.device)
+    out = torch.empty((lib.tl_gemm_partials_parts(c_int(M), c_int(N), c_int(K)), M, N), dtype=torch.float32, device=x.device)
     parts = c_int(0)
     _check(lib, lib.tl_gemm_partials(_ptr(x), _ptr(weight), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(x.stride(0)),
                                      ctypes.byref(parts), _stream()))

@@ -157,6 +157,9 @@ class GQAttention(Mixer):
             tile_req, tile_tok0, tiles = ctx.tiles(self.tile_tokens)
             ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
                                 tile_req, tile_tok0, tiles, self.tile_tokens, *common, self._splits(ctx, tiles))
+        if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, self.q_width):
+            # few rows against a narrow matrix: K split over work-groups; the next norm adds the slabs up
+            return ops.linear_partials(out, self.w_o)
         y = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
         ops.linear(out, self.w_o, None, y)
         return y

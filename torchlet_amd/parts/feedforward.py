@@ -15,13 +15,10 @@ from ..kernels import ops
 from .base import FEED_FORWARDS, FeedForward, WeightSpec
 
 
-# The down product of a decode step of 17 to 64 rows returns partial sums over slices of K when
-# K (the intermediate size) is long: the matrix is narrow, so whole-K work-groups are too few to
-# keep the memory system busy (measured at 3584 x 18944: 66 -> 42 us at 32 rows, 98 -> 68 us at
-# 64).  Up to 16 rows the plain kernel already streams at its limit and the extra slabs cost more.
-_PARTIALS_MIN_ROWS = 17
-_PARTIALS_MAX_ROWS = 64
-_PARTIALS_MIN_K = 8192
+# From 17 rows on the down product returns partial sums over slices of K where that pays (the
+# matrix is narrow, so its output tiles alone are too few to keep the GPU busy; measured at
+# 3584 x 18944 and 64 rows: 31 us in four parts against 90 us whole); the next norm adds the slabs up.
+# Up to 16 rows the plain kernel already streams at its limit and the extra slabs cost more.
 
 
 @FEED_FORWARDS.register("swiglu")
@@ -59,7 +56,7 @@ class SwiGLU(FeedForward):
             gu = torch.empty((T, 2 * self.inter), dtype=self.dtype, device=h.device)
             ops.linear(h, self.gate_up, None, gu)
             ops.swiglu(gu, z)
-        if self.fused_gate and _PARTIALS_MIN_ROWS <= T <= _PARTIALS_MAX_ROWS and self.inter >= _PARTIALS_MIN_K and self.inter % 8 == 0:
+        if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, self.inter):
             # few rows, long K, narrow matrix: split K over work-groups; the next norm adds the slabs up
             return ops.linear_partials(z, self.down)
         y = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)

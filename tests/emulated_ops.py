@@ -52,8 +52,11 @@ def linear_rope_cache_write(*args, **kwargs):
 
 
 def rope_cache_write(qkv, q_heads, kv_heads, head_dim, rot_heads, positions, inv_freq,
-                     token_req=None, block_table=None, k_plane=None, v_plane=None, page_size=0, pairs=False):
+                     token_req=None, block_table=None, k_plane=None, v_plane=None, page_size=0, pairs=False, parts=None, bias=None):
     T = qkv.shape[0]
+    if parts is not None:
+        total = parts.sum(0) + (bias.float() if bias is not None else 0.0)
+        qkv[:, : total.shape[1]] = total.to(qkv.dtype)
     x = qkv[:, : (q_heads + kv_heads) * head_dim].float().view(T, q_heads + kv_heads, head_dim)
     if inv_freq is not None:
         ang = positions.float()[:, None] * inv_freq[None, :]

@@ -294,6 +294,47 @@ def test_rope_cache_write_in_the_pair_layout(ops, dtype, nh, nkv, hd, page, thet
     assert torch.equal(pair_v, plain_v)
 
 
+@pytest.mark.parametrize("pairs", [False, True])
+@pytest.mark.parametrize("nh,nkv,hd,page,P,bias", [(28, 4, 128, 16, 3, True), (4, 2, 16, 8, 1, False), (5, 5, 48, 16, 4, True)])
+def test_rope_cache_write_from_slabs_of_partial_sums(ops, pairs, nh, nkv, hd, page, P, bias):
+    """The rows come as float slabs of a projection split over K, plus its bias: queries land rotated
+    in qkv, rotated keys and values in their pages."""
+    g = torch.Generator().manual_seed(8)
+    lens, ctxs = [20, 1, 3], [0, 37, 6]
+    T = sum(lens)
+    width = (nh + 2 * nkv) * hd
+    max_blocks = (max(a + b for a, b in zip(lens, ctxs)) + page - 1) // page
+    pages = 3 * max_blocks + 2
+    parts = torch.randn(P, T, width, generator=g)
+    b = torch.randn(width, generator=g).to(torch.bfloat16) if bias else None
+    positions = torch.cat([torch.arange(c, c + n) for n, c in zip(lens, ctxs)]).int()
+    token_req = torch.cat([torch.full((n,), r) for r, n in enumerate(lens)]).int()
+    bt = (torch.randperm(pages - 1, generator=g)[: 3 * max_blocks] + 1).view(3, max_blocks).int()
+    inv_freq = 1.0 / (1e5 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))
+    qkv = torch.full((T, width), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kp = torch.zeros(pages, nkv, page, hd, dtype=torch.bfloat16, device="cuda")
+    vp = torch.zeros(pages, nkv, hd, page, dtype=torch.bfloat16, device="cuda")
+    ops.rope_cache_write(qkv, nh, nkv, hd, nh + nkv, positions.cuda(), inv_freq.cuda(), token_req.cuda(), bt.cuda(), kp, vp, page,
+                         pairs=pairs, parts=parts.cuda(), bias=None if b is None else b.cuda())
+    exact = parts.double().sum(0) + (b.double() if bias else 0.0)
+    heads = exact[:, : (nh + nkv) * hd].view(T, nh + nkv, hd)
+    ang = (positions.float()[:, None] * inv_freq[None, :]).double()[:, None, :]
+    if pairs:
+        a, c = heads[..., 0::2], heads[..., 1::2]
+        turned = torch.stack((a * ang.cos() - c * ang.sin(), c * ang.cos() + a * ang.sin()), -1).reshape(T, nh + nkv, hd)
+    else:
+        a, c = heads[..., : hd // 2], heads[..., hd // 2:]
+        turned = torch.cat((a * ang.cos() - c * ang.sin(), c * ang.cos() + a * ang.sin()), -1)
+    tol = dict(rtol=2 ** -8, atol=1e-5 * float(exact.abs().max()))          # one rounding to bfloat16
+    torch.testing.assert_close(qkv[:, : nh * hd].double().cpu(), turned[:, :nh].reshape(T, -1), **tol)
+    v = exact[:, (nh + nkv) * hd:].view(T, nkv, hd)
+    for t in range(T):
+        p = int(positions[t]); pg = int(bt[token_req[t], p // page])
+        torch.testing.assert_close(kp[pg, :, p % page].double().cpu(), turned[t, nh:], **tol)
+        torch.testing.assert_close(vp[pg, :, :, p % page].double().cpu(), v[t], **tol)
+    assert float(kp[0].abs().sum()) == 0.0
+
+
 @pytest.mark.parametrize("M", [1, 2, 8, 16])
 @pytest.mark.parametrize("nh,nkv,hd,page,hidden,bias", [(28, 4, 128, 16, 3584, True), (4, 2, 16, 8, 64, False), (14, 2, 64, 16, 896, True),
                                                         (40, 8, 128, 32, 5120, True), (5, 5, 48, 16, 240, True)])

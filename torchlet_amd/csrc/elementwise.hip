@@ -211,7 +211,9 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
                              int head_dim, int rot_heads, const int* __restrict__ positions,
                              const float* __restrict__ inv_freq, const int* __restrict__ token_req,
                              const int* __restrict__ block_table, int bt_stride,
-                             T* __restrict__ k_plane, T* __restrict__ v_plane, int page_size, int pairs, int pair_aligned) {
+                             T* __restrict__ k_plane, T* __restrict__ v_plane, int page_size, int pairs, int pair_aligned,
+                             const float* __restrict__ parts, int num_parts, size_t part_stride, int parts_ld,
+                             const void* __restrict__ bias, int bias_f32) {
     // A wave owns one head of one token: a query head (rotated in place), a key head (rotated in
     // place and written to its page) or a value head (written to its page, transposed).  Each wave
     // takes the cosines and sines of its own pairs, so no wave waits for another.
@@ -231,13 +233,23 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
         dst = head < q_heads + kv_heads ? k_plane + base + (size_t)(pos % page_size) * head_dim
                                         : v_plane + base + (pos % page_size);
     }
+    // With `parts` the row does not come from qkv but is the sum of float slabs of partial sums
+    // [num_parts][tokens, parts_ld] plus the bias (a projection that was split over K); the rotated
+    // queries then go to qkv, keys and values to their pages only.
+    auto element = [&](int i) -> float {
+        if (!parts) return to_float(x[i]);
+        const size_t col = (size_t)head * head_dim + i;
+        float sum = bias ? load_vec(bias, bias_f32, col) : 0.f;
+        for (int p = 0; p < num_parts; ++p) sum += parts[(size_t)p * part_stride + (size_t)t * parts_ld + col];
+        return sum;
+    };
     if (head >= q_heads + kv_heads) {      // value head: [head_dim, page] inside the page
-        for (int d = lane; d < head_dim; d += TL_WAVE) dst[(size_t)d * page_size] = x[d];
+        for (int d = lane; d < head_dim; d += TL_WAVE) dst[(size_t)d * page_size] = from_float<T>(element(d));
         return;
     }
     const bool rotate = inv_freq && head < rot_heads;
-    if (!rotate && !dst) return;
-    if (pairs && pair_aligned) {
+    if (!rotate && !dst && !parts) return;
+    if (pairs && pair_aligned && !parts) {
         // pair layout: the two elements of a frequency are one aligned load and one aligned store
         struct __attribute__((aligned(2 * sizeof(T)))) Two { T a, b; };
         for (int j = lane; j < half; j += TL_WAVE) {
@@ -262,7 +274,7 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
         // the two elements that frequency j turns: (j, j + half), or neighbours (2j, 2j + 1) in the
         // pair layout (a projection whose rows were reordered that way at load time)
         const int i1 = pairs ? 2 * j : j, i2 = pairs ? 2 * j + 1 : j + half;
-        float x1 = to_float(x[i1]), x2 = to_float(x[i2]);
+        float x1 = element(i1), x2 = element(i2);
         if (rotate) {
             const float angle = (float)pos * inv_freq[j];
             const float c = cosf(angle), sn = sinf(angle);
@@ -270,6 +282,8 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
             const float y2 = x2 * c + x1 * sn;
             x1 = y1;
             x2 = y2;
+        }
+        if (rotate || parts) {
             x[i1] = from_float<T>(x1);
             x[i2] = from_float<T>(x2);
         }
@@ -284,7 +298,10 @@ extern "C" int tl_rope_cache_write(void* qkv, int row_stride, int tokens, int q_
                                    int head_dim, int rot_heads, const void* positions, const void* inv_freq,
                                    const void* token_req, const void* block_table, int bt_stride,
                                    void* k_plane, void* v_plane, int page_size, int pairs, int act_dtype,
-                                   hipStream_t stream) {
+                                   const void* parts, int num_parts, size_t part_stride, int parts_ld,
+                                   const void* bias, int bias_f32, hipStream_t stream) {
+    TL_REQUIRE(!parts || (num_parts > 0 && parts_ld >= (q_heads + kv_heads + (k_plane ? kv_heads : 0)) * head_dim),
+               "rope_cache_write: slabs of partial sums need a count and rows as wide as the heads");
     TL_REQUIRE(tokens >= 0 && q_heads >= 0 && kv_heads >= 0 && head_dim > 0 && head_dim % 2 == 0 && head_dim <= 256,
                "rope_cache_write: bad sizes tokens=%d q_heads=%d kv_heads=%d head_dim=%d (even, at most 256)", tokens, q_heads, kv_heads, head_dim);
     TL_REQUIRE(rot_heads <= q_heads + kv_heads, "rope_cache_write: rot_heads %d exceeds q+k heads", rot_heads);
@@ -301,11 +318,11 @@ extern "C" int tl_rope_cache_write(void* qkv, int row_stride, int tokens, int q_
     if (act_dtype == TL_DT_F32)
         rope_cache_write_kernel<float><<<grid, block, 0, stream>>>((float*)qkv, row_stride, q_heads, kv_heads, head_dim, rot_heads,
             (const int*)positions, (const float*)inv_freq, (const int*)token_req, (const int*)block_table, bt_stride,
-            (float*)k_plane, (float*)v_plane, page_size, pairs, pair_aligned);
+            (float*)k_plane, (float*)v_plane, page_size, pairs, pair_aligned, (const float*)parts, num_parts, part_stride, parts_ld, bias, bias_f32);
     else if (act_dtype == TL_DT_BF16)
         rope_cache_write_kernel<bf16_t><<<grid, block, 0, stream>>>((bf16_t*)qkv, row_stride, q_heads, kv_heads, head_dim, rot_heads,
             (const int*)positions, (const float*)inv_freq, (const int*)token_req, (const int*)block_table, bt_stride,
-            (bf16_t*)k_plane, (bf16_t*)v_plane, page_size, pairs, pair_aligned);
+            (bf16_t*)k_plane, (bf16_t*)v_plane, page_size, pairs, pair_aligned, (const float*)parts, num_parts, part_stride, parts_ld, bias, bias_f32);
     else TL_REQUIRE(false, "rope_cache_write: unknown dtype %d", act_dtype);
     TL_CHECK_LAUNCH("rope_cache_write");
     return TL_OK;

@@ -261,13 +261,16 @@ def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: i
                      positions: torch.Tensor, inv_freq: torch.Tensor | None,
                      token_req: torch.Tensor | None = None, block_table: torch.Tensor | None = None,
                      k_plane: torch.Tensor | None = None, v_plane: torch.Tensor | None = None,
-                     page_size: int = 0, pairs: bool = False) -> None:
+                     page_size: int = 0, pairs: bool = False, parts: torch.Tensor | None = None,
+                     bias: torch.Tensor | None = None) -> None:
     """Rotate the first ``rot_heads`` heads of each row of ``qkv [T, >= (q+2kv)*hd]`` in
     place by the token's position (``inv_freq`` float32 ``[hd/2]``; ``None``: no rotation;
     ``pairs``: frequency j turns the neighbours ``(2j, 2j+1)`` instead of ``(j, j+hd/2)``)
     and, when planes are given, store rotated k and raw v of every token in its page:
     ``k_plane [pages, kv_heads, page, hd]``, ``v_plane [pages, kv_heads, hd, page]`` (values
-    lie transposed inside a page)."""
+    lie transposed inside a page).  With ``parts`` (float32 ``[P, T, width]``, slabs of partial
+    sums of the projection, and its ``bias``) the rows are the sums of the slabs instead of what
+    ``qkv`` holds: the queries are written to ``qkv``, keys and values to their pages only."""
     T = qkv.shape[0]
     if qkv.stride(1) != 1:
         raise KernelError("rope_cache_write: qkv needs unit stride on the last axis")
@@ -280,11 +283,21 @@ def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: i
         _i32(block_table, "block_table")
         bt_stride = block_table.stride(0)
         _check_planes("rope_cache_write", k_plane, v_plane, qkv.dtype, kv_heads, page_size, head_dim)
+    num_parts = part_stride = parts_ld = bf = 0
+    if parts is not None:
+        if parts.dtype != torch.float32 or parts.dim() != 3 or parts.shape[1] != T or not parts.is_contiguous():
+            raise KernelError("rope_cache_write: parts must be contiguous float32 [P, T, width]")
+        num_parts, part_stride, parts_ld = parts.shape[0], parts.stride(0), parts.shape[2]
+        bf = _vec(bias, parts_ld, "projection bias")
+    elif bias is not None:
+        raise KernelError("rope_cache_write: a bias comes with slabs of partial sums only")
     lib = _lib("elementwise")
     _check(lib, lib.tl_rope_cache_write(_ptr(qkv), c_int(qkv.stride(0)), c_int(T), c_int(q_heads), c_int(kv_heads),
                                         c_int(head_dim), c_int(rot_heads), _ptr(positions), _ptr(inv_freq), _ptr(token_req),
                                         _ptr(block_table), c_int(bt_stride), _ptr(k_plane), _ptr(v_plane), c_int(page_size),
-                                        c_int(1 if pairs else 0), c_int(_dt(qkv, "rope_cache_write")), _stream()))
+                                        c_int(1 if pairs else 0), c_int(_dt(qkv, "rope_cache_write")),
+                                        _ptr(parts), c_int(num_parts), ctypes.c_size_t(part_stride), c_int(parts_ld),
+                                        _ptr(bias), c_int(bf), _stream()))
 
 
 def pair_layout_rows(num_heads: int, head_dim: int) -> torch.Tensor:

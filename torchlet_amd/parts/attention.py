@@ -124,7 +124,12 @@ class GQAttention(Mixer):
         cache_args = (ctx.token_req, table, k_plane, v_plane, cache.page_size) if writes else (None, None, None, None, 0)
         fused = self.pair_layout and ops.linear_rope_cache_write(h, w, b, qkv, self.heads, self.kv_heads, self.head_dim,
                                                                  ctx.positions, inv_freq, *cache_args)
-        if not fused:
+        if not fused and self.dtype == torch.bfloat16 and (inv_freq is not None or self.position is None) \
+                and ops.linear_partials_pay(T, width, self.hidden):
+            # few rows against a narrow matrix: K split over work-groups; the rotation kernel adds the slabs up
+            ops.rope_cache_write(qkv, self.heads, kv_heads, self.head_dim, self.heads + kv_heads, ctx.positions, inv_freq,
+                                 *cache_args, pairs=self.pair_layout, parts=ops.linear_partials(h, w), bias=b)
+        elif not fused:
             ops.linear(h, w, b, qkv)
             if self.position is not None and inv_freq is None:
                 q3 = qkv[:, : self.q_width].unflatten(1, (self.heads, self.head_dim))

@@ -1044,15 +1044,23 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
 // out[P, M, N] (float) = partial sums of x w^T over P ranges of K, for a product with too few output
 // tiles to fill the GPU (a narrow matrix against few rows): P work-groups per tile keep all compute
 // units busy; whoever reads the slabs adds them up.  Returns P through `parts` (the caller sizes
-// `out` for tl_gemm_partials_max()).  From 17 rows on (K a multiple of 64) the direct-load tile
+// `out` for tl_gemm_partials_max()).  Where it pays (see partials_on_tiles) the direct-load tile
 // kernel runs with 64 x 64 tiles (measured at 64 rows, 3584 x 18944: 31 us with four parts against
 // 90 us whole; 3584 x 3584: 9.5 against 20 us); up to 16 rows, or for other K, the skinny kernel
 // with R = 4 strips per work-group, which share every x fetch.
 extern "C" int tl_gemm_partials_max() { return 8; }
 
-// How many parts tl_gemm_partials would use; 1 says that splitting does not pay for this shape.
+// Whether the tile kernel does the split: from 17 rows on, and from 2 rows on against a long K
+// (measured at 3584 x 18944 with the sum in the norm: 8 rows 31.8 against 35.6 us, 16 rows 32.5 against
+// 42.0 us; against a short K, 3584 x 3584, the skinny kernel without a split stays ahead up to 16 rows).
+static bool partials_on_tiles(int M, int K) { return K % 64 == 0 && (M > 16 || (M >= 2 && K >= 8192)); }
+
+// Whether a consumer that can add slabs up should ask for them instead of the whole product.
+extern "C" int tl_gemm_partials_pay(int M, int N, int K);
+
+// How many parts tl_gemm_partials would use.
 extern "C" int tl_gemm_partials_parts(int M, int N, int K) {
-    if (M > 16 && K % 64 == 0) {
+    if (partials_on_tiles(M, K)) {
         const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
         int P = (int)(256 / tiles);                       // about one work-group per compute unit
         const int by_k = K / 512;                         // at least eight slabs of 64 per part
@@ -1065,6 +1073,10 @@ extern "C" int tl_gemm_partials_parts(int M, int N, int K) {
     return P < 1 ? 1 : P;
 }
 
+extern "C" int tl_gemm_partials_pay(int M, int N, int K) {
+    return partials_on_tiles(M, K) && tl_gemm_partials_parts(M, N, K) > 1;
+}
+
 extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int* parts,
                                 hipStream_t stream) {
     TL_REQUIRE(M > 0 && N > 0 && K > 0 && ldx >= K, "gemm_partials: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -1075,7 +1087,7 @@ extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, 
     const int k_per = ((steps + P - 1) / P) * 64;
     P = (K + k_per - 1) / k_per;
     *parts = P;
-    if (M > 16 && K % 64 == 0) {
+    if (partials_on_tiles(M, K)) {
         auto kernel = gemm_dl_tile_kernel<64, 64, 2, 2, 4, float, false>;
         constexpr size_t lds = (size_t)4 * 128 * 64 * sizeof(bf16_t);
         static hipError_t allowed = allow_lds(kernel, lds);

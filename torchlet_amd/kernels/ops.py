@@ -141,11 +141,10 @@ def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: to
 
 
 def linear_partials_pay(M: int, N: int, K: int) -> bool:
-    """Whether :func:`linear_partials` would split this bfloat16 product over K (17 rows up: when
-    its 64 x 64 output tiles are too few to fill the GPU and K is a multiple of 64)."""
-    if M <= 16 or K % 64:
-        return False
-    return _lib("gemm").tl_gemm_partials_parts(c_int(M), c_int(N), c_int(K)) > 1
+    """Whether a bfloat16 product whose consumer can add slabs up should come from
+    :func:`linear_partials`: when its 64 x 64 output tiles are too few to fill the GPU and K is a
+    multiple of 64, from 17 rows on, and from 2 rows on against a long K."""
+    return bool(_lib("gemm").tl_gemm_partials_pay(c_int(M), c_int(N), c_int(K)))
 
 
 def linear_partials(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:

@@ -155,3 +155,43 @@ def test_command_line(model_folders, tmp_path):
     lines = [json.loads(l) for l in run.stdout.strip().splitlines()]
     cfg, w = plain_qwen2.load_folder(tmp_path / "m")
     assert [l["output"] for l in lines] == [plain_qwen2.greedy(cfg, w, [5, 6, 7], 4), plain_qwen2.greedy(cfg, w, [9], 4)]
+
+
+def _write_tokenizer(folder, vocab_size):
+    """A word-level tokenizer over made-up words and a chat template in the manner of the
+    checkpoints this architecture ships with, written with the ``tokenizers`` library."""
+    import json
+    from tokenizers import Tokenizer, models, pre_tokenizers
+    special = ["<|im_start|>", "<|im_end|>", "<|endoftext|>"]
+    words = special + ["user", "assistant", "\n"] + [f"w{i}" for i in range(vocab_size - 6)]
+    tok = Tokenizer(models.WordLevel({w: i for i, w in enumerate(words)}, unk_token="w0"))
+    tok.pre_tokenizer = pre_tokenizers.Split(" ", "removed")
+    tok.add_special_tokens(special)
+    tok.save(str(folder / "tokenizer.json"))
+    template = ("{% for m in messages %}<|im_start|> {{ m['role'] }} \n {{ m['content'] }} <|im_end|> \n {% endfor %}"
+                "{% if add_generation_prompt %}<|im_start|> assistant \n{% endif %}")
+    (folder / "tokenizer_config.json").write_text(json.dumps({"chat_template": template, "eos_token": "<|endoftext|>"}))
+    return words
+
+
+def test_strings_in_strings_out_through_a_tokenizer_and_its_chat_template(model_folders, tmp_path):
+    """Prompts given as strings are wrapped as one user turn by the folder's chat template
+    (/root/reference/src/torchlet/v10_triton_paged_gqa/llm.py:87-95), generation stops at the
+    template's end-of-turn token or the tokenizer's end token (llm.py:40-44), and the answer
+    comes back as text without special tokens (engine.py:194-196)."""
+    import shutil
+    from torchlet_amd import LLM
+    folder = tmp_path / "with_tokenizer"
+    shutil.copytree(model_folders["A"], folder)
+    cfg, w = plain_qwen2.load_folder(folder)
+    words = _write_tokenizer(folder, cfg.vocab)
+    llm = LLM(str(folder), max_decode_slots=2, dtype="float32")
+    assert llm.stop_ids == frozenset({1, 2})
+    text, ids = llm.tokenizer.encode_chat("w7 w8 w9")
+    assert [words[i] for i in ids] == ["<|im_start|>", "user", "\n", "w7", "w8", "w9", "<|im_end|>", "\n", "<|im_start|>", "assistant", "\n"]
+    outs = llm.generate(["w7 w8 w9", "w20"], max_new_tokens=12)
+    for prompt, out in zip(["w7 w8 w9", "w20"], outs):
+        _, ids = llm.tokenizer.encode_chat(prompt)
+        expected = plain_qwen2.greedy(cfg, w, ids, 12, stop_ids=(1, 2))
+        assert out == " ".join(words[t] for t in expected if t > 2) or out == llm.tokenizer.decode(expected)
+        assert "<|" not in out

@@ -195,3 +195,30 @@ def test_strings_in_strings_out_through_a_tokenizer_and_its_chat_template(model_
         expected = plain_qwen2.greedy(cfg, w, ids, 12, stop_ids=(1, 2))
         assert out == " ".join(words[t] for t in expected if t > 2) or out == llm.tokenizer.decode(expected)
         assert "<|" not in out
+
+
+def test_concurrent_callers_share_the_engines_steps(model_folders):
+    """Three callers of the coroutine form arrive one after the other, as in the reference's own
+    demonstration (/root/reference/src/torchlet/v10_triton_paged_gqa/llm.py:113-140): their
+    requests run in the same steps, and each gets what it would have got alone."""
+    import asyncio
+    from torchlet_amd import LLM
+    cfg, w = plain_qwen2.load_folder(model_folders["A"])
+    prompts = list(scenarios.make_requests(cfg.vocab, [9, 30, 4], seed=7).values())
+    llm = LLM(str(model_folders["A"]), max_decode_slots=4, dtype="float32", max_num_batched_tokens=16)
+
+    async def caller(i):
+        for _ in range(2 * i):
+            await asyncio.sleep(0)          # arrive a few steps later than the caller before
+        return (await llm.generate_async([prompts[i]], max_new_tokens=10))[0]
+
+    async def main():
+        return await asyncio.gather(*(caller(i) for i in range(3)))
+
+    steps_before = llm.engine.steps
+    outs = asyncio.run(main())
+    for p, o in zip(prompts, outs):
+        assert o == plain_qwen2.greedy(cfg, w, p, 10)
+    alone = sum(-(-len(p) // 16) + 9 for p in prompts)
+    assert llm.engine.steps - steps_before < alone, "the callers' requests did not share steps"
+    assert llm.runner.cache.live_requests() == []

@@ -146,3 +146,27 @@ def test_toy_parts_and_a_layer_run_twice_on_the_host(cpu_ops):
     own, a layer that runs twice and reads its first run's cache) through the host logic."""
     import toy_parts
     toy_parts.run_toy_mix(torch.float32, torch.device("cpu"), lambda dtype, ref: dict(atol=2e-5, rtol=1e-4))
+
+
+def test_shutdown_gives_up_unfinished_requests_and_frees_their_pages(cpu_ops, model_folders):
+    from concurrent.futures import CancelledError
+    runner = runner_for(model_folders["A"], "A", pages=12)
+    engine = Engine(runner, max_tokens_per_step=16)
+    done_early = Request(prompt_tokens=[1, 2, 3], max_new_tokens=1)
+    long_one = Request(prompt_tokens=list(range(40)), max_new_tokens=30)
+    waiting = Request(prompt_tokens=list(range(100)), max_new_tokens=5)
+    for r in (done_early, long_one, waiting):
+        engine.add_request(r)
+    for _ in range(3):
+        engine.step()
+    assert done_early.finish_reason == "length" and long_one.finish_reason is None
+    ended = engine.shutdown()
+    assert {r.req_id for r in ended} >= {long_one.req_id, waiting.req_id}
+    assert isinstance(long_one.error, CancelledError) and long_one.finish_reason == "error" and waiting.finish_reason == "error"
+    assert done_early.error is None
+    assert runner.cache.live_requests() == [] and not engine.has_work()
+    runner.cache.check()
+    again = Request(prompt_tokens=[5, 6], max_new_tokens=2)      # the engine goes on working
+    engine.add_request(again)
+    engine.run_until_done()
+    assert len(again.output_tokens) == 2

@@ -8,6 +8,8 @@ asynchronous ``generate`` of the Python entry point wraps it.
 """
 from __future__ import annotations
 
+from concurrent.futures import CancelledError
+
 from ..sampling.sampler import Sampler
 from .batch import StepEntry
 from .request import Request
@@ -45,6 +47,12 @@ class Engine:
                                          [len(r.output_tokens) for r in sampling])
         self.steps += 1
         return self.scheduler.process_output(chosen, tokens)
+
+    def shutdown(self) -> list[Request]:
+        """Give up every request that is not finished (they end with a cancellation error) and take
+        back all pages, as the reference's engine does when it is shut down (engine.py:81-99 of
+        the reference); the engine can be used again afterwards."""
+        return self.scheduler.fail_all(CancelledError("the engine was shut down"))
 
     def run_until_done(self) -> list[Request]:
         """Step until no request is waiting or running; on an error every unfinished request

@@ -756,7 +756,7 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
 
 // =====================================================================================
 // Prompt portions, 128 rows per work-group (bfloat16, head size 64 or 128, pages of 8, 16, 32, ...
-// tokens, block tables of up to ATM_BT_MAX entries).
+// tokens, sequences of up to ATM_BT_MAX pages).
 //
 // Four waves of 32 rows share steps of 32 keys.  Keys and transposed values of a step go from
 // the pages straight into shared memory (global_load_lds_dwordx4, four buffers: three steps are
@@ -860,6 +860,7 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     const int shift = a.page_shift, pmask = page - 1;
     const int blk0 = (st_first * ATQ_KEYS) >> shift;
     const int blk_n = ((key_hi - 1) >> shift) - blk0 + 1;
+    if (blk_n > ATM_BT_MAX) return;            // longer than the host promised: leave the rows unwritten rather than overrun
     for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
     __syncthreads();
 
@@ -1034,7 +1035,7 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
 
 // The 128-row prompt kernel: tiles of `tq` tokens with tq * min(group, 128) <= 128.  Returns an
 // error where it is not built (head sizes other than 64 and 128, pages that are no power of two from 8 up,
-// block tables wider than tl_paged_attention_prompt_blocks()).
+// sequences longer than tl_paged_attention_prompt_blocks() pages).
 extern "C" int tl_paged_attention_prompt_rows() {
 #if AT_HD == 64 || AT_HD == 128
     return ATQ_ROWS;
@@ -1048,11 +1049,14 @@ extern "C" int tl_paged_attention_prompt_blocks() { return ATM_BT_MAX; }
 extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out, const void* k_plane, const void* v_plane,
                                          const void* block_table, int bt_stride, const void* req_indptr, const void* ctx_lens,
                                          const void* tile_req, const void* tile_tok0, int tiles, int tq,
-                                         int heads, int kv_heads, int page, int window, float scale, hipStream_t stream) {
+                                         int heads, int kv_heads, int page, int window, float scale, int used_blocks,
+                                         hipStream_t stream) {
 #if AT_HD == 64 || AT_HD == 128
     TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
     TL_REQUIRE(page >= 8 && (page & (page - 1)) == 0 && tq > 0 && window >= 0, "attention_prompt: pages of 8, 16, 32, ... tokens, not %d", page);
-    TL_REQUIRE(bt_stride > 0 && bt_stride <= ATM_BT_MAX, "attention_prompt: block tables of up to %d entries, not %d", ATM_BT_MAX, bt_stride);
+    // used_blocks: the most block-table entries any request of the step uses (its length in pages)
+    TL_REQUIRE(bt_stride > 0 && used_blocks > 0 && used_blocks <= ATM_BT_MAX,
+               "attention_prompt: sequences of up to %d pages, not %d", ATM_BT_MAX, used_blocks);
     const int group = heads / kv_heads;
     const int gcap = group < ATQ_ROWS ? group : ATQ_ROWS;
     TL_REQUIRE(tq * gcap <= ATQ_ROWS, "attention_prompt: tile of %d tokens x %d heads exceeds %d rows", tq, gcap, ATQ_ROWS);

@@ -445,12 +445,13 @@ PROMPT_ATTENTION_ROWS = 128      # rows a work-group of the 128-row prompt kerne
 PROMPT_ATTENTION_HEAD_DIMS = (64, 128)
 
 
-PROMPT_ATTENTION_MAX_BLOCKS = 2048     # block-table entries a work-group keeps in shared memory
+PROMPT_ATTENTION_MAX_BLOCKS = 2048     # pages of a sequence whose block-table entries a work-group keeps in shared memory
 
 
 def prompt_attention_fits(dtype: torch.dtype, head_dim: int, page_size: int, max_blocks: int = 0) -> bool:
     """Whether :func:`paged_attention_prompt` is built for this case: bfloat16, head size 64 or
-    128, pages of 8, 16, 32, ... tokens, block tables of up to 2048 entries."""
+    128, pages of 8, 16, 32, ... tokens, sequences of up to 2048 pages (``max_blocks``: the
+    longest sequence of the step in pages)."""
     return (dtype == torch.bfloat16 and head_dim in PROMPT_ATTENTION_HEAD_DIMS and page_size >= 8
             and page_size & (page_size - 1) == 0 and max_blocks <= PROMPT_ATTENTION_MAX_BLOCKS)
 
@@ -464,15 +465,17 @@ def paged_attention_prompt(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Te
                            block_table: torch.Tensor, req_indptr: torch.Tensor, ctx_lens: torch.Tensor,
                            tile_req: torch.Tensor, tile_tok0: torch.Tensor, num_tiles: int, tile_tokens: int,
                            num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
-                           scale: float) -> None:
+                           scale: float, max_total_len: int | None = None) -> None:
     """The attention of :func:`paged_attention` for prompt portions in tiles of 128 rows
     (``tile_tokens`` tokens times the heads of a group): bfloat16, head size 64 or 128, pages
     of a multiple of 8 tokens; keys and values go straight into shared memory once per
-    work-group.  Writes the rows of its tiles only."""
+    work-group.  Writes the rows of its tiles only.  ``max_total_len``: the longest sequence of the
+    step (cached + new tokens; default: what the block table could hold)."""
     T = q.shape[0]
-    if not prompt_attention_fits(q.dtype, head_dim, page_size, block_table.shape[1]):
-        raise KernelError("paged_attention_prompt: bfloat16, head size 64 or 128, pages of 8, 16, 32, ... tokens and block "
-                          f"tables of up to {PROMPT_ATTENTION_MAX_BLOCKS} entries only")
+    used_blocks = block_table.shape[1] if max_total_len is None else min(block_table.shape[1], -(-max_total_len // page_size))
+    if not prompt_attention_fits(q.dtype, head_dim, page_size, used_blocks):
+        raise KernelError("paged_attention_prompt: bfloat16, head size 64 or 128, pages of 8, 16, 32, ... tokens and "
+                          f"sequences of up to {PROMPT_ATTENTION_MAX_BLOCKS} pages only")
     if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
         raise KernelError("paged_attention_prompt: q/out shapes or dtypes do not fit")
     _check_planes("paged_attention_prompt", k_plane, v_plane, q.dtype, num_kv_heads, page_size, head_dim)
@@ -486,7 +489,7 @@ def paged_attention_prompt(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Te
                                               _ptr(block_table), c_int(block_table.stride(0)), _ptr(req_indptr),
                                               _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles),
                                               c_int(tile_tokens), c_int(num_heads), c_int(num_kv_heads), c_int(page_size),
-                                              c_int(window), c_float(scale), _stream()))
+                                              c_int(window), c_float(scale), c_int(max(1, used_blocks)), _stream()))
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:

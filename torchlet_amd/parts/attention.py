@@ -142,7 +142,7 @@ class GQAttention(Mixer):
         out = torch.empty((T, self.q_width), dtype=self.dtype, device=h.device)
         q = qkv[:, : self.q_width]
         common = (self.heads, self.kv_heads, self.head_dim, cache.page_size, self.window or 0, self.scale)
-        rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size, table.shape[1])
+        rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size, -(-ctx.max_total_len // cache.page_size))
                    and ctx.max_new_tokens >= _PORTION_MIN_TOKENS)
         portions = (self.dtype == torch.bfloat16 and self.head_dim <= ops.PREFILL_ATTENTION_MAX_HEAD_DIM
                     and cache.page_size % 4 == 0 and ctx.max_new_tokens >= _PORTION_MIN_TOKENS
@@ -153,7 +153,8 @@ class GQAttention(Mixer):
             tq = self.prompt_tile_tokens if rows128 else self.portion_tile_tokens
             kernel = ops.paged_attention_prompt if rows128 else ops.paged_attention_prefill
             short, long = ctx.tiles_by_length(self.tile_tokens, tq, _PORTION_MIN_TOKENS)
-            kernel(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens, long[0], long[1], long[2], tq, *common)
+            extra = dict(max_total_len=ctx.max_total_len) if rows128 else {}
+            kernel(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens, long[0], long[1], long[2], tq, *common, **extra)
             if short[2]:     # split over their keys; the merge of the parts is kept to the rows of these requests
                 ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
                                     short[0], short[1], short[2], self.tile_tokens, *common,

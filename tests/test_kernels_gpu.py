@@ -611,6 +611,42 @@ def test_paged_attention_prompt_tiles_of_128_rows(ops, nh, nkv, hd, page, window
         torch.testing.assert_close(got[a:b], ref, **tol)
 
 
+def test_paged_attention_prompt_takes_a_wide_block_table_for_short_sequences(ops):
+    """What bounds the 128-row kernel is the longest sequence of the step in pages, not the
+    room that the block table has: a table of 5000 entries holds a sequence of 200 tokens, and
+    a step that says it holds a sequence of 2049 pages is refused before any launch."""
+    nh, nkv, hd, page = 4, 2, 64, 8
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(16)
+    n = 200
+    bt = torch.zeros(1, 5000, dtype=torch.int32)
+    used = (n + page - 1) // page
+    bt[0, :used] = torch.randperm(used, generator=g).int() + 1
+    q = torch.randn(n, nh * hd, generator=g).to(dtype)
+    k = torch.randn(n, nkv, hd, generator=g).to(dtype)
+    v = torch.randn(n, nkv, hd, generator=g).to(dtype)
+    kp = torch.zeros(used + 1, nkv, page, hd, dtype=dtype)
+    vp = torch.zeros(used + 1, nkv, hd, page, dtype=dtype)
+    for p in range(n):
+        kp[bt[0, p // page], :, p % page] = k[p]
+        vp[bt[0, p // page], :, :, p % page] = v[p]
+    tq = ops.prompt_attention_tile_tokens(nh, nkv)
+    tile_tok0 = list(range(0, n, tq))
+    args = (kp.cuda(), vp.cuda(), bt.cuda(), torch.tensor([0, n], dtype=torch.int32).cuda(),
+            torch.zeros(1, dtype=torch.int32).cuda(), torch.zeros(len(tile_tok0), dtype=torch.int32).cuda(),
+            torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_tok0), tq, nh, nkv, hd, page, 0, 1.0 / math.sqrt(hd))
+    out = torch.full((n, nh * hd), float("nan"), dtype=dtype, device="cuda")
+    with pytest.raises(ops.KernelError, match="2048 pages"):
+        ops.paged_attention_prompt(q.cuda(), out, *args)                     # as long as the table is wide, for all the kernel knows
+    with pytest.raises(ops.KernelError, match="2048 pages"):
+        ops.paged_attention_prompt(q.cuda(), out, *args, max_total_len=2049 * page)
+    ops.paged_attention_prompt(q.cuda(), out, *args, max_total_len=n)
+    ref = _attention_ref(q.double().view(-1, nh, hd), k.double(), v.double(), 0)
+    tol = _tol(dtype)
+    torch.testing.assert_close(out.cpu().double().view(n, nh, hd), ref, rtol=tol["rtol"],
+                               atol=tol["atol"] + 2 ** -9 * float(v.abs().max()))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,I", [(3, 200), (17, 1001)])
 def test_swiglu(ops, dtype, T, I):

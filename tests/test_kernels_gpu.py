@@ -128,6 +128,32 @@ def test_linear(ops, dtype, M, N, K, bias):
     torch.testing.assert_close(out32.double(), ref, **tol32)
 
 
+@pytest.mark.parametrize("M", [1, 2, 3, 7, 8, 13, 16])
+@pytest.mark.parametrize("N,K", [(37, 100), (300, 1024), (129, 1028), (4608, 3584), (1, 2052), (64, 18944)])
+def test_linear_few_rows_in_32_bit(ops, M, N, K):
+    """The weight-streaming kernel of the 32-bit decode step: every count of rows, an odd number
+    of weight rows, K of less than one, exactly one and several chunks with a tail; against a
+    float64 product, and a row's result is the same whatever other rows stand beside it."""
+    g = torch.Generator().manual_seed(M * 11 + N)
+    x = torch.randn(M, K, generator=g).cuda()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).cuda()
+    b = torch.randn(N, generator=g).cuda()
+    ref = x.double() @ w.double().T + b.double()
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    out = torch.full((M, N), float("nan"), device="cuda")
+    ops.linear(x, w, b, out)
+    torch.testing.assert_close(out.double(), ref, **tol32)
+    alone = torch.empty(1, N, device="cuda")
+    ops.linear(x[M - 1:], w, b, alone)
+    assert torch.equal(alone[0], out[M - 1])
+    wide = torch.zeros(M, K + 24, device="cuda")          # a strided input view, a wider output
+    wide[:, 8:8 + K] = x
+    out2 = torch.full((M, N + 5), 3.0, device="cuda")
+    ops.linear(wide[:, 8:8 + K], w, None, out2[:, :N])
+    torch.testing.assert_close(out2[:, :N].double(), ref - b.double(), **tol32)
+    assert bool((out2[:, N:] == 3.0).all())
+
+
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K", [(48, 64), (129, 200), (4608, 3584), (3584, 1000), (16400, 256), (33000, 128)])

@@ -89,6 +89,83 @@ extern "C" int tl_gemm_general(const void* x, const void* w, const void* bias, i
 
 
 // =====================================================================================
+// True 32-bit, few rows (M <= 16): the decode step's products of the 32-bit engine.
+//
+// The tile kernel above computes a 64-row tile whatever M is; with one to sixteen rows the
+// product is a stream of the weight matrix and wants nothing but loads in flight.  A wave owns
+// two weight rows; its lanes walk them in 16-byte pieces (lane, lane + 64, ...), multiply each
+// piece with the matching piece of every x row (GV_KC columns of x at a time wait in shared
+// memory) and keep one partial sum per (x row, weight row); at the end the 64 partial sums are
+// added up in a fixed butterfly order.  A row's result therefore depends on neither M nor the
+// other rows, as in the tile kernel, but its rounding differs from the tile kernel's (another
+// order of the same sum).  Needs K % 4 == 0 and 16-byte aligned rows.
+#define GV_ROWS 8
+template <int MR>
+__global__ __launch_bounds__(256) void gemv_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                       const void* __restrict__ bias, int bias_f32,
+                                                       float* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+    constexpr int KC = MR > 8 ? 512 : 1024;        // 32 KB of x at most
+    __shared__ float4 xs[MR][KC / 4];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n0 = blockIdx.x * GV_ROWS + wave * 2;
+    const float* wa = w + (size_t)min(n0, N - 1) * K;        // rows past the end: read the last row, write nothing
+    const float* wb = w + (size_t)min(n0 + 1, N - 1) * K;
+    float acc[MR][2];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m][0] = acc[m][1] = 0.f;
+
+    for (int k0 = 0; k0 < K; k0 += KC) {
+        const int pieces = min(KC, K - k0) / 4;
+        __syncthreads();
+        for (int i = threadIdx.x; i < MR * (KC / 4); i += 256) {
+            const int m = i / (KC / 4), c = i % (KC / 4);
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m < M && c < pieces) v = *(const float4*)(x + (size_t)m * ldx + k0 + 4 * c);
+            xs[m][c] = v;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int c = lane; c < pieces; c += 64) {
+            const float4 a = *(const float4*)(wa + k0 + 4 * c);
+            const float4 b = *(const float4*)(wb + k0 + 4 * c);
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                const float4 xv = xs[m][c];
+                acc[m][0] = fmaf(a.w, xv.w, fmaf(a.z, xv.z, fmaf(a.y, xv.y, fmaf(a.x, xv.x, acc[m][0]))));
+                acc[m][1] = fmaf(b.w, xv.w, fmaf(b.z, xv.z, fmaf(b.y, xv.y, fmaf(b.x, xv.x, acc[m][1]))));
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int r = 0; r < 2; ++r) acc[m][r] = wave_sum(acc[m][r]);
+    if (lane < 2 && n0 + lane < N) {
+        const int n = n0 + lane;
+        const float b = bias ? load_vec(bias, bias_f32, n) : 0.f;
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+            if (m < M) out[(size_t)m * ldo + n] = (lane ? acc[m][1] : acc[m][0]) + b;
+    }
+}
+
+static bool gemv_f32_fits(const void* x, const void* w, int M, int K, int ldx) {
+    return M <= 16 && K % 4 == 0 && ldx % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
+}
+
+static void launch_gemv_f32(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                            int ldx, int ldo, hipStream_t stream) {
+    dim3 grid((N + GV_ROWS - 1) / GV_ROWS), block(256);
+#define GV_LAUNCH(MR) gemv_f32_kernel<MR><<<grid, block, 0, stream>>>((const float*)x, (const float*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo)
+    if (M <= 1) GV_LAUNCH(1);
+    else if (M <= 2) GV_LAUNCH(2);
+    else if (M <= 4) GV_LAUNCH(4);
+    else if (M <= 8) GV_LAUNCH(8);
+    else GV_LAUNCH(16);
+#undef GV_LAUNCH
+}
+
+// =====================================================================================
 // bfloat16 on the matrix cores, few rows (M <= 64): the decode step's products.
 //
 // Such a product is a stream of the weight matrix through the chip once; the kernel is
@@ -930,6 +1007,7 @@ static bool skinny_fits(const void* x, const void* w, int M, int K, int ldx) {
 //   bfloat16, aligned, K a multiple of 64, M > 32 (M > 8 against a wide matrix) -> gemm_dl_tile
 //                                  (matrix cores, operands straight into shared memory)
 //   bfloat16, aligned, M > 64   -> gemm_mfma_tile (matrix cores, shared-memory tiles)
+//   32-bit, aligned, M <= 16    -> gemv_f32 (true 32-bit arithmetic, weight streaming)
 //   everything else             -> gemm_tile (true 32-bit arithmetic)
 extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_f32, void* out,
                        int M, int N, int K, int ldx, int ldo, int dtype, int out_f32, hipStream_t stream) {
@@ -962,6 +1040,11 @@ extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_
         else if (M <= 32) pick_skinny<2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
         else pick_skinny<4>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
         TL_CHECK_LAUNCH("gemm_skinny");
+        return TL_OK;
+    }
+    if (dtype == TL_DT_F32 && gemv_f32_fits(x, w, M, K, ldx)) {
+        launch_gemv_f32(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream);
+        TL_CHECK_LAUNCH("gemv_f32");
         return TL_OK;
     }
     return tl_gemm_general(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, dtype, out_f32, stream);

@@ -221,16 +221,17 @@ def test_linear_many_rows_fetched_straight_into_shared_memory(ops, out_dtype, ti
     torch.testing.assert_close(out.double(), ref, **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
     wide = torch.zeros(M, K + 40, dtype=torch.bfloat16, device="cuda")
     wide[:, 16:16 + K] = x
-    out2 = torch.empty_like(out)
-    ops.linear_direct_variant(wide[:, 16:16 + K], w, None, out2, *tile)
-    torch.testing.assert_close(out2.double(), ref - b.double(), **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
+    out2 = torch.full((M, N + 8), 5.0, dtype=out_dtype, device="cuda")      # rows of a wider buffer
+    ops.linear_direct_variant(wide[:, 16:16 + K], w, None, out2[:, :N], *tile)
+    torch.testing.assert_close(out2[:, :N].double(), ref - b.double(), **(tol32 if out_dtype == torch.float32 else _tol(torch.bfloat16)))
+    assert bool((out2[:, N:] == 5.0).all())
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 32, 33, 64, 65, 300])
-@pytest.mark.parametrize("I,K", [(128, 64), (200, 96), (112, 80), (18944, 256), (32768 + 40, 64)])
+@pytest.mark.parametrize("I,K", [(128, 64), (200, 96), (112, 80), (18944, 256), (32768 + 40, 64), (100, 128), (36, 64)])
 def test_linear_swiglu_fused(ops, M, I, K):
     """The gate/up product with the gate applied to the accumulators: every kernel behind it
-    (few rows, 64-row tile, 128 and 256-row tiles), with I not a multiple of 32."""
+    (few rows, 64-row tile, 128 and 256-row tiles), with I not a multiple of 32 or of 8."""
     g = torch.Generator().manual_seed(M + I)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
     gate = (torch.randn(I, K, generator=g) / math.sqrt(K) * 2).to(torch.bfloat16).cuda()

@@ -747,13 +747,19 @@ __device__ __forceinline__ void load_to_lds(const void* gptr, unsigned lds_addr)
 template <int N>
 __device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW = false>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW = false, int TK = 64>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                       const void* __restrict__ bias, int bias_f32,
                                                                       TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
                                                                       int out_cols, int k_per_split) {
     static_assert(!SW || (BN / WGN) % 64 == 0, "the fused gate needs whole 64-row blocks per wave");
-    constexpr int TK = 64;
+    static_assert(TK == 64 || TK == 32, "slabs of 64 or 32 columns");
+    // A slab row holds PPR pieces of 16 bytes; one load instruction of a wave fills RPL rows.  With
+    // slabs of 32 columns a row is 64 bytes and piece c of row r lies in slot c ^ ((r >> 2) & 3): the
+    // sixteen rows a quarter-wave reads then fall on all 64 banks as well.  Half the slab is half the
+    // shared memory per stage: twice as many stages fit, and a request has twice as long to arrive.
+    constexpr int PPR = TK / 8, RPL = 64 / PPR;
+#define DL_SWZ(r) (TK == 64 ? (((r) >> 1) & 7) : (((r) >> 2) & 3))
     // Split K (k_per_split > 0, a multiple of 64): blockIdx.y owns the columns [y * k_per_split, ...) of
     // x and w and writes its own [M, ldo] slab of partial sums to out; whoever reads them adds the slabs up.
     const int ldw = K;
@@ -768,10 +774,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
     constexpr int WM = BM / WGM, WN = BN / WGN;          // wave tile
     constexpr int FM = WM / 32, FN = WN / 32;            // 32x32 blocks per wave
     constexpr int ROWS = BM + BN;
-    constexpr int LOADS = ROWS / 8 / NW;                 // load instructions per wave and slab (8 rows each)
-    static_assert(ROWS % (8 * NW) == 0, "slab rows must divide over the waves");
-    static_assert(LOADS * (STAGES - 2) < 64, "outstanding loads must fit the counter");
-    extern __shared__ __attribute__((aligned(16))) bf16_t lds_raw[];   // [STAGES][ROWS][64]
+    constexpr int LOADS = ROWS / RPL / NW;               // load instructions per wave and slab (RPL rows each)
+    static_assert(ROWS % (RPL * NW) == 0, "slab rows must divide over the waves");
+    static_assert(LOADS * (STAGES - 1) < 64, "outstanding loads must fit the counter");
+    extern __shared__ __attribute__((aligned(16))) bf16_t lds_raw[];   // [STAGES][ROWS][TK]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -792,14 +798,14 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
     }
     const int m0 = tm * BM, n0 = tn * BN;
 
-    // instruction j of this wave fills rows 8 (wave + j NW) .. + 8 of the stacked [x rows; w rows] slab
+    // instruction j of this wave fills rows RPL (wave + j NW) .. + RPL of the stacked [x rows; w rows] slab
     const bf16_t* src[LOADS];
     int ldst[LOADS];
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
-        const int base_row = 8 * (wave + j * NW);
-        const int row = base_row + (lane >> 3);
-        const int c = (lane & 7) ^ ((row >> 1) & 7);
+        const int base_row = RPL * (wave + j * NW);
+        const int row = base_row + lane / PPR;
+        const int c = (lane % PPR) ^ DL_SWZ(row);
         if (row < BM) src[j] = x + (size_t)min(m0 + row, M - 1) * ldx + c * 8;
         else src[j] = w + (size_t)min(n0 + row - BM, N - 1) * ldw + c * 8;
         ldst[j] = __builtin_amdgcn_readfirstlane(base_row * TK * 2);
@@ -815,106 +821,162 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
     const int slabs = K / TK;
-#pragma unroll
-    for (int st = 0; st < STAGES - 1; ++st) {
-        const int k0 = min(st, slabs - 1) * TK;
-#pragma unroll
-        for (int j = 0; j < LOADS; ++j) load_to_lds(src[j] + k0, lds_base + st * ROWS * TK * 2 + ldst[j]);
-    }
-    wait_direct_loads<(STAGES - 2) * LOADS>();
-    __syncthreads();
-
     const int fr = lane & 31, fh = lane >> 5;
     int arow[FM], brow[FN], akey[FM], bkey[FN];
 #pragma unroll
-    for (int i = 0; i < FM; ++i) { arow[i] = wm * WM + i * 32 + fr; akey[i] = (arow[i] >> 1) & 7; }
+    for (int i = 0; i < FM; ++i) { arow[i] = wm * WM + i * 32 + fr; akey[i] = DL_SWZ(arow[i]); }
 #pragma unroll
-    for (int j = 0; j < FN; ++j) { brow[j] = BM + wn * WN + j * 32 + fr; bkey[j] = (brow[j] >> 1) & 7; }
+    for (int j = 0; j < FN; ++j) { brow[j] = BM + wn * WN + j * 32 + fr; bkey[j] = DL_SWZ(brow[j]); }
+#undef DL_SWZ
 
+    // The loop is a hand-laid pipeline; scheduling fences keep the compiler from undoing it.  A step
+    // of TK columns has TK / 16 phases of FM * FN products.  Each phase first issues the operand reads
+    // of the next phase into the other register set, then its products, so a read has a whole
+    // phase to arrive.  The last phase of a step waits for the next slab, meets the other waves at
+    // the barrier (they have all read their last operands of this slab by then), requests the slab
+    // STAGES - 1 ahead into the buffer just given up, and reads the first operands of the next slab,
+    // all before its own products.  Past the end the last slab is requested again (nobody reads
+    // it), so the count of requests in flight is the same in every step, which the wait relies on.
+    Frag16 af[2][FM], bfr[2][FN];
+    auto read_operands = [&](int set, const bf16_t* cb, int kk) {
+        const int c = 2 * kk + fh;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) af[set][i].u = *(const uint4*)(cb + arow[i] * TK + ((c ^ akey[i]) * 8));
+#pragma unroll
+        for (int j = 0; j < FN; ++j) bfr[set][j].u = *(const uint4*)(cb + brow[j] * TK + ((c ^ bkey[j]) * 8));
+    };
+    auto request_slab = [&](int slab) {
+        const int k0 = min(slab, slabs - 1) * TK;
+        const unsigned nb = lds_base + (slab % STAGES) * ROWS * TK * 2;
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j) load_to_lds(src[j] + k0, nb + ldst[j]);
+    };
+#pragma unroll
+    for (int st = 0; st < STAGES - 1; ++st) request_slab(st);
+    wait_direct_loads<(STAGES - 2) * LOADS>();
+    __syncthreads();
+    request_slab(STAGES - 1);
+    read_operands(0, lds_raw, 0);
+    __builtin_amdgcn_sched_barrier(0);
+
+    constexpr int PHASES = TK / 16;
     for (int sl = 0; sl < slabs; ++sl) {
-        {   // past the end the last slab is requested again (nobody reads it): the count of requests
-            // in flight stays the same in every step, which the wait below relies on
-            const int k0 = min(sl + STAGES - 1, slabs - 1) * TK;
-            const unsigned nb = lds_base + ((sl + STAGES - 1) % STAGES) * ROWS * TK * 2;
-#pragma unroll
-            for (int j = 0; j < LOADS; ++j) load_to_lds(src[j] + k0, nb + ldst[j]);
-        }
         const bf16_t* cb = lds_raw + (sl % STAGES) * ROWS * TK;
-        Frag16 af[2][FM], bfr[2][FN];
 #pragma unroll
-        for (int i = 0; i < FM; ++i) af[0][i].u = *(const uint4*)(cb + arow[i] * TK + ((fh ^ akey[i]) * 8));
-#pragma unroll
-        for (int j = 0; j < FN; ++j) bfr[0][j].u = *(const uint4*)(cb + brow[j] * TK + ((fh ^ bkey[j]) * 8));
-#pragma unroll
-        for (int kk = 0; kk < TK / 16; ++kk) {
-            if (kk + 1 < TK / 16) {
-                const int c = 2 * (kk + 1) + fh;
-#pragma unroll
-                for (int i = 0; i < FM; ++i) af[(kk + 1) & 1][i].u = *(const uint4*)(cb + arow[i] * TK + ((c ^ akey[i]) * 8));
-#pragma unroll
-                for (int j = 0; j < FN; ++j) bfr[(kk + 1) & 1][j].u = *(const uint4*)(cb + brow[j] * TK + ((c ^ bkey[j]) * 8));
+        for (int kk = 0; kk < PHASES; ++kk) {
+            const int cur = kk & 1, nxt = cur ^ 1;
+            if (kk + 1 < PHASES) {
+                read_operands(nxt, cb, kk + 1);
+            } else {
+                wait_direct_loads<(STAGES - 2) * LOADS>();
+                __syncthreads();
+                request_slab(sl + STAGES);
+                read_operands(nxt, lds_raw + ((sl + 1) % STAGES) * ROWS * TK, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i].v, bfr[kk & 1][j].v, acc[i][j], 0, 0, 0);
-            if (kk + 1 < TK / 16) {      // one operand read of the next step between the products of this one
-#pragma unroll
-                for (int q = 0; q < FM + FN; ++q) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                }
-                if (FM * FN > FM + FN) __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - (FM + FN), 0);
-            }
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j].v, af[cur][i].v, acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        wait_direct_loads<(STAGES - 2) * LOADS>();
-        __syncthreads();
     }
     wait_direct_loads<0>();
 
-    // block result: lane holds column (lane % 32), rows 8 * (v / 4) + 4 * (lane / 32) + v % 4
-    if (SW) {   // even blocks hold gate columns, the next block the up columns of the same outputs
+    // The products are taken as weight block times x block, so of a 32x32 block a lane holds one
+    // row of x, m = lane % 32, and sixteen output columns n = 8 (v / 4) + 4 (lane / 32) + v % 4:
+    // four neighbours at a time.  With the fused gate, even blocks hold gate columns and the next
+    // block the up columns of the same 32 outputs.
+    const int lm = lane & 31, half = lane >> 5;
+    constexpr int WNO = SW ? WN / 2 : WN;                   // output columns of a wave tile
+    constexpr int FNO = SW ? FN / 2 : FN;                   // and its blocks of 32 of them
+    const int cols = SW ? out_cols : N;                     // output columns in all
+    const int c0 = (SW ? n0 / 2 : n0) + wn * WNO;           // first output column and row of this wave
+    const int r0 = m0 + wm * WM;
+    auto value = [&](int i, int jo, int v) -> float {
+        if constexpr (SW) return silu_mul(acc[i][2 * jo][v], acc[i][2 * jo + 1][v]);
+        else return acc[i][jo][v];
+    };
+    auto bias_at = [&](int n) -> float { return (!SW && bias && n < cols) ? load_vec(bias, bias_f32, n) : 0.f; };
+
+    if constexpr (sizeof(TOut) == 2) {
+        if (cols % 8 == 0 && ldo % 8 == 0 && ((uintptr_t)out % 16) == 0) {
+            // bfloat16 rows that can be stored in 16-byte pieces: the wave lays its tile out row by
+            // row in shared memory (the slab buffers are free now; 16-byte piece c of row r in slot
+            // c ^ (r % C) against bank conflicts) and stores it in whole rows, 64 lanes times 16
+            // bytes per instruction, instead of two bytes per lane and store.
+            constexpr int C = WNO / 8;
+            static_assert((C & (C - 1)) == 0, "pieces per row must be a power of two");
+            static_assert(BM * (SW ? BN / 2 : BN) <= STAGES * ROWS * TK, "the result tile must fit the slab buffers");
+            __syncthreads();
+            bf16_t* stage = lds_raw + wave * (WM * WNO);
 #pragma unroll
-        for (int j = 0; j + 1 < FN; j += 2) {
-            const int col = (n0 + wn * WN + j * 32) / 2 + (lane & 31);
-            if (col >= out_cols) continue;
+            for (int i = 0; i < FM; ++i)
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
+                for (int jo = 0; jo < FNO; ++jo)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                    if (m < M) out[(size_t)m * ldo + col] = from_float<TOut>(silu_mul(acc[i][j][v], acc[i][j + 1][v]));
+                    for (int g = 0; g < 4; ++g) {
+                        const int n = jo * 32 + 8 * g + 4 * half;
+                        bf16_t h[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) h[e] = from_float<bf16_t>(value(i, jo, 4 * g + e) + bias_at(c0 + n + e));
+                        uint2 packed;
+                        packed.x = (uint32_t)h[0].bits | ((uint32_t)h[1].bits << 16);
+                        packed.y = (uint32_t)h[2].bits | ((uint32_t)h[3].bits << 16);
+                        const int row = i * 32 + lm;
+                        *(uint2*)(stage + row * WNO + (((n >> 3) ^ (row & (C - 1))) * 8) + (n & 4)) = packed;
+                    }
+            // (one wave's shared-memory accesses are carried out in order: no wait in between)
+#pragma unroll
+            for (int q = 0; q < WM * C / 64; ++q) {
+                const int idx = q * 64 + lane;
+                const int row = idx / C, piece = idx % C;
+                const uint4 val = *(const uint4*)(stage + row * WNO + ((piece ^ (row & (C - 1))) * 8));
+                const int m = r0 + row, n = c0 + piece * 8;
+                if (m < M && n < cols) *(uint4*)((bf16_t*)out + (size_t)m * ldo + n) = val;
+            }
+            return;
+        }
+    }
+    const bool quads = sizeof(TOut) == 4 && cols % 4 == 0 && ldo % 4 == 0 && ((uintptr_t)out % 16) == 0;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const int m = r0 + i * 32 + lm;
+        if (m >= M) continue;
+#pragma unroll
+        for (int jo = 0; jo < FNO; ++jo)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = c0 + jo * 32 + 8 * g + 4 * half;
+                if (quads) {
+                    if (n < cols) {
+                        float4 f;
+                        f.x = value(i, jo, 4 * g) + bias_at(n);
+                        f.y = value(i, jo, 4 * g + 1) + bias_at(n + 1);
+                        f.z = value(i, jo, 4 * g + 2) + bias_at(n + 2);
+                        f.w = value(i, jo, 4 * g + 3) + bias_at(n + 3);
+                        *(float4*)((float*)out + (size_t)m * ldo + n) = f;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < cols) out[(size_t)m * ldo + n + e] = from_float<TOut>(value(i, jo, 4 * g + e) + bias_at(n + e));
                 }
             }
-        }
-        return;
-    }
-#pragma unroll
-    for (int j = 0; j < FN; ++j) {
-        const int n = n0 + wn * WN + j * 32 + (lane & 31);
-        if (n >= N) continue;
-        const float b = bias ? load_vec(bias, bias_f32, n) : 0.f;
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                if (m < M) out[(size_t)m * ldo + n] = from_float<TOut>(acc[i][j][v] + b);
-            }
-        }
     }
 }
 
 // Tile shapes of the direct-load kernel and which one a product gets.  Estimate per shape: the
 // tiles are dealt to 256 compute units, each works through ceil(tiles / 256) of them one after
-// the other at the rate the shape reaches on a full machine (measured at Qwen2.5-7B sizes,
-// TFLOP/s: 64x64 700, 64x256 800, 128x128 900, 128x256 950, 256x128 1000, 256x256 1100), plus
-// about 2 us per tile for filling the pipeline and storing the result.
+// the other; a tile takes a fixed time (filling the pipeline, storing the result) plus its
+// products at the rate one compute unit reaches with that shape (fitted to measurements at
+// 2048 rows against the Qwen2.5-7B and 14B matrices, K from 3584 to 18944).
 enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_256x256, DL_TILES };
 static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 256};
 static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256};
-static const double DL_RATE[DL_TILES] = {700e12, 800e12, 900e12, 950e12, 1000e12, 1100e12};
+static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 6.1e12};     // FLOP/s of one compute unit
+static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 14e-6};        // seconds per tile
 
 static DlTile pick_dl_tile(int M, int N, int K, bool sw) {
     DlTile best = DL_128x128;
@@ -922,18 +984,18 @@ static DlTile pick_dl_tile(int M, int N, int K, bool sw) {
     for (int t = 0; t < DL_TILES; ++t) {
         if (sw && t == DL_64x64) continue;               // a wave of the fused gate needs 64 weight rows
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
-        const double per_tile = 2.0 * DL_BM[t] * DL_BN[t] * K / (DL_RATE[t] / 256) + 2e-6;
+        const double per_tile = 2.0 * DL_BM[t] * DL_BN[t] * K / DL_RATE[t] + DL_FIXED[t];
         const double est = (double)((tiles + 255) / 256) * per_tile;
         if (est < best_t) { best_t = est; best = (DlTile)t; }
     }
     return best;
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW>
+template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW, int TK = 64>
 static int launch_dl_tile_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                             int ldx, int ldo, int out_cols, hipStream_t stream) {
-    constexpr size_t lds = (size_t)STAGES * (BM + BN) * 64 * sizeof(bf16_t);
-    auto kernel = gemm_dl_tile_kernel<BM, BN, WGM, WGN, STAGES, TOut, SW>;
+    constexpr size_t lds = (size_t)STAGES * (BM + BN) * TK * sizeof(bf16_t);
+    auto kernel = gemm_dl_tile_kernel<BM, BN, WGM, WGN, STAGES, TOut, SW, TK>;
     static hipError_t allowed = allow_lds(kernel, lds);
     if (allowed != hipSuccess) {
         tl_set_error("gemm_dl_tile: cannot get %zu bytes of shared memory: %s", lds, hipGetErrorString(allowed));

@@ -904,10 +904,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
         if (cols % 8 == 0 && ldo % 8 == 0 && ((uintptr_t)out % 16) == 0) {
             // bfloat16 rows that can be stored in 16-byte pieces: the wave lays its tile out row by
             // row in shared memory (the slab buffers are free now; 16-byte piece c of row r in slot
-            // c ^ (r % C) against bank conflicts) and stores it in whole rows, 64 lanes times 16
+            // c ^ (r % CX) against bank conflicts) and stores it in whole rows, 64 lanes times 16
             // bytes per instruction, instead of two bytes per lane and store.
             constexpr int C = WNO / 8;
-            static_assert((C & (C - 1)) == 0, "pieces per row must be a power of two");
+            constexpr int CX = C & -C;                       // the slots are exchanged within groups of CX, a power of two
+            static_assert((WM * C) % 64 == 0, "the rows of a wave tile must divide over its lanes");
             static_assert(BM * (SW ? BN / 2 : BN) <= STAGES * ROWS * TK, "the result tile must fit the slab buffers");
             __syncthreads();
             bf16_t* stage = lds_raw + wave * (WM * WNO);
@@ -925,14 +926,14 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
                         packed.x = (uint32_t)h[0].bits | ((uint32_t)h[1].bits << 16);
                         packed.y = (uint32_t)h[2].bits | ((uint32_t)h[3].bits << 16);
                         const int row = i * 32 + lm;
-                        *(uint2*)(stage + row * WNO + (((n >> 3) ^ (row & (C - 1))) * 8) + (n & 4)) = packed;
+                        *(uint2*)(stage + row * WNO + (((n >> 3) ^ (row & (CX - 1))) * 8) + (n & 4)) = packed;
                     }
             // (one wave's shared-memory accesses are carried out in order: no wait in between)
 #pragma unroll
             for (int q = 0; q < WM * C / 64; ++q) {
                 const int idx = q * 64 + lane;
                 const int row = idx / C, piece = idx % C;
-                const uint4 val = *(const uint4*)(stage + row * WNO + ((piece ^ (row & (C - 1))) * 8));
+                const uint4 val = *(const uint4*)(stage + row * WNO + ((piece ^ (row & (CX - 1))) * 8));
                 const int m = r0 + row, n = c0 + piece * 8;
                 if (m < M && n < cols) *(uint4*)((bf16_t*)out + (size_t)m * ldo + n) = val;
             }
@@ -972,17 +973,17 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
 // the other; a tile takes a fixed time (filling the pipeline, storing the result) plus its
 // products at the rate one compute unit reaches with that shape (fitted to measurements at
 // 2048 rows against the Qwen2.5-7B and 14B matrices, K from 3584 to 18944).
-enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_256x256, DL_TILES };
-static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 256};
-static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256};
-static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 6.1e12};     // FLOP/s of one compute unit
-static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 14e-6};        // seconds per tile
+enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_TILES };
+static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 192, 256, 256};
+static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256};
+static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12};   // FLOP/s of one compute unit
+static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6};         // seconds per tile
 
 static DlTile pick_dl_tile(int M, int N, int K, bool sw) {
     DlTile best = DL_128x128;
     double best_t = 1e30;
     for (int t = 0; t < DL_TILES; ++t) {
-        if (sw && t == DL_64x64) continue;               // a wave of the fused gate needs 64 weight rows
+        if (sw && (t == DL_64x64 || t == DL_256x192)) continue;      // a wave of the fused gate needs whole 64-row blocks of weights
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
         const double per_tile = 2.0 * DL_BM[t] * DL_BN[t] * K / DL_RATE[t] + DL_FIXED[t];
         const double est = (double)((tiles + 255) / 256) * per_tile;
@@ -1017,6 +1018,10 @@ static int launch_dl_tile(DlTile tile, const void* x, const void* w, const void*
     case DL_128x128: return launch_dl_tile_t<128, 128, 2, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
     case DL_128x256: return launch_dl_tile_t<128, 256, 2, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
     case DL_256x128: return launch_dl_tile_t<256, 128, 4, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    case DL_192x256: return launch_dl_tile_t<192, 256, 2, 4, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    case DL_256x192:
+        if constexpr (!SW) return launch_dl_tile_t<256, 192, 4, 2, 2, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+        else break;
     case DL_256x256: return launch_dl_tile_t<256, 256, 4, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
     default: break;
     }

@@ -88,12 +88,53 @@ class LayerCache:
     writable: bool                    # False: the run reads another run's cache
 
 
+class _PageTable:
+    """The pages of one request in one group, by logical block (0: none): a growing int32
+    array, so that a step copies rows into its block tables without touching every entry."""
+    __slots__ = ("_pages", "_n")
+
+    def __init__(self):
+        self._pages = np.zeros(16, dtype=np.int32)
+        self._n = 0
+
+    def __len__(self) -> int:
+        return self._n
+
+    def __getitem__(self, b: int) -> int:
+        if not 0 <= b < self._n:
+            raise IndexError(b)
+        return int(self._pages[b])
+
+    def __setitem__(self, b: int, page: int) -> None:
+        if not 0 <= b < self._n:
+            raise IndexError(b)
+        self._pages[b] = page
+
+    def __iter__(self):
+        return iter(self._pages[: self._n].tolist())
+
+    def extend(self, pages) -> None:
+        need = self._n + len(pages)
+        if need > len(self._pages):
+            grown = np.zeros(max(need, 2 * len(self._pages)), dtype=np.int32)
+            grown[: self._n] = self._pages[: self._n]
+            self._pages = grown
+        self._pages[self._n: need] = pages
+        self._n = need
+
+    def append(self, page: int) -> None:
+        self.extend([page])
+
+    def view(self) -> np.ndarray:
+        return self._pages[: self._n]
+
+
 class _Group:
     def __init__(self, need: PagedNeed, num_pages: int):
         self.need = need
         self.runs: list[int] = []                 # indices into the run order, in order
         self.pool = PagePool(num_pages)
-        self.tables: dict[object, list[int]] = {}  # request -> page of each logical block (0: none)
+        self.tables: dict[object, _PageTable] = {}  # request -> page of each logical block (0: none)
         self.tensor: torch.Tensor | None = None
 
 
@@ -196,15 +237,16 @@ class CacheManager:
         return max(0, length - g.need.window + 1) // self.page_size
 
     def pages_missing(self, req_id, new_length: int) -> list[int]:
-        """Per group, the pages that ``reserve(req_id, new_length)`` would take."""
+        """Per group, the pages that ``reserve(req_id, new_length)`` would take.  (A request's
+        table holds pages exactly from the first block a query at its length can still read to
+        the table's end: what is missing is counted, not looked for.)"""
         length = self._requests[req_id].length if req_id in self._requests else 0
         blocks = -(-new_length // self.page_size)
         out = []
         for g in self.groups:
-            table = g.tables.get(req_id, [])
+            held_to = len(g.tables.get(req_id, ()))
             first = self._first_live_block(g, length)
-            have = sum(1 for b in range(first, min(len(table), blocks)) if table[b])
-            out.append(max(0, blocks - first) - have)
+            out.append(max(0, blocks - max(first, held_to)))
         return out
 
     def pages_for(self, length: int) -> list[int]:
@@ -220,7 +262,7 @@ class CacheManager:
         slot = self._free_slots.pop()
         self._requests[req_id] = _Request(slot)
         for g in self.groups:
-            g.tables[req_id] = []
+            g.tables[req_id] = _PageTable()
         for s in self._states:
             if s is not None:
                 s[slot].zero_()
@@ -239,11 +281,10 @@ class CacheManager:
         for g in self.groups:
             table = g.tables[req_id]
             first = self._first_live_block(g, r.length)
-            while len(table) < blocks:
-                table.append(0)
-            for b in range(first, blocks):
-                if table[b] == 0:
-                    table[b] = g.pool.take(1)[0]
+            if len(table) < min(first, blocks):         # blocks no query of the step can read: never held
+                table.extend([0] * (min(first, blocks) - len(table)))
+            if len(table) < blocks:
+                table.extend(g.pool.take(blocks - len(table)))
         return True
 
     def commit(self, req_id, new_length: int) -> None:
@@ -252,13 +293,14 @@ class CacheManager:
         r = self._req(req_id)
         if new_length < r.length:
             raise CacheError(f"request {req_id!r} holds {r.length} tokens; cannot shrink to {new_length}")
-        r.length = new_length
+        old_length, r.length = r.length, new_length
         for g in self.groups:
             if g.need.window is None:
                 continue
             table = g.tables[req_id]
             first = min(self._first_live_block(g, new_length), len(table))
-            dead = [b for b in range(first) if table[b]]
+            was_first = min(self._first_live_block(g, old_length), first)     # blocks below were given back earlier
+            dead = [b for b in range(was_first, first) if table[b]]
             g.pool.give([table[b] for b in dead])
             for b in dead:
                 table[b] = 0
@@ -288,7 +330,7 @@ class CacheManager:
         out = np.zeros((len(tables), width), dtype=np.int32)
         for i, t in enumerate(tables):
             n = min(len(t), width)
-            out[i, :n] = t[:n]
+            out[i, :n] = t.view()[:n]
         return out
 
     def layer_cache(self, run: int) -> LayerCache | None:
@@ -308,6 +350,10 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             held: dict[int, object] = {}
             for req, table in g.tables.items():
+                pages = list(table)
+                held_from = next((b for b, p in enumerate(pages) if p), len(pages))
+                if not all(pages[held_from:]):
+                    raise CacheError(f"group {gi}: request {req!r} has a gap among its held pages")
                 for p in table:
                     if p == 0:
                         continue

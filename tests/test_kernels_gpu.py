@@ -66,13 +66,18 @@ def test_add_rmsnorm(ops, dtype, wdtype, T, H, eps):
     torch.testing.assert_close(out3.double(), ref[rows.long()], **_tol(dtype))
 
 
-@pytest.mark.parametrize("M", [1, 8, 16, 33, 64])
+@pytest.mark.parametrize("M", [1, 8, 16, 33, 64, 65, 200, 513])
 @pytest.mark.parametrize("N,K", [(3584, 18944), (100, 8192 + 200), (64, 64), (130, 4096)])
 def test_linear_partials_and_their_sum_in_the_norm(ops, M, N, K):
     """Split-K slabs of partial sums: their sum is the product, and add_rmsnorm adds them up."""
     g = torch.Generator().manual_seed(M + N)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).cuda()
+    if M > 64 and K % 64:
+        assert not ops.linear_partials_pay(M, N, K)
+        with pytest.raises(ops.KernelError, match="multiple of 64"):
+            ops.linear_partials(x, w)
+        return
     parts = ops.linear_partials(x, w)
     assert parts.dim() == 3 and parts.shape[1:] == (M, N) and parts.dtype == torch.float32
     assert parts.shape[0] == min(8, max(1, -(-K // 64) // 32)) or parts.shape[0] >= 1

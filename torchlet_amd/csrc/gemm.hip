@@ -979,22 +979,58 @@ static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256};
 static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12};   // FLOP/s of one compute unit
 static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6};         // seconds per tile
 
-static DlTile pick_dl_tile(int M, int N, int K, bool sw) {
+// Seconds for `groups` work-groups of tile t over k columns each.  The two smallest tiles run two
+// to a compute unit: each then works at half the unit's rate, and one that has a unit to itself
+// (not more work-groups than units) at about 0.62 of it.
+static double dl_estimate(DlTile t, long groups, int k) {
+    const bool pairs = t == DL_64x64 || t == DL_128x128;
+    const double products = 2.0 * DL_BM[t] * DL_BN[t] * k;
+    if (!pairs) return (double)((groups + 255) / 256) * (products / DL_RATE[t] + DL_FIXED[t]);
+    const double rate = groups > 256 ? DL_RATE[t] / 2 : DL_RATE[t] * 0.62;
+    return (double)((groups + 511) / 512) * (products / rate + DL_FIXED[t]);
+}
+
+static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = nullptr) {
     DlTile best = DL_128x128;
     double best_t = 1e30;
     for (int t = 0; t < DL_TILES; ++t) {
         if (sw && (t == DL_64x64 || t == DL_256x192)) continue;      // a wave of the fused gate needs whole 64-row blocks of weights
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
-        const double per_tile = 2.0 * DL_BM[t] * DL_BN[t] * K / DL_RATE[t] + DL_FIXED[t];
-        const double est = (double)((tiles + 255) / 256) * per_tile;
+        const double est = dl_estimate((DlTile)t, tiles, K);
         if (est < best_t) { best_t = est; best = (DlTile)t; }
+    }
+    if (estimate) *estimate = best_t;
+    return best;
+}
+
+// More than 64 rows against a matrix whose output tiles leave compute units idle (a few hundred rows
+// of a prompt portion against the down projection, say): K split over `parts` work-groups per tile
+// into float slabs that the consumer adds up.  Only the tiles that have a compute unit to themselves
+// are considered; the slabs cost their bytes once written and once read.  parts == 1: no split pays.
+struct DlSplit { DlTile tile; int parts; int k_per; };
+static DlSplit plan_dl_split(int M, int N, int K) {
+    double best_t;
+    DlSplit best{pick_dl_tile(M, N, K, false, &best_t), 1, 0};
+    best_t += (double)M * N * 2 * 2 / 3e12;
+    const int steps = K / 64;
+    static const DlTile alone[] = {DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256};
+    for (DlTile t : alone) {
+        const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
+        for (int P = 2; P <= 8 && K / P >= 512; ++P) {
+            const int k_per = ((steps + P - 1) / P) * 64;
+            if ((K + k_per - 1) / k_per != P) continue;
+            // (a tenth on top: float slabs leave the kernel more slowly than the estimate's bfloat16 rows)
+            const double est = 1.1 * dl_estimate(t, tiles * P, k_per) + (double)P * M * N * 4 * 2 / 3e12;
+            if (est < best_t) { best_t = est; best = DlSplit{t, P, k_per}; }
+        }
     }
     return best;
 }
 
+// parts > 1 (float results only): K is split into `parts` ranges of k_per columns and out holds that many [M, ldo] slabs.
 template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW, int TK = 64>
 static int launch_dl_tile_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
-                            int ldx, int ldo, int out_cols, hipStream_t stream) {
+                            int ldx, int ldo, int out_cols, hipStream_t stream, int parts = 1, int k_per = 0) {
     constexpr size_t lds = (size_t)STAGES * (BM + BN) * TK * sizeof(bf16_t);
     auto kernel = gemm_dl_tile_kernel<BM, BN, WGM, WGN, STAGES, TOut, SW, TK>;
     static hipError_t allowed = allow_lds(kernel, lds);
@@ -1002,27 +1038,28 @@ static int launch_dl_tile_t(const void* x, const void* w, const void* bias, int 
         tl_set_error("gemm_dl_tile: cannot get %zu bytes of shared memory: %s", lds, hipGetErrorString(allowed));
         return TL_ERR_HIP;
     }
-    dim3 grid(((M + BM - 1) / BM) * ((N + BN - 1) / BN)), block(64 * WGM * WGN);
-    kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0);
+    dim3 grid(((M + BM - 1) / BM) * ((N + BN - 1) / BN), parts), block(64 * WGM * WGN);
+    kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols,
+                                         parts > 1 ? k_per : 0);
     return TL_OK;
 }
 
 template <typename TOut, bool SW>
 static int launch_dl_tile(DlTile tile, const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
-                          int ldx, int ldo, int out_cols, hipStream_t stream) {
+                          int ldx, int ldo, int out_cols, hipStream_t stream, int parts = 1, int k_per = 0) {
     switch (tile) {
     case DL_64x64:
-        if constexpr (!SW) return launch_dl_tile_t<64, 64, 2, 2, 4, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+        if constexpr (!SW) return launch_dl_tile_t<64, 64, 2, 2, 4, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
         else break;
-    case DL_64x256: return launch_dl_tile_t<64, 256, 1, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
-    case DL_128x128: return launch_dl_tile_t<128, 128, 2, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
-    case DL_128x256: return launch_dl_tile_t<128, 256, 2, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
-    case DL_256x128: return launch_dl_tile_t<256, 128, 4, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
-    case DL_192x256: return launch_dl_tile_t<192, 256, 2, 4, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    case DL_64x256: return launch_dl_tile_t<64, 256, 1, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+    case DL_128x128: return launch_dl_tile_t<128, 128, 2, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+    case DL_128x256: return launch_dl_tile_t<128, 256, 2, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+    case DL_256x128: return launch_dl_tile_t<256, 128, 4, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+    case DL_192x256: return launch_dl_tile_t<192, 256, 2, 4, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_256x192:
-        if constexpr (!SW) return launch_dl_tile_t<256, 192, 4, 2, 2, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+        if constexpr (!SW) return launch_dl_tile_t<256, 192, 4, 2, 2, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
         else break;
-    case DL_256x256: return launch_dl_tile_t<256, 256, 4, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+    case DL_256x256: return launch_dl_tile_t<256, 256, 4, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     default: break;
     }
     tl_set_error("gemm_dl_tile: no instance of tile %d", (int)tile);
@@ -1061,6 +1098,24 @@ extern "C" int tl_gemm_direct_variant(const void* x, const void* w, const void* 
                            : launch_dl_tile<bf16_t, false>((DlTile)tile, x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
     if (rc != TL_OK) return rc;
     TL_CHECK_LAUNCH("gemm_dl_tile");
+    return TL_OK;
+}
+
+// One tile shape with K split into `parts` (float slabs [parts, M, N]); for tests and tuning.
+extern "C" int tl_gemm_direct_split_variant(const void* x, const void* w, void* out, int M, int N, int K, int ldx,
+                                            int BM, int BN, int parts, hipStream_t stream) {
+    TL_REQUIRE(M > 0 && K % 64 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0 && parts >= 1,
+               "gemm_direct_split: needs M > 0, K a multiple of 64 and 16-byte aligned rows");
+    int tile = -1;
+    for (int t = 0; t < DL_TILES; ++t)
+        if (DL_BM[t] == BM && DL_BN[t] == BN) tile = t;
+    TL_REQUIRE(tile >= 0, "gemm_direct_split: no tile of %d x %d", BM, BN);
+    const int steps = K / 64;
+    const int k_per = ((steps + parts - 1) / parts) * 64;
+    TL_REQUIRE((K + k_per - 1) / k_per == parts, "gemm_direct_split: %d parts leave one empty (K=%d)", parts, K);
+    const int rc = launch_dl_tile<float, false>((DlTile)tile, x, w, nullptr, 0, out, M, N, K, ldx, N, 0, stream, parts, k_per);
+    if (rc != TL_OK) return rc;
+    TL_CHECK_LAUNCH("gemm_direct_split");
     return TL_OK;
 }
 
@@ -1194,7 +1249,9 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
 // out[P, M, N] (float) = partial sums of x w^T over P ranges of K, for a product with too few output
 // tiles to fill the GPU (a narrow matrix against few rows): P work-groups per tile keep all compute
 // units busy; whoever reads the slabs adds them up.  Returns P through `parts` (the caller sizes
-// `out` for tl_gemm_partials_max()).  Where it pays (see partials_on_tiles) the direct-load tile
+// `out` for tl_gemm_partials_max()).  More than 64 rows: see plan_dl_split (measured at 512 rows:
+// 3584 x 18944 147 -> 82 us, 5120 x 13824 179 -> 82 us, 5120 x 27648 348 -> 150 us, the norm's sum
+// included).  Up to 64 rows, where it pays (see partials_on_tiles), the direct-load tile
 // kernel runs with 64 x 64 tiles (measured at 64 rows, 3584 x 18944: 31 us with four parts against
 // 90 us whole; 3584 x 3584: 9.5 against 20 us); up to 16 rows, or for other K, the skinny kernel
 // with R = 4 strips per work-group, which share every x fetch.
@@ -1210,6 +1267,7 @@ extern "C" int tl_gemm_partials_pay(int M, int N, int K);
 
 // How many parts tl_gemm_partials would use.
 extern "C" int tl_gemm_partials_parts(int M, int N, int K) {
+    if (M > 64 && K % 64 == 0) return plan_dl_split(M, N, K).parts;
     if (partials_on_tiles(M, K)) {
         const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
         int P = (int)(256 / tiles);                       // about one work-group per compute unit
@@ -1232,6 +1290,14 @@ extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, 
     TL_REQUIRE(M > 0 && N > 0 && K > 0 && ldx >= K, "gemm_partials: bad sizes M=%d N=%d K=%d", M, N, K);
     TL_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
                "gemm_partials: needs K and the row stride of x to be multiples of 8 and 16-byte aligned operands");
+    if (M > 64 && K % 64 == 0) {
+        const DlSplit plan = plan_dl_split(M, N, K);
+        *parts = plan.parts;
+        const int rc = launch_dl_tile<float, false>(plan.tile, x, w, nullptr, 0, out, M, N, K, ldx, N, 0, stream, plan.parts, plan.k_per);
+        if (rc != TL_OK) return rc;
+        TL_CHECK_LAUNCH("gemm_partials");
+        return TL_OK;
+    }
     const int steps = (K + 63) / 64;
     int P = tl_gemm_partials_parts(M, N, K);
     const int k_per = ((steps + P - 1) / P) * 64;

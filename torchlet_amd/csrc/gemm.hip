@@ -178,7 +178,12 @@ static void launch_gemv_f32(const void* x, const void* w, const void* bias, int 
 // one full 128-byte line; the two 16-byte halves feed two MFMAs (how k is dealt to lanes is
 // free as long as A and B agree).  The KS waves of a work-group take the steps s = wave,
 // wave + KS, ... and add their partial tiles through shared memory in a fixed order, so
-// the result is deterministic.  x is small and stays in L2.
+// the result is deterministic.  One row of x is as good as free (the lanes of a wave that read the
+// same address share the fetch); with more rows x costs M / 16 of the weight traffic again, so it is
+// copied into shared memory (XL) by no more work-groups than the compute units hold at once, each
+// of which then walks the strips blockIdx.x, blockIdx.x + gridDim.x, ... and requests the first
+// steps of its next strip before it adds up the sums of this one (measured at M = 8, 7B sizes:
+// gate/up 57 -> 51 us, LM head 207 -> 189 us).
 // Needs K % 8 == 0 and 16-byte aligned rows; other shapes go to the general kernel.
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
@@ -238,7 +243,7 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
                                                               const void* __restrict__ bias, int bias_f32,
                                                               TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
                                                               int out_cols, int k_per_split, RopeArgs ra) {
-    static_assert(!SW || (R == 4 && KS > 1), "the fused gate needs four strips per work-group");
+    static_assert(!SW || (R == 1 && KS % 2 == 0), "the fused gate deals a work-group's waves to a gate strip and its up strip");
     static_assert(!RP || (R == 1 && MT == 1 && !SW), "the fused rotation is built for one strip and up to 16 rows");
     // Split K (k_per_split > 0, a multiple of 64): blockIdx.y owns the columns
     // [y * k_per_split, ...) of x and w and writes its own [M, ldo] slab of partial sums to out
@@ -256,7 +261,17 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
     bf16_t* xs = (bf16_t*)(skinny_lds + KS * R * MT * 256);             // XL: M rows of K + 8 elements
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
-    const int n0 = blockIdx.x * (16 * R);
+    // A work-group takes the strips of 16 R weight rows blockIdx.x, blockIdx.x + gridDim.x, ...: with
+    // fewer work-groups than strips, x is copied into shared memory (XL) once for all of them, and the
+    // first fetches of the next strip are on their way while the sums of this one are added up.
+    // With the fused gate (SW) a strip is 16 outputs: the first KS / 2 waves walk K for their 16 gate rows,
+    // the others for the 16 up rows of the same outputs (the interleaved matrix holds blocks of 32 gate
+    // rows followed by their 32 up rows), and the sums of both meet in shared memory.
+    constexpr int KW = SW ? KS / 2 : KS;       // waves along K per strip
+    const int kwave = SW ? wave % KW : wave;
+    const int strips = SW ? N / 32 : (N + 16 * R - 1) / (16 * R);
+    auto first_row = [&](int st) { return SW ? (st / 2) * 64 + (wave / KW) * 32 + (st % 2) * 16 : st * (16 * R); };
+    int strip = blockIdx.x;
     int rp_pos = 0, rp_page = 0;               // RP: this lane's row (li), fetched now, used in the epilogue
     if (RP) {
         const int row = min(li, M - 1);
@@ -268,7 +283,7 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
     const bf16_t* xrow[MT];
     int xoff[MT];
 #pragma unroll
-    for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + li, N - 1) * ldw;
+    for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)min(first_row(strip) + r * 16 + li, N - 1) * ldw;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         xrow[t] = x + (size_t)min(t * 16 + li, M - 1) * ldx;
@@ -277,18 +292,13 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
 #define SK_LOADB(t, k) (XL ? *(const uint4*)(&xs[xoff[t] + (k)]) : *(const uint4*)(xrow[t] + (k)))
 
     f32x4_t acc[R][MT];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int t = 0; t < MT; ++t) acc[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
     const int full = K / 64;                   // steps that lie wholly inside K
-    // this wave's steps are s = wave + i * KS, i = 0 .. mine - 1; slot d of the ring holds step i = d (mod D)
-    const int mine = full > wave ? (full - wave + KS - 1) / KS : 0;
+    // this wave's steps are s = kwave + i * KW, i = 0 .. mine - 1; slot d of the ring holds step i = d (mod D)
+    const int mine = full > kwave ? (full - kwave + KW - 1) / KW : 0;
     Frag16 wa0[D][R], wa1[D][R], wb0[D][MT], wb1[D][MT];
 #define SK_ISSUE(d, i)                                                                              \
     {                                                                                               \
-        const int k_ = 64 * (wave + (i) * KS) + SK_KOFF(lg);                                        \
+        const int k_ = 64 * (kwave + (i) * KW) + SK_KOFF(lg);                                       \
         _Pragma("unroll") for (int r = 0; r < R; ++r) {                                             \
             wa0[d][r].u = SK_LOAD(wrow[r] + k_);                                                    \
             wa1[d][r].u = SK_LOAD(wrow[r] + k_ + SK_SECOND);                                        \
@@ -311,147 +321,164 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
         }
         lds_barrier();
     }
-    for (int i = 0; i < mine; i += D) {
+    while (true) {
+        const int n0 = strip * (16 * R);       // (not SW) first output column of the strip
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            if (i + d < mine) {
-                if (XL) {
-                    const int k = 64 * (wave + (i + d) * KS) + SK_KOFF(lg);
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-                    for (int t = 0; t < MT; ++t) {
-                        wb0[d][t].u = *(const uint4*)(&xs[xoff[t] + k]);
-                        wb1[d][t].u = *(const uint4*)(&xs[xoff[t] + k + SK_SECOND]);
+            for (int t = 0; t < MT; ++t) acc[r][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < mine; i += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                if (i + d < mine) {
+                    if (XL) {
+                        const int k = 64 * (kwave + (i + d) * KW) + SK_KOFF(lg);
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) {
+                            wb0[d][t].u = *(const uint4*)(&xs[xoff[t] + k]);
+                            wb1[d][t].u = *(const uint4*)(&xs[xoff[t] + k + SK_SECOND]);
+                        }
                     }
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) {
+                            acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa0[d][r].v, wb0[d][t].v, acc[r][t], 0, 0, 0);
+                            acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa1[d][r].v, wb1[d][t].v, acc[r][t], 0, 0, 0);
+                        }
+                    if (i + d + D < mine) SK_ISSUE(d, i + d + D)
                 }
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-#pragma unroll
-                    for (int t = 0; t < MT; ++t) {
-                        acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa0[d][r].v, wb0[d][t].v, acc[r][t], 0, 0, 0);
-                        acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa1[d][r].v, wb1[d][t].v, acc[r][t], 0, 0, 0);
-                    }
-                if (i + d + D < mine) SK_ISSUE(d, i + d + D)
             }
         }
+        // the tail step (K % 64 != 0) belongs to the wave whose turn it is; pieces beyond K count as zero
+        if ((K & 63) && (full % KW) == kwave) {
+            Frag16 a0[R], a1[R], b0[MT], b1[MT];
+            const int k = 64 * full + SK_KOFF(lg);
+            const bool v0 = k + 8 <= K, v1 = k + SK_SECOND + 8 <= K;
+            const uint4 zero = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                a0[r].u = v0 ? *(const uint4*)(wrow[r] + k) : zero;
+                a1[r].u = v1 ? *(const uint4*)(wrow[r] + k + SK_SECOND) : zero;
+            }
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                b0[t].u = v0 ? SK_LOADB(t, k) : zero;
+                b1[t].u = v1 ? SK_LOADB(t, k + SK_SECOND) : zero;
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[r].v, b0[t].v, acc[r][t], 0, 0, 0);
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[r].v, b1[t].v, acc[r][t], 0, 0, 0);
+                }
+        }
+        const int next = XL ? strip + (int)gridDim.x : strips;      // without the copy of x: one strip per work-group
+        if (next < strips) {                   // the next strip's first steps, before this strip's sums
+#pragma unroll
+            for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)min(first_row(next) + r * 16 + li, N - 1) * ldw;
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+                if (d < mine) SK_ISSUE(d, d)
+        }
+
+        // D[i][j]: lane holds i = 4 * (lane / 16) + v (weight row), j = lane % 16 (activation row)
+        if (KS > 1) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    float* dst = red + ((size_t)(wave * R * MT + r * MT + t) * 64 + lane) * 4;
+                    *(f32x4_t*)dst = acc[r][t];
+                }
+            lds_barrier();
+        }
+        if (SW) {
+            for (int t = wave; t < MT; t += KS) {
+                f32x4_t gs = f32x4_t{0.f, 0.f, 0.f, 0.f}, us = gs;
+#pragma unroll
+                for (int wv = 0; wv < KW; ++wv) {
+                    gs += *(const f32x4_t*)(red + ((size_t)(wv * MT + t) * 64 + lane) * 4);
+                    us += *(const f32x4_t*)(red + ((size_t)((KW + wv) * MT + t) * 64 + lane) * 4);
+                }
+                const int m = t * 16 + li;
+                const int col = strip * 16 + 4 * lg;
+                if (m < M) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (col + v < out_cols) out[(size_t)m * ldo + col + v] = from_float<TOut>(silu_mul(gs[v], us[v]));
+                }
+            }
+        } else {
+            for (int tile = wave; tile < R * MT; tile += KS) {
+                const int r = tile / MT, t = tile % MT;
+                f32x4_t sum;
+                if (KS > 1) {
+                    sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int wv = 0; wv < KS; ++wv) sum += *(const f32x4_t*)(red + ((size_t)(wv * R * MT + tile) * 64 + lane) * 4);
+                } else {
+                    sum = acc[0][0];
+#pragma unroll
+                    for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+                        for (int tt = 0; tt < MT; ++tt)
+                            if (rr == r && tt == t) sum = acc[rr][tt];
+                }
+                const int m = t * 16 + li;
+                const int n = n0 + r * 16 + 4 * lg;
+                if (RP) {
+                    if (m >= M || n >= N) continue;                    // N is a multiple of 16 here
+                    float val[4];
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) val[v] = sum[v] + (bias ? load_vec(bias, bias_f32, n + v) : 0.f);
+                    const int head = n / ra.head_dim, dd = n - head * ra.head_dim;
+                    if (head < ra.q_heads + ra.kv_heads) {
+#pragma unroll
+                        for (int pr = 0; pr < 2; ++pr) {
+                            const float angle = (float)rp_pos * ra.inv_freq[dd / 2 + pr];
+                            const float c = cosf(angle), sn = sinf(angle);
+                            const float y1 = val[2 * pr] * c - val[2 * pr + 1] * sn;
+                            const float y2 = val[2 * pr + 1] * c + val[2 * pr] * sn;
+                            val[2 * pr] = y1;
+                            val[2 * pr + 1] = y2;
+                        }
+                    }
+                    union { uint2 u; uint16_t e[4]; } pk;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(val[v]).bits;
+                    if (head < ra.q_heads || !ra.k_plane) {
+                        *(uint2*)((bf16_t*)out + (size_t)m * ldo + n) = pk.u;
+                    } else {
+                        const int kvh = (head - ra.q_heads) % ra.kv_heads, off = rp_pos % ra.page;
+                        const size_t base = ((size_t)rp_page * ra.kv_heads + kvh) * ra.page * ra.head_dim;
+                        if (head < ra.q_heads + ra.kv_heads) {
+                            *(uint2*)(ra.k_plane + base + (size_t)off * ra.head_dim + dd) = pk.u;
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 4; ++v) ra.v_plane[base + (size_t)(dd + v) * ra.page + off].bits = pk.e[v];
+                        }
+                    }
+                    continue;
+                }
+                if (m < M) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        if (n + v < N) {
+                            float val = sum[v];
+                            if (bias) val += load_vec(bias, bias_f32, n + v);
+                            out[(size_t)m * ldo + n + v] = from_float<TOut>(val);
+                        }
+                    }
+                }
+            }
+        }
+        if (next >= strips) break;
+        strip = next;
+        if (KS > 1) lds_barrier();             // the sums are read until here; the next strip's overwrite them
     }
 #undef SK_ISSUE
-    Frag16 a0[R], a1[R], b0[MT], b1[MT];
-    // the tail step (K % 64 != 0) belongs to the wave whose turn it is; pieces beyond K count as zero
-    if ((K & 63) && (full % KS) == wave) {
-        const int k = 64 * full + SK_KOFF(lg);
-        const bool v0 = k + 8 <= K, v1 = k + SK_SECOND + 8 <= K;
-        const uint4 zero = make_uint4(0, 0, 0, 0);
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            a0[r].u = v0 ? *(const uint4*)(wrow[r] + k) : zero;
-            a1[r].u = v1 ? *(const uint4*)(wrow[r] + k + SK_SECOND) : zero;
-        }
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            b0[t].u = v0 ? SK_LOADB(t, k) : zero;
-            b1[t].u = v1 ? SK_LOADB(t, k + SK_SECOND) : zero;
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[r].v, b0[t].v, acc[r][t], 0, 0, 0);
-                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[r].v, b1[t].v, acc[r][t], 0, 0, 0);
-            }
-    }
-
-    // D[i][j]: lane holds i = 4 * (lane / 16) + v (weight row), j = lane % 16 (activation row)
-    if (KS > 1) {
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                float* dst = red + ((size_t)(wave * R * MT + r * MT + t) * 64 + lane) * 4;
-                *(f32x4_t*)dst = acc[r][t];
-            }
-        __syncthreads();
-    }
-    if (SW) {
-        for (int pt = wave; pt < 2 * MT; pt += KS) {
-            const int pr = pt / MT, t = pt % MT;
-            f32x4_t gs = f32x4_t{0.f, 0.f, 0.f, 0.f}, us = gs;
-#pragma unroll
-            for (int wv = 0; wv < KS; ++wv) {
-                gs += *(const f32x4_t*)(red + ((size_t)(wv * R * MT + pr * MT + t) * 64 + lane) * 4);
-                us += *(const f32x4_t*)(red + ((size_t)(wv * R * MT + (pr + 2) * MT + t) * 64 + lane) * 4);
-            }
-            const int m = t * 16 + li;
-            const int col = (n0 / 64) * 32 + pr * 16 + 4 * lg;
-            if (m < M) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    if (col + v < out_cols) out[(size_t)m * ldo + col + v] = from_float<TOut>(silu_mul(gs[v], us[v]));
-            }
-        }
-        return;
-    }
-    for (int tile = wave; tile < R * MT; tile += KS) {
-        const int r = tile / MT, t = tile % MT;
-        f32x4_t sum;
-        if (KS > 1) {
-            sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int wv = 0; wv < KS; ++wv) sum += *(const f32x4_t*)(red + ((size_t)(wv * R * MT + tile) * 64 + lane) * 4);
-        } else {
-            sum = acc[0][0];
-#pragma unroll
-            for (int rr = 0; rr < R; ++rr)
-#pragma unroll
-                for (int tt = 0; tt < MT; ++tt)
-                    if (rr == r && tt == t) sum = acc[rr][tt];
-        }
-        const int m = t * 16 + li;
-        const int n = n0 + r * 16 + 4 * lg;
-        if (RP) {
-            if (m >= M || n >= N) continue;                    // N is a multiple of 16 here
-            float val[4];
-#pragma unroll
-            for (int v = 0; v < 4; ++v) val[v] = sum[v] + (bias ? load_vec(bias, bias_f32, n + v) : 0.f);
-            const int head = n / ra.head_dim, dd = n - head * ra.head_dim;
-            if (head < ra.q_heads + ra.kv_heads) {
-#pragma unroll
-                for (int pr = 0; pr < 2; ++pr) {
-                    const float angle = (float)rp_pos * ra.inv_freq[dd / 2 + pr];
-                    const float c = cosf(angle), sn = sinf(angle);
-                    const float y1 = val[2 * pr] * c - val[2 * pr + 1] * sn;
-                    const float y2 = val[2 * pr + 1] * c + val[2 * pr] * sn;
-                    val[2 * pr] = y1;
-                    val[2 * pr + 1] = y2;
-                }
-            }
-            union { uint2 u; uint16_t e[4]; } pk;
-#pragma unroll
-            for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(val[v]).bits;
-            if (head < ra.q_heads || !ra.k_plane) {
-                *(uint2*)((bf16_t*)out + (size_t)m * ldo + n) = pk.u;
-            } else {
-                const int kvh = (head - ra.q_heads) % ra.kv_heads, off = rp_pos % ra.page;
-                const size_t base = ((size_t)rp_page * ra.kv_heads + kvh) * ra.page * ra.head_dim;
-                if (head < ra.q_heads + ra.kv_heads) {
-                    *(uint2*)(ra.k_plane + base + (size_t)off * ra.head_dim + dd) = pk.u;
-                } else {
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) ra.v_plane[base + (size_t)(dd + v) * ra.page + off].bits = pk.e[v];
-                }
-            }
-            continue;
-        }
-        if (m < M) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                if (n + v < N) {
-                    float val = sum[v];
-                    if (bias) val += load_vec(bias, bias_f32, n + v);
-                    out[(size_t)m * ldo + n + v] = from_float<TOut>(val);
-                }
-            }
-        }
-    }
 }
 
 // Shared memory beyond 64 KB has to be allowed per kernel, once per process.
@@ -467,16 +494,20 @@ static hipError_t allow_lds(Kernel kernel, size_t bytes) {
 template <int R, int MT, int KS, typename TOut, bool SW, int D>
 static void launch_skinny_d(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                             int ldx, int ldo, int out_cols, hipStream_t stream) {
-    dim3 grid((N + 16 * R - 1) / (16 * R)), block(KS * 64);
+    const int strips = SW ? N / 32 : (N + 16 * R - 1) / (16 * R);
+    dim3 grid(strips), block(KS * 64);
     const size_t red_bytes = (size_t)KS * R * MT * 1024;
     const size_t x_bytes = (size_t)M * (K + 8) * 2;
-    // (not with few waves per work-group: the copy of x then takes longer than it saves; measured on the
-    // fused gate/up kernel, 87 us with against 64 us without at M = 8)
-    if (M > 1 && KS >= 8 && x_bytes <= SKINNY_XL_MAX_BYTES) {
+    // More than one row of x: two work-groups per compute unit copy x into shared memory once and walk
+    // the strips between them (each strip's own copy took longer than it saved: 87 against 64 us on the
+    // fused gate/up product at M = 8 with four waves).
+    if (M > 1 && red_bytes + x_bytes <= 156 * 1024) {
         auto kernel = gemm_skinny_kernel<R, MT, KS, TOut, SW, true, D>;
-        static hipError_t allowed = allow_lds(kernel, 96 * 1024);
+        static hipError_t allowed = allow_lds(kernel, 156 * 1024);
         if (allowed == hipSuccess) {
-            kernel<<<grid, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{});
+            const int most = x_bytes <= SKINNY_XL_MAX_BYTES ? 512 : 256;      // a larger x leaves room for one work-group only
+            dim3 few(strips < most ? strips : most);
+            kernel<<<few, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{});
             return;
         }
     }
@@ -1227,8 +1258,8 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
     const bf16_t* wb = (const bf16_t*)w;
     bf16_t* ob = (bf16_t*)out;
     if (M <= 16 || (M <= 32 && K % 64 != 0)) {
-        if (M <= 16) launch_skinny_t<4, 1, 4, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
-        else launch_skinny_t<4, 2, 4, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
+        if (M <= 16) launch_skinny_t<1, 1, 16, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
+        else launch_skinny_t<1, 2, 16, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
     } else if (K % 64 == 0) {
         const int rc = launch_dl_tile<bf16_t, true>(pick_dl_tile(M, N, K, true), xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
         if (rc != TL_OK) return rc;

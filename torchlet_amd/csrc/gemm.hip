@@ -215,8 +215,11 @@ constexpr int skinny_depth() {
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + expf(-g)) * u; }
 
 // SW (gate/up product with the SwiGLU gate applied to the accumulators): w holds blocks of 64
-// rows, 32 gate rows followed by the 32 up rows of the same columns; needs R == 4, so that a
-// work-group's strips are [gate 0-15, gate 16-31, up 0-15, up 16-31]; out has N / 2 columns.
+// rows, 32 gate rows followed by the 32 up rows of the same columns; a work-group's strip is 16
+// outputs, whose gate rows half of its waves walk and whose up rows the other half (R == 1: each
+// wave streams one strip of 16 rows, which is what reaches the memory's rate; four strips per
+// wave, as an earlier version had, stayed at 56-58 us on the 7B's matrix where this takes 50-53);
+// out has N / 2 columns.
 // XL (x through shared memory): with more than one activation row the 16 lanes of a group read
 // 16 different rows of x, which no longer fit the L1 cache once M * K * 2 bytes exceed it, and
 // every operand load of x becomes a trip to L2 that competes with the weight stream (measured:

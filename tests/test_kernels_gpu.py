@@ -210,7 +210,7 @@ def test_linear_many_rows_on_matrix_cores(ops, out_dtype, tile, M, N, K):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("tile", [(64, 64), (64, 256), (128, 128), (128, 256), (256, 128), (192, 256), (256, 192), (256, 256)])
+@pytest.mark.parametrize("tile", [(64, 64), (64, 128), (64, 256), (128, 128), (128, 256), (256, 128), (192, 256), (256, 192), (256, 256)])
 @pytest.mark.parametrize("M,N,K", [(65, 129, 64), (300, 520, 192), (1000, 257, 1024), (33, 48, 3584), (40, 4608, 128), (513, 700, 320)])
 def test_linear_many_rows_fetched_straight_into_shared_memory(ops, out_dtype, tile, M, N, K):
     """Every tile shape of the direct-load matrix-core kernel, with tails in M and N, one slab to

@@ -1007,21 +1007,24 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
 // the other; a tile takes a fixed time (filling the pipeline, storing the result) plus its
 // products at the rate one compute unit reaches with that shape (fitted to measurements at
 // 2048 rows against the Qwen2.5-7B and 14B matrices, K from 3584 to 18944).
-enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_TILES };
-static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 192, 256, 256};
-static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256};
-static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12};   // FLOP/s of one compute unit
-static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6};         // seconds per tile
+enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_64x128, DL_TILES };
+static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 192, 256, 256, 64};
+static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256, 128};
+static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12, 2.1e12};   // FLOP/s of one compute unit
+static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6, 5e-6};       // seconds per tile
 
 // Seconds for `groups` work-groups of tile t over k columns each.  The two smallest tiles run two
 // to a compute unit: each then works at half the unit's rate, and one that has a unit to itself
-// (not more work-groups than units) at about 0.62 of it.
+// (not more work-groups than units) at about 0.62 of it.  With few rows the products wait for the
+// weights: a work-group draws its BN rows of them at about 32 GB/s (measured at 17-64 rows: 108
+// work-groups of 64 x 256 on the 14B's gate/up matrix take 81 us, 216 of 64 x 128 take 56).
 static double dl_estimate(DlTile t, long groups, int k) {
     const bool pairs = t == DL_64x64 || t == DL_128x128;
     const double products = 2.0 * DL_BM[t] * DL_BN[t] * k;
-    if (!pairs) return (double)((groups + 255) / 256) * (products / DL_RATE[t] + DL_FIXED[t]);
+    const double stream = 2.0 * DL_BN[t] * k / 32e9;
+    if (!pairs) return (double)((groups + 255) / 256) * fmax(products / DL_RATE[t] + DL_FIXED[t], stream);
     const double rate = groups > 256 ? DL_RATE[t] / 2 : DL_RATE[t] * 0.62;
-    return (double)((groups + 511) / 512) * (products / rate + DL_FIXED[t]);
+    return (double)((groups + 511) / 512) * fmax(products / rate + DL_FIXED[t], groups > 256 ? 2 * stream : stream);
 }
 
 static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = nullptr) {
@@ -1089,6 +1092,7 @@ static int launch_dl_tile(DlTile tile, const void* x, const void* w, const void*
     case DL_128x128: return launch_dl_tile_t<128, 128, 2, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_128x256: return launch_dl_tile_t<128, 256, 2, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_256x128: return launch_dl_tile_t<256, 128, 4, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+    case DL_64x128: return launch_dl_tile_t<64, 128, 1, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_192x256: return launch_dl_tile_t<192, 256, 2, 4, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_256x192:
         if constexpr (!SW) return launch_dl_tile_t<256, 192, 4, 2, 2, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);

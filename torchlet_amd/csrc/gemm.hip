@@ -1264,7 +1264,10 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
     bf16_t* ob = (bf16_t*)out;
-    if (M <= 16 || (M <= 32 && K % 64 != 0)) {
+    // the few-rows kernel where its copy of x fits shared memory (else every wave fetches x as often
+    // as its weights: 32B sizes, 16 rows, 20.2 against 18.9 ms a step)
+    const bool x_fits = M == 1 || (size_t)16 * 1024 + (size_t)M * (K + 8) * 2 <= 156 * 1024;
+    if ((M <= 16 && (x_fits || K % 64 != 0)) || (M <= 32 && K % 64 != 0)) {
         if (M <= 16) launch_skinny_t<1, 1, 16, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
         else launch_skinny_t<1, 2, 16, bf16_t, true>(xb, wb, nullptr, 0, ob, M, N, K, ldx, ldo, I, stream);
     } else if (K % 64 == 0) {

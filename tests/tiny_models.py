@@ -1,10 +1,12 @@
 """Tiny random-weight model folders for the tests.
 
-Four configurations of the one architecture that differ in every size and option:
+Five configurations of the one architecture that differ in every size and option:
 A and B are the two tiny workloads the benchmark contract names; C adds what they leave
 out (no QKV bias, one KV head per query head, a window on the later layers); D has heads of
 64 (the size from which the 128-row prompt attention kernel is built), groups of three, a
-window wider than a step of keys and pages of 8.
+window wider than a step of keys and pages of 8; E has a width, a feed-forward width and a
+vocabulary that are no multiples of 8 (the matrix-core kernels refuse them: the bfloat16 engine
+runs its general kernels), seven heads of 16 and pages of 4.
 """
 import json
 from pathlib import Path
@@ -35,9 +37,14 @@ CONFIGS = {
         max_position_embeddings=400, rope_theta=30000.0, rms_norm_eps=2e-6, tie_word_embeddings=True,
         use_sliding_window=True, sliding_window=70, max_window_layers=1,
     ),
+    "E": dict(
+        architectures=["Qwen2ForCausalLM"], vocab_size=131, hidden_size=100, num_hidden_layers=2,
+        num_attention_heads=7, num_key_value_heads=7, head_dim=16, intermediate_size=75,
+        max_position_embeddings=300, rope_theta=20000.0, rms_norm_eps=5e-6, tie_word_embeddings=False,
+    ),
 }
-SEEDS = {"A": 0, "B": 1, "C": 5, "D": 8}
-PAGE_SIZES = {"A": 16, "B": 8, "C": 16, "D": 8}
+SEEDS = {"A": 0, "B": 1, "C": 5, "D": 8, "E": 9}
+PAGE_SIZES = {"A": 16, "B": 8, "C": 16, "D": 8, "E": 4}
 
 
 def write(name: str, root: Path, dtype=torch.bfloat16) -> Path:

@@ -630,17 +630,35 @@ def test_paged_attention_prompt_tiles_of_128_rows(ops, nh, nkv, hd, page, window
     out = torch.full((T, nh * hd), float("nan"), dtype=dtype, device="cuda")
     wide = torch.zeros(T, nh * hd + 32, dtype=dtype, device="cuda")
     wide[:, : nh * hd] = q.cuda()
-    ops.paged_attention_prompt(wide[:, : nh * hd], out, kp.cuda(), vp.cuda(), bt.cuda(), indptr.cuda(),
-                               torch.tensor(ctxs, dtype=torch.int32).cuda(), torch.tensor(tile_req, dtype=torch.int32).cuda(),
-                               torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq, nh, nkv, hd, page, window,
-                               1.0 / math.sqrt(hd))
-    got = out.cpu().double().view(T, nh, hd)
-    for r in range(R):
-        a, b = int(indptr[r]), int(indptr[r + 1])
-        ref = _attention_ref(q[a:b].double().view(-1, nh, hd), ks[r].double(), vs[r].double(), window)
-        tol = _tol(dtype)
-        tol = dict(rtol=tol["rtol"], atol=tol["atol"] + 2 ** -9 * float(vs[r].abs().max()))
-        torch.testing.assert_close(got[a:b], ref, **tol)
+    args = (kp.cuda(), vp.cuda(), bt.cuda(), indptr.cuda(),
+            torch.tensor(ctxs, dtype=torch.int32).cuda(), torch.tensor(tile_req, dtype=torch.int32).cuda(),
+            torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq, nh, nkv, hd, page, window,
+            1.0 / math.sqrt(hd))
+    ops.paged_attention_prompt(wide[:, : nh * hd], out, *args)
+    # the same with every tile's keys dealt to two, three and five work-groups (some shares are empty:
+    # the single token has 100 keys, four steps of 32) and merged for all tokens but those of request 2
+    listed = [t for r in range(R) if r != 2 for t in range(int(indptr[r]), int(indptr[r + 1]))]
+    keep = [i for i, r in enumerate(tile_req) if r != 2]
+    some = (args[0], args[1], args[2], args[3], args[4], torch.tensor([tile_req[i] for i in keep], dtype=torch.int32).cuda(),
+            torch.tensor([tile_tok0[i] for i in keep], dtype=torch.int32).cuda(), len(keep)) + args[8:]
+    outs = [out]
+    for splits in (2, 3, 5):
+        o = torch.full((T, nh * hd), 9.0, dtype=dtype, device="cuda")
+        ops.paged_attention_prompt(wide[:, : nh * hd], o, *some, splits=splits,
+                                   merge_tokens=(torch.tensor(listed, dtype=torch.int32).cuda(), len(listed)))
+        a2, b2 = int(indptr[2]), int(indptr[3])
+        assert bool((o[a2:b2] == 9.0).all()), "rows of a request outside the list were written"
+        outs.append(o)
+    for k, o in enumerate(outs):
+        got = o.cpu().double().view(T, nh, hd)
+        for r in range(R):
+            if k and r == 2:
+                continue
+            a, b = int(indptr[r]), int(indptr[r + 1])
+            ref = _attention_ref(q[a:b].double().view(-1, nh, hd), ks[r].double(), vs[r].double(), window)
+            tol = _tol(dtype)
+            tol = dict(rtol=tol["rtol"], atol=tol["atol"] + 2 ** -9 * float(vs[r].abs().max()))
+            torch.testing.assert_close(got[a:b], ref, **tol)
 
 
 def test_paged_attention_prompt_takes_a_wide_block_table_for_short_sequences(ops):

@@ -847,7 +847,14 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
 
     const int key_hi = ctx + tok0 + ntok;
     const int key_lo = a.window > 0 ? max(0, ctx + tok0 - a.window + 1) : 0;
-    const int st_first = key_lo / ATQ_KEYS, st_last = (key_hi + ATQ_KEYS - 1) / ATQ_KEYS;
+    // the tile's steps of ATQ_KEYS keys; with a.splits > 1 work-group blockIdx.z takes its share of them
+    // and leaves unnormalised sums, maxima and denominators for attention_merge_kernel
+    int st_first = key_lo / ATQ_KEYS, st_last = (key_hi + ATQ_KEYS - 1) / ATQ_KEYS;
+    if (a.splits > 1) {
+        const int per = (st_last - st_first + a.splits - 1) / a.splits;
+        st_first = min(st_first + (int)blockIdx.z * per, st_last);
+        st_last = min(st_first + per, st_last);
+    }
 
     const bf16_t* kp = (const bf16_t*)a.k_plane;
     const bf16_t* vp = (const bf16_t*)a.v_plane;
@@ -863,6 +870,7 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     if (blk_n > ATM_BT_MAX) return;            // longer than the host promised: leave the rows unwritten rather than overrun
     for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
     __syncthreads();
+    const bool any_step = st_first < st_last;  // (a share of the steps can be empty)
 
     // requests of one step: K rows of AT_HD * 2 bytes, then V^T rows of ATQ_VROW bytes
     constexpr int KPI = 1024 / (AT_HD * 2);                 // keys per load instruction (4 or 8)
@@ -914,10 +922,12 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
 
     // Steps st .. st + ATQ_STAGES - 2 are requested ahead; past the end the last step is requested
     // again (nobody reads it), so that the number of requests in flight is the same at every wait.
+    if (any_step) {
 #pragma unroll
-    for (int i = 0; i < ATQ_STAGES - 1; ++i) request_step(min(st_first + i, st_last - 1), i);
-    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * K_INSTR * (ATQ_STAGES - 2)) : "memory");
-    __syncthreads();
+        for (int i = 0; i < ATQ_STAGES - 1; ++i) request_step(min(st_first + i, st_last - 1), i);
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * K_INSTR * (ATQ_STAGES - 2)) : "memory");
+        __syncthreads();
+    }
     for (int st = st_first; st < st_last; ++st) {
         const int buf = (st - st_first) % ATQ_STAGES;
         request_step(min(st + ATQ_STAGES - 1, st_last - 1), (st - st_first + ATQ_STAGES - 1) % ATQ_STAGES);
@@ -1019,6 +1029,24 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     l += __shfl_xor(l, 32, TL_WAVE);
     if (!row_ok) return;
     // lane holds d = 32 b + 8 q + 4 h + v of its row
+    if (a.splits > 1) {
+        const size_t pr = ((size_t)r_token * a.heads + r_head) * a.splits + blockIdx.z;
+        float* po = a.part_o + pr * AT_HD;
+#pragma unroll
+        for (int b = 0; b < AT_HD / 32; ++b)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                f32x4_t f;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) f[v] = acc[b][4 * q + v];
+                *(f32x4_t*)(po + 32 * b + 8 * q + 4 * h) = f;
+            }
+        if (h == 0) {
+            a.part_ml[pr * 2] = m * 0.69314718055994531f;      // back to natural logarithms for the merge
+            a.part_ml[pr * 2 + 1] = l;
+        }
+        return;
+    }
     bf16_t* o = (bf16_t*)a.out + (size_t)r_token * a.heads * AT_HD + (size_t)r_head * AT_HD;
     const float inv = 1.f / l;
 #pragma unroll
@@ -1050,7 +1078,11 @@ extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out,
                                          const void* block_table, int bt_stride, const void* req_indptr, const void* ctx_lens,
                                          const void* tile_req, const void* tile_tok0, int tiles, int tq,
                                          int heads, int kv_heads, int page, int window, float scale, int used_blocks,
+                                         int splits, void* part_o, void* part_ml, const void* merge_tokens, int merge_count,
                                          hipStream_t stream) {
+    // splits > 1: every tile's keys are dealt to that many work-groups, whose parts (scratch as for
+    // tl_paged_attention) are merged for the `merge_count` tokens listed in `merge_tokens`: for prompt
+    // portions whose tiles alone leave most compute units idle.
 #if AT_HD == 64 || AT_HD == 128
     TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
     TL_REQUIRE(page >= 8 && (page & (page - 1)) == 0 && tq > 0 && window >= 0, "attention_prompt: pages of 8, 16, 32, ... tokens, not %d", page);
@@ -1067,16 +1099,23 @@ extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out,
     a.q = q; a.out = out; a.k_plane = k_plane; a.v_plane = v_plane;
     a.block_table = (const int*)block_table; a.req_indptr = (const int*)req_indptr; a.ctx_lens = (const int*)ctx_lens;
     a.tile_req = (const int*)tile_req; a.tile_tok0 = (const int*)tile_tok0;
-    a.part_o = nullptr; a.part_ml = nullptr;
+    TL_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || (part_o && part_ml && merge_tokens && merge_count > 0)),
+               "attention_prompt: splits > 1 need scratch and the tokens to merge");
+    a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
     a.q_stride = q_stride; a.bt_stride = bt_stride; a.heads = heads; a.kv_heads = kv_heads; a.page = page;
-    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = 1; a.scale = scale;
+    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = splits; a.scale = scale;
     a.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz(page) : -1;
     const int chunks = (group + gcap - 1) / gcap;
     static hipError_t allowed = hipFuncSetAttribute((const void*)paged_attention_prompt_kernel,
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, ATQ_SMEM);
     TL_REQUIRE(allowed == hipSuccess, "attention_prompt: cannot get %d bytes of shared memory", ATQ_SMEM);
-    paged_attention_prompt_kernel<<<dim3(tiles, kv_heads * chunks), dim3(256), ATQ_SMEM, stream>>>(a);
+    paged_attention_prompt_kernel<<<dim3(tiles, kv_heads * chunks, splits), dim3(256), ATQ_SMEM, stream>>>(a);
     TL_CHECK_LAUNCH("paged_attention_prompt");
+    if (splits > 1) {
+        attention_merge_kernel<bf16_t><<<dim3((unsigned)merge_count * heads), dim3(AT_HD), 0, stream>>>(
+            (const float*)part_o, (const float*)part_ml, (bf16_t*)out, splits, (const int*)merge_tokens, heads);
+        TL_CHECK_LAUNCH("attention_merge");
+    }
     return TL_OK;
 #else
     TL_REQUIRE(false, "attention_prompt: built for head sizes 64 and 128, this library is for %d", AT_HD);

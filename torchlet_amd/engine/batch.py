@@ -117,8 +117,10 @@ class StepContext:
     def tiles_by_length(self, tq_short: int, tq_long: int, threshold: int):
         """Two tile lists: requests that bring fewer than ``threshold`` tokens in tiles of
         ``tq_short`` tokens, the others in tiles of ``tq_long``.  The first list comes with the
-        indices of its requests' tokens and the largest sequence length among them:
-        ``((tile_req, tile_tok0, tiles, tokens, number of tokens, longest), (tile_req, tile_tok0, tiles))``."""
+        indices of its requests' tokens and the largest sequence length among them, the second
+        with its requests' tokens and the smallest sequence length among them:
+        ``((tile_req, tile_tok0, tiles, tokens, number of tokens, longest),
+        (tile_req, tile_tok0, tiles, tokens, number of tokens, shortest))``."""
         key = (tq_short, tq_long, threshold)
         t = self._tiles.get(key)
         if t is None:
@@ -129,10 +131,14 @@ class StepContext:
             np.cumsum(self._host_new_lens, out=starts[1:])
             short_tokens = np.concatenate([np.arange(starts[r], starts[r + 1]) for r in np.nonzero(~long)[0]] or
                                           [np.zeros(0, dtype=np.int64)]).astype(np.int32)
-            longest = int((self._host_new_lens + self._host_ctx_lens)[~long].max()) if (~long).any() else 0
-            v = self._upload({"sr": sr, "s0": s0, "lr": lr, "l0": l0, "st": short_tokens})
+            long_tokens = np.concatenate([np.arange(starts[r], starts[r + 1]) for r in np.nonzero(long)[0]] or
+                                         [np.zeros(0, dtype=np.int64)]).astype(np.int32)
+            totals = self._host_new_lens + self._host_ctx_lens
+            longest = int(totals[~long].max()) if (~long).any() else 0
+            shortest = int(totals[long].min()) if long.any() else 0
+            v = self._upload({"sr": sr, "s0": s0, "lr": lr, "l0": l0, "st": short_tokens, "lt": long_tokens})
             t = self._tiles[key] = ((v["sr"], v["s0"], len(sr), v["st"], len(short_tokens), longest),
-                                    (v["lr"], v["l0"], len(lr)))
+                                    (v["lr"], v["l0"], len(lr), v["lt"], len(long_tokens), shortest))
         return t
 
 

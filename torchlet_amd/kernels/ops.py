@@ -465,12 +465,16 @@ def paged_attention_prompt(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Te
                            block_table: torch.Tensor, req_indptr: torch.Tensor, ctx_lens: torch.Tensor,
                            tile_req: torch.Tensor, tile_tok0: torch.Tensor, num_tiles: int, tile_tokens: int,
                            num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
-                           scale: float, max_total_len: int | None = None) -> None:
+                           scale: float, max_total_len: int | None = None, splits: int = 1,
+                           merge_tokens: tuple[torch.Tensor, int] | None = None) -> None:
     """The attention of :func:`paged_attention` for prompt portions in tiles of 128 rows
     (``tile_tokens`` tokens times the heads of a group): bfloat16, head size 64 or 128, pages
     of a multiple of 8 tokens; keys and values go straight into shared memory once per
     work-group.  Writes the rows of its tiles only.  ``max_total_len``: the longest sequence of the
-    step (cached + new tokens; default: what the block table could hold)."""
+    step (cached + new tokens; default: what the block table could hold).  ``splits`` > 1 deals
+    every tile's keys to that many work-groups (for few tiles against long sequences) and merges
+    their parts for the tokens listed in ``merge_tokens`` (int32 indices, how many): the tokens
+    of the tiles' requests."""
     T = q.shape[0]
     used_blocks = block_table.shape[1] if max_total_len is None else min(block_table.shape[1], -(-max_total_len // page_size))
     if not prompt_attention_fits(q.dtype, head_dim, page_size, used_blocks):
@@ -485,11 +489,23 @@ def paged_attention_prompt(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Te
     if tile_req.numel() < num_tiles or tile_tok0.numel() < num_tiles:
         raise KernelError("paged_attention_prompt: tile arrays shorter than the number of tiles")
     lib = _lib(f"attention_hd{head_dim}")
+    part_o = part_ml = tokens = None
+    count = 0
+    if splits > 1:
+        if merge_tokens is None or merge_tokens[1] <= 0:
+            raise KernelError("paged_attention_prompt: splits > 1 need the tokens whose parts are merged")
+        tokens, count = merge_tokens
+        _i32(tokens, "merge_tokens")
+        if tokens.numel() < count:
+            raise KernelError("paged_attention_prompt: merge_tokens shorter than its count")
+        part_o = torch.empty((T * num_heads * splits, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T * num_heads * splits, 2), dtype=torch.float32, device=q.device)
     _check(lib, lib.tl_paged_attention_prompt(_ptr(q), c_int(q.stride(0)), _ptr(out), _ptr(k_plane), _ptr(v_plane),
                                               _ptr(block_table), c_int(block_table.stride(0)), _ptr(req_indptr),
                                               _ptr(ctx_lens), _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles),
                                               c_int(tile_tokens), c_int(num_heads), c_int(num_kv_heads), c_int(page_size),
-                                              c_int(window), c_float(scale), c_int(max(1, used_blocks)), _stream()))
+                                              c_int(window), c_float(scale), c_int(max(1, used_blocks)),
+                                              c_int(splits), _ptr(part_o), _ptr(part_ml), _ptr(tokens), c_int(count), _stream()))
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:

@@ -26,6 +26,9 @@ _PORTION_MIN_TOKENS = 16     # requests that bring at least this many tokens go 
                              # tokens; measured on MI355X at 28/4 heads of 128: 2048 new tokens 222 -> 110 us,
                              # 8192 new tokens 2.9 -> 0.84 ms), else the 64-row one ...
 _PORTION_MIN_CONTEXT = 4096  # ... which pays only in steps whose longest sequence has at least this many tokens
+_PROMPT_TARGET_WORKGROUPS = 512   # the 128-row kernel: two work-groups fit a compute unit
+_PROMPT_MIN_KEYS_PER_SPLIT = 512
+_PROMPT_MAX_SPLITS = 4
 
 
 @MIXERS.register("gqa_attention")
@@ -153,7 +156,14 @@ class GQAttention(Mixer):
             tq = self.prompt_tile_tokens if rows128 else self.portion_tile_tokens
             kernel = ops.paged_attention_prompt if rows128 else ops.paged_attention_prefill
             short, long = ctx.tiles_by_length(self.tile_tokens, tq, _PORTION_MIN_TOKENS)
-            extra = dict(max_total_len=ctx.max_total_len) if rows128 else {}
+            extra = {}
+            if rows128:
+                # few tiles against long sequences (a portion of a few hundred tokens deep into a prompt):
+                # each tile's keys are dealt to several work-groups, so that the compute units have work
+                groups = long[2] * self.kv_heads * -(-(self.heads // self.kv_heads) // ops.PROMPT_ATTENTION_ROWS)
+                keys = ctx.max_total_len if self.window is None else min(ctx.max_total_len, self.window + tq)
+                splits = max(1, min(_PROMPT_MAX_SPLITS, _PROMPT_TARGET_WORKGROUPS // max(groups, 1), keys // _PROMPT_MIN_KEYS_PER_SPLIT))
+                extra = dict(max_total_len=ctx.max_total_len, splits=splits, merge_tokens=(long[3], long[4]))
             kernel(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens, long[0], long[1], long[2], tq, *common, **extra)
             if short[2]:     # split over their keys; the merge of the parts is kept to the rows of these requests
                 ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,

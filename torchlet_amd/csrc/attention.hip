@@ -716,24 +716,32 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(AttnArgs a
 #endif
 
 // out[row] = sum_s exp(m_s - M) acc_s / sum_s exp(m_s - M) l_s over the parts of a row.
-// The parts are read eight at a time with all loads issued before the first use.
+// A thread owns four neighbouring elements of a row, a work-group of 256 threads as many rows as
+// fit; the parts are read eight at a time with all loads issued before the first use.
 // Rows are (token, head) pairs: all of them, or those of the tokens listed in `tokens`.
+#define ATG_TPR (AT_HD / 4)            // threads per row
+#define ATG_RPW (256 / ATG_TPR)        // rows per work-group
 template <typename T>
-__global__ void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                       T* __restrict__ out, int splits, const int* __restrict__ tokens, int heads) {
-    const size_t r = tokens ? (size_t)tokens[blockIdx.x / heads] * heads + blockIdx.x % heads : blockIdx.x;
+__global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                              T* __restrict__ out, int splits, const int* __restrict__ tokens,
+                                                              int heads, int rows) {
+    const int local = threadIdx.x / ATG_TPR;
+    const long listed = (long)blockIdx.x * ATG_RPW + local;
+    if (local >= ATG_RPW || listed >= rows) return;
+    const size_t r = tokens ? (size_t)tokens[listed / heads] * heads + listed % heads : (size_t)listed;
     const float2* ml = (const float2*)(part_ml + r * splits * 2);
     const float* po = part_o + r * splits * AT_HD;
-    const int d = threadIdx.x;                     // blockDim.x == AT_HD
-    float mx = -INFINITY, denom = 0.f, num = 0.f;
+    const int d = 4 * (threadIdx.x % ATG_TPR);
+    float mx = -INFINITY, denom = 0.f;
+    float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s0 = 0; s0 < splits; s0 += 8) {
         float2 w[8];
-        float o[8];
+        float4 o[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int sp = min(s0 + i, splits - 1);
             w[i] = ml[sp];
-            o[i] = po[(size_t)sp * AT_HD + d];
+            o[i] = *(const float4*)(po + (size_t)sp * AT_HD + d);
         }
         float m8 = mx;
 #pragma unroll
@@ -741,17 +749,28 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_o, const f
             if (s0 + i < splits) m8 = fmaxf(m8, w[i].x);
         const float rescale = (mx == -INFINITY) ? 0.f : expf(mx - m8);
         denom *= rescale;
-        num *= rescale;
+        num.x *= rescale; num.y *= rescale; num.z *= rescale; num.w *= rescale;
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             if (s0 + i < splits && w[i].x != -INFINITY) {
                 const float e = expf(w[i].x - m8);
                 denom += e * w[i].y;
-                num += e * o[i];
+                num.x += e * o[i].x; num.y += e * o[i].y; num.z += e * o[i].z; num.w += e * o[i].w;
             }
         mx = m8;
     }
-    out[r * AT_HD + d] = from_float<T>(num / denom);
+    T* dst = out + r * AT_HD + d;
+    dst[0] = from_float<T>(num.x / denom);
+    dst[1] = from_float<T>(num.y / denom);
+    dst[2] = from_float<T>(num.z / denom);
+    dst[3] = from_float<T>(num.w / denom);
+}
+
+static void launch_merge(const void* part_o, const void* part_ml, void* out, int splits, const void* tokens, int heads,
+                         long rows, bool f32, hipStream_t stream) {
+    dim3 grid((unsigned)((rows + ATG_RPW - 1) / ATG_RPW)), block(256);
+    if (f32) attention_merge_kernel<float><<<grid, block, 0, stream>>>((const float*)part_o, (const float*)part_ml, (float*)out, splits, (const int*)tokens, heads, (int)rows);
+    else attention_merge_kernel<bf16_t><<<grid, block, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, splits, (const int*)tokens, heads, (int)rows);
 }
 
 // =====================================================================================
@@ -1112,8 +1131,7 @@ extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out,
     paged_attention_prompt_kernel<<<dim3(tiles, kv_heads * chunks, splits), dim3(256), ATQ_SMEM, stream>>>(a);
     TL_CHECK_LAUNCH("paged_attention_prompt");
     if (splits > 1) {
-        attention_merge_kernel<bf16_t><<<dim3((unsigned)merge_count * heads), dim3(AT_HD), 0, stream>>>(
-            (const float*)part_o, (const float*)part_ml, (bf16_t*)out, splits, (const int*)merge_tokens, heads);
+        launch_merge(part_o, part_ml, out, splits, merge_tokens, heads, (long)merge_count * heads, false, stream);
         TL_CHECK_LAUNCH("attention_merge");
     }
     return TL_OK;
@@ -1161,9 +1179,7 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
         // merge_tokens: the tokens whose rows the tiles cover, when these are not all tokens of the step
         const size_t rows = (size_t)(merge_tokens ? merge_count : tokens) * heads;
         if (rows == 0) return TL_OK;
-        dim3 mgrid((unsigned)rows), mblock(AT_HD);
-        if (dtype == TL_DT_F32) attention_merge_kernel<float><<<mgrid, mblock, 0, stream>>>((const float*)part_o, (const float*)part_ml, (float*)out, splits, (const int*)merge_tokens, heads);
-        else attention_merge_kernel<bf16_t><<<mgrid, mblock, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, splits, (const int*)merge_tokens, heads);
+        launch_merge(part_o, part_ml, out, splits, merge_tokens, heads, (long)rows, dtype == TL_DT_F32, stream);
         TL_CHECK_LAUNCH("attention_merge");
     }
     return TL_OK;

@@ -142,8 +142,10 @@ def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: to
 
 def linear_partials_pay(M: int, N: int, K: int) -> bool:
     """Whether a bfloat16 product whose consumer can add slabs up should come from
-    :func:`linear_partials`: when its 64 x 64 output tiles are too few to fill the GPU and K is a
-    multiple of 64, from 17 rows on, and from 2 rows on against a long K."""
+    :func:`linear_partials` (K a multiple of 64): up to 64 rows when its 64 x 64 output tiles are
+    too few to fill the GPU (from 17 rows on, and from 2 rows on against a long K); with more rows
+    when the library's estimate finds a tile shape with K split 2-8 ways faster than the best
+    whole product, slabs included."""
     return bool(_lib("gemm").tl_gemm_partials_pay(c_int(M), c_int(N), c_int(K)))
 
 
@@ -151,7 +153,7 @@ def linear_partials(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``x @ weight.T`` as float32 slabs ``[P, M, N]`` of partial sums over P ranges of K (bfloat16
     operands, K a multiple of 8; more than 64 rows need a multiple of 64): for a product with too
     few output tiles to fill the GPU, where splitting K over work-groups does.  The slabs are
-    summed by :func:`add_rmsnorm`."""
+    summed by :func:`add_rmsnorm` (or by :func:`rope_cache_write`); P may be 1."""
     M, K = x.shape
     N = weight.shape[0]
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or weight.shape[1] != K or not weight.is_contiguous() or x.stride(1) != 1:

@@ -15,10 +15,10 @@ from ..kernels import ops
 from .base import FEED_FORWARDS, FeedForward, WeightSpec
 
 
-# From 17 rows on the down product returns partial sums over slices of K where that pays (the
-# matrix is narrow, so its output tiles alone are too few to keep the GPU busy; measured at
-# 3584 x 18944 and 64 rows: 31 us in four parts against 90 us whole); the next norm adds the slabs up.
-# Up to 16 rows the plain kernel already streams at its limit and the extra slabs cost more.
+# The down product returns partial sums over slices of K where the kernel library finds that it
+# pays (the matrix is narrow, so its output tiles alone are too few to keep the GPU busy; measured
+# at 3584 x 18944: 64 rows 31 us in four parts against 90 us whole, 512 rows 82 against 147 us);
+# the next norm adds the slabs up.
 
 
 @FEED_FORWARDS.register("swiglu")

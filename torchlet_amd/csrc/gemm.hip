@@ -1,39 +1,42 @@
 // Matrix products out[M, N] = x[M, K] * w[N, K]^T (+ bias[N]).
 //
 // Both operands are row-major with K contiguous, which is how activations and
-// nn.Linear-layout weights are stored.  This file holds the general kernel: a 64x64
-// tile, 256 threads with a 4x4 micro-tile each, products and sums in true 32-bit
+// nn.Linear-layout weights are stored.  This file holds the general kernel: a 64x64 or 128x128
+// tile, 256 threads with a 4x4 or 8x8 micro-tile each, products and sums in true 32-bit
 // (v_fma_f32; no matrix-core instruction of reduced precision).  It is the matrix
 // product of the 32-bit path and the fallback of the bfloat16 path for shapes that
 // the matrix-core kernels refuse.  The sum over K runs in one fixed order for every
 // output element, whatever M is, so a row's result does not depend on the batch.
 #include "common.h"
 
-#define GT_M 64
-#define GT_N 64
 #define GT_K 16
 
-template <typename TIn, typename TOut>
+// BT x BT tile, 256 threads with a (BT / 16) x (BT / 16) micro-tile each: 64 x 64 for small products,
+// 128 x 128 (64 products per thread and K step against four 16-byte reads of shared memory) for
+// large ones.  Both add the products of an output element in the same order, k = 0, 1, 2, ...
+template <typename TIn, typename TOut, int BT>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(const TIn* __restrict__ x, const TIn* __restrict__ w,
                                                         const void* __restrict__ bias, int bias_f32,
                                                         TOut* __restrict__ out, int M, int N, int K,
                                                         int ldx, int ldo) {
-    __shared__ float xs[GT_K][GT_M + 4];
-    __shared__ float ws[GT_K][GT_N + 4];
-    const int m0 = blockIdx.y * GT_M, n0 = blockIdx.x * GT_N;
+    constexpr int MT = BT / 16;                     // micro-tile edge
+    constexpr int PER = BT * GT_K / 256;            // elements of each operand a thread loads per K step
+    __shared__ float xs[GT_K][BT + 4];
+    __shared__ float ws[GT_K][BT + 4];
+    const int m0 = blockIdx.y * BT, n0 = blockIdx.x * BT;
     const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
-    // loaders: 64 rows x 16 k per operand = 1024 elements, 4 per thread
-    const int lrow = threadIdx.x / 4;         // 0..63
-    const int lk = (threadIdx.x % 4) * 4;     // 0,4,8,12
-    float acc[4][4];
+    // loaders: BT rows x 16 k per operand, PER consecutive k per thread
+    const int lrow = threadIdx.x / (GT_K / PER);
+    const int lk = (threadIdx.x % (GT_K / PER)) * PER;
+    float acc[MT][MT];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+        for (int j = 0; j < MT; ++j) acc[i][j] = 0.f;
 
     for (int k0 = 0; k0 < K; k0 += GT_K) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < PER; ++i) {
             const int k = k0 + lk + i;
             const int m = m0 + lrow, n = n0 + lrow;
             xs[lk + i][lrow] = (m < M && k < K) ? to_float(x[(size_t)m * ldx + k]) : 0.f;
@@ -42,30 +45,42 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const TIn* __restrict__ 
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < GT_K; ++k) {
-            float a[4], b[4];
+            float a[MT], b[MT];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = xs[k][ty * 4 + i];
+            for (int i = 0; i < MT; ++i) a[i] = xs[k][ty * MT + i];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = ws[k][tx * 4 + j];
+            for (int j = 0; j < MT; ++j) b[j] = ws[k][tx * MT + j];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < MT; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+                for (int j = 0; j < MT; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
         }
         __syncthreads();
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = m0 + ty * 4 + i;
+    for (int i = 0; i < MT; ++i) {
+        const int m = m0 + ty * MT + i;
         if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + tx * 4 + j;
+        for (int j = 0; j < MT; ++j) {
+            const int n = n0 + tx * MT + j;
             if (n >= N) continue;
             float v = acc[i][j];
             if (bias) v += load_vec(bias, bias_f32, n);
             out[(size_t)m * ldo + n] = from_float<TOut>(v);
         }
+    }
+}
+
+template <typename TIn, typename TOut>
+static void launch_gemm_tile(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                             int ldx, int ldo, hipStream_t stream) {
+    if (M >= 128 && N >= 128) {
+        dim3 grid((N + 127) / 128, (M + 127) / 128), block(256);
+        gemm_tile_kernel<TIn, TOut, 128><<<grid, block, 0, stream>>>((const TIn*)x, (const TIn*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo);
+    } else {
+        dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
+        gemm_tile_kernel<TIn, TOut, 64><<<grid, block, 0, stream>>>((const TIn*)x, (const TIn*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo);
     }
 }
 
@@ -75,13 +90,9 @@ extern "C" int tl_gemm_general(const void* x, const void* w, const void* bias, i
                                hipStream_t stream) {
     TL_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldo >= N, "gemm: bad sizes M=%d N=%d K=%d ldx=%d ldo=%d", M, N, K, ldx, ldo);
     if (M == 0) return TL_OK;
-    dim3 grid((N + GT_N - 1) / GT_N, (M + GT_M - 1) / GT_M), block(256);
-    if (dtype == TL_DT_F32)
-        gemm_tile_kernel<float, float><<<grid, block, 0, stream>>>((const float*)x, (const float*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo);
-    else if (dtype == TL_DT_BF16 && out_f32)
-        gemm_tile_kernel<bf16_t, float><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo);
-    else if (dtype == TL_DT_BF16)
-        gemm_tile_kernel<bf16_t, bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo);
+    if (dtype == TL_DT_F32) launch_gemm_tile<float, float>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream);
+    else if (dtype == TL_DT_BF16 && out_f32) launch_gemm_tile<bf16_t, float>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream);
+    else if (dtype == TL_DT_BF16) launch_gemm_tile<bf16_t, bf16_t>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream);
     else TL_REQUIRE(false, "gemm: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("gemm_general");
     return TL_OK;

@@ -14,7 +14,7 @@ class RequestState(Enum):
     FINISHED = "finished"
 
 
-@dataclass
+@dataclass(eq=False)          # a request is itself: lists of requests are searched by identity, not by field values
 class Request:
     prompt_tokens: list[int]
     max_new_tokens: int = 128

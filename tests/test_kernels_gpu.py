@@ -297,12 +297,14 @@ def test_rope_cache_write(ops, dtype, nh, nkv, hd, page, theta):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("lens", [[5, 1, 11], [70, 1, 130]])
 @pytest.mark.parametrize("nh,nkv,hd,page,theta", [(4, 2, 16, 16, 1e4), (28, 4, 128, 16, 1e6), (5, 5, 48, 4, 5e5)])
-def test_rope_cache_write_in_the_pair_layout(ops, dtype, nh, nkv, hd, page, theta):
+def test_rope_cache_write_in_the_pair_layout(ops, dtype, lens, nh, nkv, hd, page, theta):
     """With the dimensions of every head reordered so that the two that a frequency turns are
-    neighbours, the kernel's pair mode gives the reordered result of the usual rotation."""
+    neighbours, the kernel's pair mode gives the reordered result of the usual rotation (a few
+    tokens: one wave per head; many tokens in bfloat16: the kernel that moves 16 bytes at a time)."""
     g = torch.Generator().manual_seed(6)
-    lens, ctxs = [5, 1, 11], [0, 37, 6]
+    ctxs = [0, 37, 6]
     T = sum(lens)
     max_blocks = (max(a + b for a, b in zip(lens, ctxs)) + page - 1) // page
     pages = 3 * max_blocks + 2

@@ -27,6 +27,8 @@ _PORTION_MIN_TOKENS = 16     # requests that bring at least this many tokens go 
                              # 8192 new tokens 2.9 -> 0.84 ms), else the 64-row one ...
 _PORTION_MIN_CONTEXT = 4096  # ... which pays only in steps whose longest sequence has at least this many tokens
 _PROMPT_TARGET_WORKGROUPS = 1024  # the 128-row kernel: two work-groups fit a compute unit; two rounds of them (measured: 14B serving 16.2k -> 16.5k tokens/s against one round)
+_PROMPT_SPLIT_BELOW = 256        # ... but only steps whose tiles alone cannot give every compute unit one (a whole prompt of
+                                 # 2048 tokens has 456: split in two it took 85 + 19 us of merge against 90 us)
 _PROMPT_MIN_KEYS_PER_SPLIT = 512
 _PROMPT_MAX_SPLITS = 4
 
@@ -162,7 +164,8 @@ class GQAttention(Mixer):
                 # each tile's keys are dealt to several work-groups, so that the compute units have work
                 groups = long[2] * self.kv_heads * -(-(self.heads // self.kv_heads) // ops.PROMPT_ATTENTION_ROWS)
                 keys = ctx.max_total_len if self.window is None else min(ctx.max_total_len, self.window + tq)
-                splits = max(1, min(_PROMPT_MAX_SPLITS, _PROMPT_TARGET_WORKGROUPS // max(groups, 1), keys // _PROMPT_MIN_KEYS_PER_SPLIT))
+                splits = 1 if groups > _PROMPT_SPLIT_BELOW else \
+                    max(1, min(_PROMPT_MAX_SPLITS, _PROMPT_TARGET_WORKGROUPS // max(groups, 1), keys // _PROMPT_MIN_KEYS_PER_SPLIT))
                 extra = dict(max_total_len=ctx.max_total_len, splits=splits, merge_tokens=(long[3], long[4]))
             kernel(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens, long[0], long[1], long[2], tq, *common, **extra)
             if short[2]:     # split over their keys; the merge of the parts is kept to the rows of these requests

@@ -576,20 +576,16 @@ static void pick_skinny(const void* x, const void* w, const void* bias, int bias
     }
 }
 
-// One named instance of the few-rows kernel (tests cover every instance; tuning times them).
+// One named instance of the few-rows kernel, of those the dispatch below can pick (for tests and tuning).
 extern "C" int tl_gemm_skinny_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
                                       int M, int N, int K, int ldx, int ldo, int out_f32, int R, int KS, hipStream_t stream) {
     TL_REQUIRE(M > 0 && M <= 64 && K % 8 == 0 && ldx % 8 == 0, "gemm_skinny: needs 0 < M <= 64 and K, ldx multiples of 8");
     const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
 #define TL_SKINNY_CASE(r, t, k) \
     if (R == r && MT == t && KS == k) { launch_skinny<r, t, k>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream); TL_CHECK_LAUNCH("gemm_skinny"); return TL_OK; }
-    TL_SKINNY_CASE(1, 1, 4) TL_SKINNY_CASE(1, 2, 4) TL_SKINNY_CASE(1, 4, 4)
-    TL_SKINNY_CASE(2, 1, 4) TL_SKINNY_CASE(2, 2, 4) TL_SKINNY_CASE(2, 4, 4)
-    TL_SKINNY_CASE(4, 1, 4) TL_SKINNY_CASE(4, 2, 4) TL_SKINNY_CASE(4, 4, 4)
-    TL_SKINNY_CASE(1, 1, 8) TL_SKINNY_CASE(1, 2, 8) TL_SKINNY_CASE(1, 4, 8)
-    TL_SKINNY_CASE(2, 1, 8) TL_SKINNY_CASE(2, 2, 8) TL_SKINNY_CASE(2, 4, 8)
-    TL_SKINNY_CASE(1, 1, 16) TL_SKINNY_CASE(1, 2, 16) TL_SKINNY_CASE(1, 4, 16)
-    TL_SKINNY_CASE(1, 1, 2) TL_SKINNY_CASE(2, 1, 2) TL_SKINNY_CASE(4, 1, 2) TL_SKINNY_CASE(4, 4, 2) TL_SKINNY_CASE(2, 4, 2)
+    // the instances pick_skinny can choose
+    TL_SKINNY_CASE(1, 1, 16) TL_SKINNY_CASE(1, 2, 16) TL_SKINNY_CASE(1, 1, 8) TL_SKINNY_CASE(1, 2, 8)
+    TL_SKINNY_CASE(4, 4, 4) TL_SKINNY_CASE(2, 4, 2) TL_SKINNY_CASE(1, 4, 8)
 #undef TL_SKINNY_CASE
     TL_REQUIRE(false, "gemm_skinny: no instance R=%d MT=%d KS=%d", R, MT, KS);
 }
@@ -1135,11 +1131,9 @@ extern "C" int tl_gemm_tile_variant(const void* x, const void* w, const void* bi
     int rc = -1;
 #define TL_TILE_CASE(bm, bn, gm, gn, tk) \
     if (BM == bm && BN == bn && TK == tk) rc = launch_mfma_tile<bm, bn, gm, gn, tk>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
+    // the tile shapes pick_tile can choose
     TL_TILE_CASE(128, 128, 2, 2, 32) TL_TILE_CASE(128, 128, 2, 2, 64)
-    TL_TILE_CASE(256, 128, 4, 2, 32) TL_TILE_CASE(256, 128, 4, 2, 64)
-    TL_TILE_CASE(128, 256, 2, 4, 32) TL_TILE_CASE(128, 256, 2, 4, 64)
-    TL_TILE_CASE(64, 128, 1, 4, 32) TL_TILE_CASE(64, 128, 2, 2, 64)
-    TL_TILE_CASE(256, 256, 4, 2, 32) TL_TILE_CASE(256, 256, 4, 2, 64)
+    TL_TILE_CASE(64, 128, 2, 2, 64) TL_TILE_CASE(256, 256, 4, 2, 64)
 #undef TL_TILE_CASE
     TL_REQUIRE(rc != -1, "gemm_tile: no instance BM=%d BN=%d TK=%d", BM, BN, TK);
     if (rc != TL_OK) return rc;

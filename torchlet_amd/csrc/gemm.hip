@@ -1319,7 +1319,12 @@ extern "C" int tl_gemm_partials_max() { return 8; }
 // Whether the tile kernel does the split: from 17 rows on, and from 2 rows on against a long K
 // (measured at 3584 x 18944 with the sum in the norm: 8 rows 31.8 against 35.6 us, 16 rows 32.5 against
 // 42.0 us; against a short K, 3584 x 3584, the skinny kernel without a split stays ahead up to 16 rows).
-static bool partials_on_tiles(int M, int K) { return K % 64 == 0 && (M > 16 || (M >= 2 && K >= 8192)); }
+// One row against a long K: where the few-rows kernel would need a second, nearly empty round of work-groups
+// (more than 256 strips of 16 weight rows, one work-group of eight waves with eight steps in flight per
+// compute unit), the split keeps every unit busy in one (5120 x 27648: 70.8 -> 53 us, 5120 x 13824: 38.6 -> 28.5 us).
+static bool partials_on_tiles(int M, int N, int K) {
+    return K % 64 == 0 && (M > 16 || (M >= 2 && K >= 8192) || (M == 1 && K >= 8192 && N > 16 * 256));
+}
 
 // Whether a consumer that can add slabs up should ask for them instead of the whole product.
 extern "C" int tl_gemm_partials_pay(int M, int N, int K);
@@ -1327,7 +1332,7 @@ extern "C" int tl_gemm_partials_pay(int M, int N, int K);
 // How many parts tl_gemm_partials would use.
 extern "C" int tl_gemm_partials_parts(int M, int N, int K) {
     if (M > 64 && K % 64 == 0) return plan_dl_split(M, N, K).parts;
-    if (partials_on_tiles(M, K)) {
+    if (partials_on_tiles(M, N, K)) {
         const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
         int P = (int)(256 / tiles);                       // about one work-group per compute unit
         const int by_k = K / 512;                         // at least eight slabs of 64 per part
@@ -1341,7 +1346,7 @@ extern "C" int tl_gemm_partials_parts(int M, int N, int K) {
 }
 
 extern "C" int tl_gemm_partials_pay(int M, int N, int K) {
-    return partials_on_tiles(M, K) && tl_gemm_partials_parts(M, N, K) > 1;
+    return partials_on_tiles(M, N, K) && tl_gemm_partials_parts(M, N, K) > 1;
 }
 
 extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int* parts,
@@ -1362,7 +1367,7 @@ extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, 
     const int k_per = ((steps + P - 1) / P) * 64;
     P = (K + k_per - 1) / k_per;
     *parts = P;
-    if (partials_on_tiles(M, K)) {
+    if (partials_on_tiles(M, N, K)) {
         auto kernel = gemm_dl_tile_kernel<64, 64, 2, 2, 4, float, false>;
         constexpr size_t lds = (size_t)4 * 128 * 64 * sizeof(bf16_t);
         static hipError_t allowed = allow_lds(kernel, lds);

@@ -1312,18 +1312,19 @@ extern "C" int tl_gemm_swiglu(const void* x, const void* w, void* out, int M, in
 // 3584 x 18944 147 -> 82 us, 5120 x 13824 179 -> 82 us, 5120 x 27648 348 -> 150 us, the norm's sum
 // included).  Up to 64 rows, where it pays (see partials_on_tiles), the direct-load tile
 // kernel runs with 64 x 64 tiles (measured at 64 rows, 3584 x 18944: 31 us with four parts against
-// 90 us whole; 3584 x 3584: 9.5 against 20 us); up to 16 rows, or for other K, the skinny kernel
+// 90 us whole; 3584 x 3584: 9.5 against 20 us); for other K the skinny kernel
 // with R = 4 strips per work-group, which share every x fetch.
 extern "C" int tl_gemm_partials_max() { return 8; }
 
-// Whether the tile kernel does the split: from 17 rows on, and from 2 rows on against a long K
-// (measured at 3584 x 18944 with the sum in the norm: 8 rows 31.8 against 35.6 us, 16 rows 32.5 against
-// 42.0 us; against a short K, 3584 x 3584, the skinny kernel without a split stays ahead up to 16 rows).
-// One row against a long K: where the few-rows kernel would need a second, nearly empty round of work-groups
-// (more than 256 strips of 16 weight rows, one work-group of eight waves with eight steps in flight per
-// compute unit), the split keeps every unit busy in one (5120 x 27648: 70.8 -> 53 us, 5120 x 13824: 38.6 -> 28.5 us).
+// Whether the tile kernel does the split: from 2 rows on, and for one row where the few-rows kernel
+// has more than 256 strips of 16 weight rows to deal out.  Measured with the consumer's sum left out
+// (us, few-rows kernel against split tiles): 3584 x 3584: 1 row 7.0 / 7.4, 2 rows 8.0 / 7.4, 8 rows 9.1 / 7.5,
+// 16 rows 10.6 / 7.6; 5120 x 5120: 1 row 16.2 / 13.2, 8 rows 19.0 / 12.7, 16 rows 22.5 / 13.1;
+// 3584 x 18944: 1 row 28.2 / 27.2, 8 rows 31.6 / 26.1, 16 rows 38.2 / 26.6; 5120 x 27648, one row: 70.8 / 53
+// (320 strips, one work-group of eight waves with eight steps in flight per compute unit: two rounds,
+// the second nearly empty).
 static bool partials_on_tiles(int M, int N, int K) {
-    return K % 64 == 0 && (M > 16 || (M >= 2 && K >= 8192) || (M == 1 && K >= 8192 && N > 16 * 256));
+    return K % 64 == 0 && (M >= 2 || N > 16 * 256);
 }
 
 // Whether a consumer that can add slabs up should ask for them instead of the whole product.

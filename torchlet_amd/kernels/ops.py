@@ -143,7 +143,7 @@ def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: to
 def linear_partials_pay(M: int, N: int, K: int) -> bool:
     """Whether a bfloat16 product whose consumer can add slabs up should come from
     :func:`linear_partials` (K a multiple of 64): up to 64 rows when its 64 x 64 output tiles are
-    too few to fill the GPU (from 17 rows on, and from 2 rows on against a long K); with more rows
+    too few to fill the GPU (from 2 rows on; one row against a matrix of more than 4096 rows); with more rows
     when the library's estimate finds a tile shape with K split 2-8 ways faster than the best
     whole product, slabs included."""
     return bool(_lib("gemm").tl_gemm_partials_pay(c_int(M), c_int(N), c_int(K)))

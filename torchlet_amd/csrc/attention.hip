@@ -506,12 +506,15 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(AttnArgs a
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, g = lane >> 4;
 
-    // later tiles of a prompt see more keys: start them first, so that the short ones fill the end
-    const int tile = gridDim.x - 1 - blockIdx.x;
+    // later tiles of a prompt see more keys: start them first, each with all its key/value heads (launch
+    // order runs along x first), so that the short ones fill the end
+    const int rank = blockIdx.y * gridDim.x + blockIdx.x;
+    const int tile = gridDim.x - 1 - rank / (int)gridDim.y;
+    const int by = rank % (int)gridDim.y;
     const int group = a.heads / a.kv_heads;
     const int chunks_h = (group + a.gcap - 1) / a.gcap;
-    const int kvh = blockIdx.y / chunks_h;
-    const int g0 = (blockIdx.y % chunks_h) * a.gcap;
+    const int kvh = by / chunks_h;
+    const int g0 = (by % chunks_h) * a.gcap;
     const int gcount = min(a.gcap, group - g0);
 
     const int req = a.tile_req[tile];
@@ -827,11 +830,19 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lr = lane & 31, h = lane >> 5;
 
-    const int tile = gridDim.x - 1 - blockIdx.x;            // late tiles see the most keys: they start first
+    // Late tiles see the most keys: they start first, each with all its key/value heads, so that the
+    // work-groups still running at the end are the light ones (launch order runs along x first; taking
+    // the tile from x alone started the heavy tiles of the last head after the light ones of the first:
+    // a 2048-token prompt 83 -> 75 us, 4096 tokens 231 -> 180 us, 2048 tokens with 40 heads in 8 groups
+    // 102 -> 81 us).
+    const int per_tile = gridDim.y;
+    const int rank = blockIdx.y * gridDim.x + blockIdx.x;
+    const int tile = gridDim.x - 1 - rank / per_tile;
+    const int by = rank % per_tile;
     const int group = a.heads / a.kv_heads;
     const int chunks_h = (group + a.gcap - 1) / a.gcap;
-    const int kvh = blockIdx.y / chunks_h;
-    const int g0 = (blockIdx.y % chunks_h) * a.gcap;
+    const int kvh = by / chunks_h;
+    const int g0 = (by % chunks_h) * a.gcap;
     const int gcount = min(a.gcap, group - g0);
 
     const int req = a.tile_req[tile];

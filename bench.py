@@ -132,18 +132,25 @@ def time_decode(model, batch: int, steps: int, warmup: int, context: int = CONTE
     from torchlet_amd.engine.loading import make_runner
     from torchlet_amd.sampling.sampler import Sampler
 
-    pages = batch * (-(-(context + steps + warmup + 1) // PAGE)) + 1
+    pages = batch * (-(-(context + steps + warmup + 2) // PAGE)) + 1
     runner = make_runner(model, page_size=PAGE, num_pages=pages, max_requests=batch, use_graphs=True)
     ids = [f"b{i}" for i in range(batch)]
     fill_context(runner, ids, context)
     sampler = Sampler(0)
-    tokens = [1 + i for i in range(batch)]
     zeros = [0.0] * batch
+    # As the engine runs decode steps: a step takes its tokens on the GPU from the sampling of the step
+    # before it and is enqueued while the host still waits for those tokens; every token is read.
+    logits = runner.step([StepEntry(r, [1 + i], [0]) for i, r in enumerate(ids)])
+    drawn = sampler.launch(logits, zeros, zeros, zeros)
+    entries = [StepEntry(r, [0], [0]) for r in ids]
+    generated = []
 
     def step():
-        nonlocal tokens
-        logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(ids, tokens)])
-        tokens = sampler.sample(logits, zeros, zeros, zeros)
+        nonlocal drawn
+        logits = runner.step(entries, device_tokens=(drawn.device, None))
+        following = sampler.launch(logits, zeros, zeros, zeros)
+        generated.append(drawn.tokens())
+        drawn = following
 
     for _ in range(warmup):
         step()
@@ -153,6 +160,7 @@ def time_decode(model, batch: int, steps: int, warmup: int, context: int = CONTE
         step()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / steps
+    assert len(generated) == warmup + steps and all(len(t) == batch for t in generated)
     del runner
     torch.cuda.empty_cache()
     return ms

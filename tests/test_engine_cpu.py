@@ -121,6 +121,42 @@ def test_temperature_sampling_is_the_same_alone_batched_and_after_preemption(cpu
     assert r.output_tokens != alone[1]                          # another sampler seed, other draws
 
 
+def test_a_step_enqueued_ahead_of_its_tokens_changes_nothing_that_is_generated(cpu_ops, model_folders):
+    """Decode steps that take their tokens from the sampler's output before the host has read them:
+    same tokens as without, for requests that end by length at different times, that end on a stop
+    token (found out one step late: the place in the step already enqueued counts for nothing), that
+    sample with a temperature, and with a request that arrives in between."""
+    cfg = json.loads((model_folders["B"] / "config.json").read_text())
+    prompts = list(scenarios.make_requests(cfg["vocab_size"], [3, 9, 20, 14], seed=7).values())
+
+    def run(lookahead, stop=frozenset(), late=True):
+        e = Engine(runner_for(model_folders["B"], "B"), max_tokens_per_step=64, seed=9, lookahead=lookahead)
+        reqs = [Request(prompt_tokens=p, seed=i, max_new_tokens=n, temperature=t, stop_token_ids=stop)
+                for i, (p, n, t) in enumerate(zip(prompts, (5, 17, 11, 9), (0.0, 0.9, 0.0, 0.7)))]
+        for r in reqs[:3]:
+            e.add_request(r)
+        step = 0
+        while e.has_work() or step < 8:
+            if step == 7 and late:
+                e.add_request(reqs[3])
+            if e.has_work():
+                e.step()
+            e.runner.cache.check()
+            step += 1
+        assert e.runner.cache.live_requests() == [] and e._ahead is None
+        return e, [(r.output_tokens, r.finish_reason) for r in reqs[:4 if late else 3]]
+
+    e0, plain = run(False)
+    e1, ahead = run(True)
+    assert ahead == plain and e0.steps_ahead == 0 and e1.steps_ahead >= 8
+    assert [len(t) for t, _ in plain] == [5, 17, 11, 9]
+    # a stop token: one that the second request generates in the middle of its run
+    stop = frozenset({plain[1][0][6]})
+    e0, plain_s = run(False, stop)
+    e1, ahead_s = run(True, stop)
+    assert ahead_s == plain_s and plain_s[1][1] == "stop" and len(plain_s[1][0]) <= 6 and e1.steps_ahead > 0
+
+
 def test_draw_keys_differ_in_every_argument():
     keys = {draw_key(s, r, i) for s in (0, 1, 2 ** 40) for r in (0, 1, 2 ** 33) for i in range(4)}
     assert len(keys) == 36 and all(-2 ** 31 <= k < 2 ** 31 for k in keys)

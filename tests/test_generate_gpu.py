@@ -46,6 +46,38 @@ def test_greedy_generation_through_the_entry_point(model_folders, dtype):
     assert llm.runner.cache.live_requests() == []
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("graphs", [False, True])
+def test_decode_steps_enqueued_ahead_of_their_tokens_generate_the_same(model_folders, dtype, graphs):
+    """Decode steps that take their tokens on the GPU from the sampling kernel's output, enqueued
+    while the host still waits for those tokens (eagerly and as replayed graphs): the same tokens
+    as step after step, with a temperature, with requests that end at different times, and with a
+    stop token that ends one of them a step before the host finds out."""
+    from torchlet_amd import LLM
+    cfg = json.loads((model_folders["D"] / "config.json").read_text())
+    prompts = list(scenarios.make_requests(cfg["vocab_size"], [3, 40, 21], seed=4).values())
+
+    def run(lookahead, stop=None):
+        llm = LLM(str(model_folders["D"]), max_decode_slots=4, kv_block_size=8, dtype=dtype, use_graphs=graphs,
+                  lookahead=lookahead, seed=5)
+        outs = [llm.generate([p], max_new_tokens=n, temperature=t, seed=i, stop_token_ids=stop)[0]
+                for i, (p, n, t) in enumerate(zip(prompts, (30, 9, 17), (0.0, 0.8, 0.0)))]
+        together = llm.generate(prompts, max_new_tokens=24, temperature=0.7, seed=11, stop_token_ids=stop)
+        assert llm.runner.cache.live_requests() == [] and llm.engine._ahead is None
+        return llm, outs, together
+
+    plain_llm, alone, together = run(False)
+    ahead_llm, alone2, together2 = run(True)
+    assert alone2 == alone and together2 == together
+    assert plain_llm.engine.steps_ahead == 0 and ahead_llm.engine.steps_ahead >= 40
+    if graphs:
+        assert ahead_llm.runner.graph_replays > 20
+    stop = [alone[0][12]]                                  # the first request meets it after 12 tokens, or earlier
+    _, alone_s, together_s = run(False, stop)
+    _, alone_s2, together_s2 = run(True, stop)
+    assert alone_s2 == alone_s and together_s2 == together_s and len(alone_s[0]) <= 12
+
+
 def test_continuous_batching_with_temperature_and_few_pages(model_folders):
     """Configuration B's workload (temperature 0.8, fixed seed, 12 new tokens, arrivals at steps
     0, 0, 3, 5) with so few pages that requests are preempted: tokens equal each request alone."""

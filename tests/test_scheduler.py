@@ -141,3 +141,46 @@ def test_nobody_can_move_raises_and_fail_all_resets():
     failed = s.fail_all(RuntimeError("boom"))
     assert a in failed and a.state == RequestState.FINISHED and isinstance(a.error, RuntimeError)
     assert cache.free_pages() == [3] and cache.free_slots() == 2 and not s.has_work()
+
+
+def test_the_scheduler_looks_ahead_only_where_the_next_step_is_certain():
+    """The step after a decode step, decided before that step's tokens are known."""
+    s, cache = make(pages=9, page=4, slots=3, budget=8, max_positions=64)
+    a, b = req(3, new=3), req(5, new=2)
+    s.add_request(a)
+    s.add_request(b)
+    first = s.schedule()
+    assert s.schedule_ahead(first) == []                         # prompts, not decoded tokens
+    s.process_output(first, [10, 11])
+    second = s.schedule()
+    assert [(c.start, c.count, c.samples) for c in second] == [(3, 1, True), (5, 1, True)]
+    late = req(1, new=2)
+    s.add_request(late)
+    assert s.schedule_ahead(second) == []                        # somebody waits: the next step is for schedule() to decide
+    s.waiting.clear()
+    ahead = s.schedule_ahead(second)                             # b ends with the token of `second`: only a goes on
+    assert [(c.request is a, c.start, c.count, c.samples) for c in ahead] == [(True, 4, 1, True)]
+    cache.check()
+    s.process_output(second, [12, 13])
+    assert b.finish_reason == "length" and a.output_tokens == [10, 12]
+    s.process_output(ahead, [14])
+    assert a.finish_reason == "length" and a.output_tokens == [10, 12, 14] and not s.has_work()
+    cache.check()
+    assert cache.free_pages() == [8] and cache.free_slots() == 3
+    # the tokens after next need two pages and one is left: no step ahead, and no page taken for it
+    s, cache = make(pages=4, page=4, slots=2, budget=8, max_positions=64)
+    for r in (req(3, new=6), req(3, new=6)):
+        s.add_request(r)
+    s.process_output(s.schedule(), [5, 5])
+    step = s.schedule()                                          # the tokens at position 3 fill the requests' first pages
+    assert [(x.start, x.count) for x in step] == [(3, 1), (3, 1)] and cache.free_pages() == [1]
+    assert s.schedule_ahead(step) == [] and cache.free_pages() == [1]
+    cache.check()
+    # a budget smaller than the running requests leaves somebody out: nothing to foresee
+    s, cache = make(pages=20, page=4, slots=3, budget=3, max_positions=64)
+    for r in (req(1, new=4), req(1, new=4), req(1, new=4)):
+        s.add_request(r)
+    s.process_output(s.schedule(), [7, 7, 7])
+    s.max_tokens_per_step = 2
+    chosen = s.schedule()
+    assert len(s.running) == 3 and len(chosen) == 2 and not s.waiting and s.schedule_ahead(chosen) == []

@@ -48,23 +48,40 @@ class ModelRunner:
         self._graphs: dict[tuple[int, int], _DecodeGraph] = {}
         self.graph_replays = 0
 
-    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+    def step(self, entries: list[StepEntry], device_tokens: tuple | None = None) -> torch.Tensor | None:
         """Logits ``[number of wanted places, vocab]`` (float32, on the GPU), in the order
-        of the entries and of their ``want`` lists; ``None`` if nothing is wanted."""
+        of the entries and of their ``want`` lists; ``None`` if nothing is wanted.
+
+        ``device_tokens = (tokens, places)``: every entry brings one token, and entry ``i`` takes it
+        from ``tokens[places[i]]`` (an int32 tensor on the GPU, ``places`` a list or ``None`` for
+        ``0, 1, 2, ...``) instead of from its own list, whose one element only stands in.  The step
+        is then enqueued without the host knowing the tokens: a step can follow the sampling of the
+        one before it while the host still waits for those tokens."""
         if not entries:
             return None
         cache = self.cache
         added = []
         try:
-            return self._step(entries, added)
+            return self._step(entries, added, device_tokens)
         except Exception:
             for req_id in added:            # a failed step leaves no trace of requests it introduced
                 if cache.has(req_id) and cache.length(req_id) == 0:
                     cache.release(req_id)
             raise
 
-    def _step(self, entries: list[StepEntry], added: list) -> torch.Tensor | None:
+    def _step(self, entries: list[StepEntry], added: list, device_tokens: tuple | None = None) -> torch.Tensor | None:
         cache = self.cache
+        taken = None
+        if device_tokens is not None:
+            source, places = device_tokens
+            if any(len(e.tokens) != 1 for e in entries):
+                raise ValueError("tokens taken from the GPU: every request brings exactly one")
+            if places is None or list(places) == list(range(len(entries))):
+                taken = source[: len(entries)]
+            else:
+                taken = source[torch.as_tensor(list(places), dtype=torch.int64).to(source.device)]
+            if taken.numel() != len(entries):
+                raise ValueError(f"{len(entries)} requests, but {taken.numel()} tokens on the GPU")
         seen = set()
         for e in entries:
             if e.req_id in seen:
@@ -100,7 +117,7 @@ class ModelRunner:
         blocks = -(-max(c + n for c, n in zip(ctx_lens, new_lens)) // cache.page_size)
         if (self.use_graphs and max(new_lens) == 1 and len(entries) <= self.max_graph_width
                 and all(e.want == [0] for e in entries)):
-            logits = self._graph_step(entries, req_ids, ctx_lens, blocks)
+            logits = self._graph_step(entries, req_ids, ctx_lens, blocks, taken)
             for e, c in zip(entries, ctx_lens):
                 cache.commit(e.req_id, c + 1)
             return logits
@@ -114,12 +131,14 @@ class ModelRunner:
             token_ids=token_ids, want_rows=want_rows,
             block_tables=[cache.block_table(g, req_ids, blocks) for g in range(len(cache.groups))],
             tile_sizes=self.tile_sizes, device=self.device)
+        if taken is not None:
+            ctx.token_ids.copy_(taken)
         logits = self.model.forward(ctx, self.caches)
         for e, c, n in zip(entries, ctx_lens, new_lens):
             cache.commit(e.req_id, c + n)
         return logits
 
-    def _graph_step(self, entries, req_ids, ctx_lens, blocks) -> torch.Tensor:
+    def _graph_step(self, entries, req_ids, ctx_lens, blocks, taken=None) -> torch.Tensor:
         cache = self.cache
         width = _next_pow2(len(entries))
         most = -(-self.max_positions // cache.page_size)
@@ -133,6 +152,8 @@ class ModelRunner:
         dg.ctx.fill(token_ids=[e.tokens[0] for e in entries], ctx_lens=ctx_lens,
                     slots=[cache.slot(r) for r in req_ids],
                     block_tables=[cache.block_table(g, req_ids, bucket) for g in range(len(cache.groups))])
+        if taken is not None:
+            dg.ctx.token_ids[: len(entries)].copy_(taken)             # after the copy of the step's other numbers
         if dg.graph is None:
             logits = self.model.forward(dg.ctx, self.caches)          # eager: this step's result
             result = logits[: len(entries)].clone()

@@ -134,6 +134,30 @@ class Scheduler:
             raise RuntimeError("cache pool exhausted; no request can make progress")
         return chosen
 
+    def schedule_ahead(self, prev: list[Scheduled]) -> list[Scheduled]:
+        """The step after ``prev``, decided before the tokens of ``prev`` are known, or nothing where
+        it cannot be foreseen.  It can when ``prev`` gave every running request one decoded token and
+        nobody waits: the next step then gives each of them one more, except those that end with the
+        token of ``prev`` for having ``max_new_tokens``.  A request that the token of ``prev`` ends
+        as a stop token is in this step for nothing; the caller drops its place when it learns so.
+        Pages are taken for all or for none."""
+        if self.waiting or not prev or len(prev) != len(self.running) or len(prev) > self.max_tokens_per_step:
+            return []
+        if any(c.count != 1 or not c.samples or c.request.state is not RequestState.RUNNING for c in prev):
+            return []
+        going = [c.request for c in prev if len(c.request.output_tokens) + 1 < c.request.max_new_tokens]
+        if not going:
+            return []
+        need = [0] * len(self.cache.groups)
+        for r in going:
+            for g, m in enumerate(self.cache.pages_missing(r.req_id, r.computed_tokens + 2)):
+                need[g] += m
+        if any(n > f for n, f in zip(need, self.cache.free_pages())):
+            return []
+        for r in going:
+            self.cache.reserve(r.req_id, r.computed_tokens + 2)
+        return [Scheduled(r, r.computed_tokens + 1, 1, True) for r in going]
+
     # ------------------------------------------------------------------ applying results
     def process_output(self, chosen: list[Scheduled], sampled: list[int]) -> list[Request]:
         """``sampled``: one token per entry of ``chosen`` with ``samples`` set, in order.

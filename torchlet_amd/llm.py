@@ -39,7 +39,8 @@ from .engine.request import Request
 class LLM:
     def __init__(self, model_id: str, max_decode_slots: int = 4, kv_block_size: int = 16,
                  max_num_blocks: int | None = None, *, dtype: str = "bfloat16",
-                 max_num_batched_tokens: int = 2048, seed: int = 0, use_graphs: bool = True):
+                 max_num_batched_tokens: int = 2048, seed: int = 0, use_graphs: bool = True,
+                 lookahead: bool = True):
         self.device = require_gpu()
         if kv_block_size <= 0:
             raise ValueError("kv_block_size must be positive")
@@ -58,7 +59,7 @@ class LLM:
             max_num_blocks = max(2, min(max_num_blocks, int(free * 0.8) // per_page))
         self.runner = make_runner(self.model, page_size=kv_block_size, num_pages=max_num_blocks,
                                   max_requests=max_decode_slots, use_graphs=use_graphs)
-        self.engine = Engine(self.runner, max_tokens_per_step=max_num_batched_tokens, seed=seed)
+        self.engine = Engine(self.runner, max_tokens_per_step=max_num_batched_tokens, seed=seed, lookahead=lookahead)
         self.tokenizer = _load_tokenizer(self.model_dir)
         self.stop_ids = self._stop_ids()
         self._next_seed = 0
@@ -117,7 +118,7 @@ class LLM:
             try:
                 self.engine.step()
             except Exception as exc:
-                self.engine.scheduler.fail_all(exc)
+                self.engine.fail_all(exc)
                 raise
             await asyncio.sleep(0)
         self.engine.scheduler.drain_finished()

@@ -42,9 +42,11 @@ class Sampler:
     def __init__(self, seed: int = 0):
         self.seed = int(seed)
 
-    def sample(self, logits: torch.Tensor, temperatures: list[float], request_seeds: list[int],
-               token_indices: list[int]) -> list[int]:
-        """One token per row of ``logits [N, vocab]`` (float32, on the GPU)."""
+    def launch(self, logits: torch.Tensor, temperatures: list[float], request_seeds: list[int],
+               token_indices: list[int]) -> "Drawn":
+        """Start the draw of one token per row of ``logits [N, vocab]`` (float32, on the GPU) and the
+        copy of the tokens to the host; nothing waits.  The tokens stay on the GPU as well
+        (``Drawn.device``), where the next step can take them from before the host has seen them."""
         n = logits.shape[0]
         out = torch.empty(n, dtype=torch.int32, device=logits.device)
         if any(t > 0 for t in temperatures):
@@ -54,4 +56,29 @@ class Sampler:
             ops.sample(logits, temp, keys, out)
         else:
             ops.sample(logits, None, None, out)
-        return out.cpu().tolist()
+        return Drawn(out)
+
+    def sample(self, logits: torch.Tensor, temperatures: list[float], request_seeds: list[int],
+               token_indices: list[int]) -> list[int]:
+        """One token per row of ``logits [N, vocab]`` (float32, on the GPU)."""
+        return self.launch(logits, temperatures, request_seeds, token_indices).tokens()
+
+
+class Drawn:
+    """Tokens of one draw: on the GPU at once, on the host when :meth:`tokens` has waited for the copy."""
+
+    def __init__(self, device_tokens: torch.Tensor):
+        self.device = device_tokens
+        self._host = None
+        self._copied = None
+        if device_tokens.is_cuda:
+            self._host = torch.empty(device_tokens.shape, dtype=device_tokens.dtype, pin_memory=True)
+            self._host.copy_(device_tokens, non_blocking=True)
+            self._copied = torch.cuda.Event()
+            self._copied.record()
+
+    def tokens(self) -> list[int]:
+        if self._copied is None:
+            return self.device.tolist()
+        self._copied.synchronize()
+        return self._host.tolist()

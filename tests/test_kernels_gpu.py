@@ -231,6 +231,23 @@ def test_linear_many_rows_fetched_straight_into_shared_memory(ops, out_dtype, ti
     assert bool((out2[:, N:] == 5.0).all())
 
 
+@pytest.mark.parametrize("tile", [(64, 64, 0), (128, 128, 0), (128, 128, 4), (128, 256, 0), (256, 128, 0), (192, 256, 0), (256, 192, 0), (256, 256, 0)])
+@pytest.mark.parametrize("M,N,K,parts", [(65, 129, 128, 2), (128, 520, 1024, 4), (100, 3584, 2048, 8), (300, 257, 1088, 3), (7, 48, 3584, 7)])
+def test_linear_split_over_k_on_every_tile_shape(ops, tile, M, N, K, parts):
+    """Slabs of partial sums from every tile shape of the direct-load kernel (the four-slab 128 x 128
+    instance among them), with tails in M and N and parts of unequal length: their sum is the product."""
+    g = torch.Generator().manual_seed(M + N + K + parts)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).cuda()
+    ref = x.double() @ w.double().T
+    slabs = ops.linear_direct_split_variant(x, w, tile[0], tile[1], parts, tile[2])
+    assert slabs.shape == (parts, M, N)
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    torch.testing.assert_close(slabs.double().sum(0), ref, **tol32)
+    k_per = -(-(K // 64) // parts) * 64
+    torch.testing.assert_close(slabs[0].double(), x[:, :k_per].double() @ w[:, :k_per].double().T, **tol32)
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 32, 33, 64, 65, 300])
 @pytest.mark.parametrize("I,K", [(128, 64), (200, 96), (112, 80), (18944, 256), (32768 + 40, 64), (100, 128), (36, 64)])
 def test_linear_swiglu_fused(ops, M, I, K):

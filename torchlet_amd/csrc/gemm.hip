@@ -1023,11 +1023,14 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
 // the other; a tile takes a fixed time (filling the pipeline, storing the result) plus its
 // products at the rate one compute unit reaches with that shape (fitted to measurements at
 // 2048 rows against the Qwen2.5-7B and 14B matrices, K from 3584 to 18944).
-enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_64x128, DL_TILES };
-static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 192, 256, 256, 64};
-static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256, 128};
-static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12, 2.1e12};   // FLOP/s of one compute unit
-static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6, 5e-6};       // seconds per tile
+// (DL_128x128_S4: 128 x 128 with four slabs in shared memory, one work-group to a compute unit: for products of up
+// to 128 rows split over K, where what counts is how many bytes of weights a work-group has on their way; measured
+// at 128 rows against the best other tile: 3584 x 18944 48.8 -> 37.1 us, 3584 x 3584 18.6 -> 15.8, 5120 x 5120 29.7 -> 21.4)
+enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_64x128, DL_128x128_S4, DL_TILES };
+static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 192, 256, 256, 64, 128};
+static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256, 128, 128};
+static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12, 2.1e12, 4.2e12};   // FLOP/s of one compute unit
+static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6, 5e-6, 4.5e-6};       // seconds per tile
 
 // Seconds for `groups` work-groups of tile t over k columns each.  The two smallest tiles run two
 // to a compute unit: each then works at half the unit's rate, and one that has a unit to itself
@@ -1052,6 +1055,7 @@ static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = null
     double best_t = 1e30;
     for (int t = 0; t < DL_TILES; ++t) {
         if (sw && (t == DL_64x64 || t == DL_256x192)) continue;      // a wave of the fused gate needs whole 64-row blocks of weights
+        if (t == DL_128x128_S4) continue;                            // for products split over K (plan_dl_split)
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
         const double est = dl_estimate((DlTile)t, tiles, K);
         if (est < best_t) { best_t = est; best = (DlTile)t; }
@@ -1070,12 +1074,13 @@ static DlSplit plan_dl_split(int M, int N, int K) {
     DlSplit best{pick_dl_tile(M, N, K, false, &best_t), 1, 0};
     best_t += (double)M * N * 2 * 2 / 3e12;
     const int steps = K / 64;
-    static const DlTile alone[] = {DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256};
+    static const DlTile alone[] = {DL_128x128_S4, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256};
     for (DlTile t : alone) {
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
         for (int P = 2; P <= 8 && K / P >= 512; ++P) {
             const int k_per = ((steps + P - 1) / P) * 64;
             if ((K + k_per - 1) / k_per != P) continue;
+            if (t == DL_128x128_S4 && tiles * P > 256) continue;       // measured in one round of work-groups only
             // (a tenth on top: float slabs leave the kernel more slowly than the estimate's bfloat16 rows)
             const double est = 1.1 * dl_estimate(t, tiles * P, k_per) + (double)P * M * N * 4 * 2 / 3e12;
             if (est < best_t) { best_t = est; best = DlSplit{t, P, k_per}; }
@@ -1110,6 +1115,9 @@ static int launch_dl_tile(DlTile tile, const void* x, const void* w, const void*
         else break;
     case DL_64x256: return launch_dl_tile_t<64, 256, 1, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_128x128: return launch_dl_tile_t<128, 128, 2, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+    case DL_128x128_S4:
+        if constexpr (!SW) return launch_dl_tile_t<128, 128, 2, 2, 4, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+        else break;
     case DL_128x256: return launch_dl_tile_t<128, 256, 2, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_256x128: return launch_dl_tile_t<256, 128, 4, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_64x128: return launch_dl_tile_t<64, 128, 1, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
@@ -1148,7 +1156,7 @@ extern "C" int tl_gemm_direct_variant(const void* x, const void* w, const void* 
                "gemm_direct: needs M > 0, K a multiple of 64 and 16-byte aligned rows");
     int tile = -1;
     for (int t = 0; t < DL_TILES; ++t)
-        if (DL_BM[t] == BM && DL_BN[t] == BN) tile = t;
+        if (DL_BM[t] == BM && DL_BN[t] == BN && t != DL_128x128_S4) tile = t;
     TL_REQUIRE(tile >= 0, "gemm_direct: no tile of %d x %d", BM, BN);
     const int rc = out_f32 ? launch_dl_tile<float, false>((DlTile)tile, x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream)
                            : launch_dl_tile<bf16_t, false>((DlTile)tile, x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
@@ -1158,14 +1166,15 @@ extern "C" int tl_gemm_direct_variant(const void* x, const void* w, const void* 
 }
 
 // One tile shape with K split into `parts` (float slabs [parts, M, N]); for tests and tuning.
+// stages == 4 with 128 x 128: the four-slab instance.
 extern "C" int tl_gemm_direct_split_variant(const void* x, const void* w, void* out, int M, int N, int K, int ldx,
-                                            int BM, int BN, int parts, hipStream_t stream) {
+                                            int BM, int BN, int parts, int stages, hipStream_t stream) {
     TL_REQUIRE(M > 0 && K % 64 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0 && parts >= 1,
                "gemm_direct_split: needs M > 0, K a multiple of 64 and 16-byte aligned rows");
     int tile = -1;
     for (int t = 0; t < DL_TILES; ++t)
-        if (DL_BM[t] == BM && DL_BN[t] == BN) tile = t;
-    TL_REQUIRE(tile >= 0, "gemm_direct_split: no tile of %d x %d", BM, BN);
+        if (DL_BM[t] == BM && DL_BN[t] == BN && (t == DL_128x128_S4) == (stages == 4)) tile = t;
+    TL_REQUIRE(tile >= 0, "gemm_direct_split: no tile of %d x %d with %d stages", BM, BN, stages);
     const int steps = K / 64;
     const int k_per = ((steps + parts - 1) / parts) * 64;
     TL_REQUIRE((K + k_per - 1) / k_per == parts, "gemm_direct_split: %d parts leave one empty (K=%d)", parts, K);

@@ -231,6 +231,21 @@ def linear_direct_variant(x, weight, bias, out, tile_m: int, tile_n: int) -> Non
                                            c_int(1 if out.dtype == torch.float32 else 0), c_int(tile_m), c_int(tile_n), _stream()))
 
 
+def linear_direct_split_variant(x, weight, tile_m: int, tile_n: int, parts: int, stages: int = 0) -> torch.Tensor:
+    """One named tile shape of the direct-load kernel with K split into ``parts``: float32 slabs
+    ``[parts, M, N]`` (K a multiple of 64; ``stages=4`` with 128 x 128: the four-slab instance; for
+    tests and tuning)."""
+    M, K = x.shape
+    N = weight.shape[0]
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or weight.shape[1] != K or not weight.is_contiguous() or x.stride(1) != 1:
+        raise KernelError("linear_direct_split_variant: bfloat16 operands and fitting shapes only")
+    out = torch.empty((parts, M, N), dtype=torch.float32, device=x.device)
+    lib = _lib("gemm")
+    _check(lib, lib.tl_gemm_direct_split_variant(_ptr(x), _ptr(weight), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(x.stride(0)),
+                                                 c_int(tile_m), c_int(tile_n), c_int(parts), c_int(stages), _stream()))
+    return out
+
+
 def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """The layout :func:`linear_swiglu` wants: blocks of 64 rows, 32 rows of ``gate`` then the
     32 rows of ``up`` with the same indices; the last block is padded with zero rows."""

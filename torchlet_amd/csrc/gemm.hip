@@ -1055,8 +1055,8 @@ static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = null
     double best_t = 1e30;
     for (int t = 0; t < DL_TILES; ++t) {
         if (sw && (t == DL_64x64 || t == DL_256x192)) continue;      // a wave of the fused gate needs whole 64-row blocks of weights
-        if (t == DL_128x128_S4) continue;                            // for products split over K (plan_dl_split)
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
+        if (t == DL_128x128_S4 && (tiles > 256 || M > 128)) continue;      // one round of work-groups, every weight drawn once
         const double est = dl_estimate((DlTile)t, tiles, K);
         if (est < best_t) { best_t = est; best = (DlTile)t; }
     }
@@ -1115,9 +1115,7 @@ static int launch_dl_tile(DlTile tile, const void* x, const void* w, const void*
         else break;
     case DL_64x256: return launch_dl_tile_t<64, 256, 1, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_128x128: return launch_dl_tile_t<128, 128, 2, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
-    case DL_128x128_S4:
-        if constexpr (!SW) return launch_dl_tile_t<128, 128, 2, 2, 4, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
-        else break;
+    case DL_128x128_S4: return launch_dl_tile_t<128, 128, 2, 2, 4, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_128x256: return launch_dl_tile_t<128, 256, 2, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_256x128: return launch_dl_tile_t<256, 128, 4, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_64x128: return launch_dl_tile_t<64, 128, 1, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);

@@ -121,7 +121,20 @@ __global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const void*
                 for (int v = 0; v < 4; ++v) r[it][v] += p[v];
             }
             if (pparts) {
-                for (int q = 0; q < parts; ++q) {
+                // four slabs at a time, all requested before the first is added (a loop over a count known
+                // only at run time fetches one slab after the other: a trip to memory each); the sums are
+                // added in the order of the slabs either way
+                int q = 0;
+                for (; q + 4 <= parts; q += 4) {
+                    float p[4][4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) Vec4<float>::load(pparts + (q + u) * part_stride + i, p[u]);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) r[it][v] += p[u][v];
+                }
+                for (; q < parts; ++q) {
                     float p[4];
                     Vec4<float>::load(pparts + q * part_stride + i, p);
 #pragma unroll
@@ -249,7 +262,16 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
         if (!parts) return to_float(x[i]);
         const size_t col = (size_t)head * head_dim + i;
         float sum = bias ? load_vec(bias, bias_f32, col) : 0.f;
-        for (int p = 0; p < num_parts; ++p) sum += parts[(size_t)p * part_stride + (size_t)t * parts_ld + col];
+        const float* src = parts + (size_t)t * parts_ld + col;
+        int p = 0;
+        for (; p + 4 <= num_parts; p += 4) {       // four slabs requested before the first is added, in their order
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = src[(size_t)(p + u) * part_stride];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) sum += v[u];
+        }
+        for (; p < num_parts; ++p) sum += src[(size_t)p * part_stride];
         return sum;
     };
     if (head >= q_heads + kv_heads) {      // value head: [head_dim, page] inside the page

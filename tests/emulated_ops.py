@@ -90,8 +90,12 @@ def _attend(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_re
             tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale):
     group = num_heads // num_kv_heads
     for tile in range(num_tiles):
-        r = int(tile_req[tile]); t0 = int(tile_tok0[tile])
-        first = int(req_indptr[r]); n_new = int(req_indptr[r + 1]) - first; ctx = int(ctx_lens[r])
+        if tile_req is None:        # every request brings one token: tile i is the token of request i
+            r, t0, first, n_new = tile, 0, tile, 1
+        else:
+            r = int(tile_req[tile]); t0 = int(tile_tok0[tile])
+            first = int(req_indptr[r]); n_new = int(req_indptr[r + 1]) - first
+        ctx = int(ctx_lens[r])
         for i in range(t0, min(t0 + tile_tokens, n_new)):
             pos = ctx + i
             lo = max(0, pos - window + 1) if window else 0

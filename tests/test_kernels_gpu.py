@@ -515,6 +515,40 @@ def test_paged_attention(ops, dtype, general, nh, nkv, hd, page, window, splits)
         torch.testing.assert_close(got[a:b], ref, **tol)
 
 
+@pytest.mark.parametrize("dtype,general", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+@pytest.mark.parametrize("nh,nkv,hd,page,window,splits,wide", [
+    (28, 4, 128, 16, 0, 3, 0), (6, 2, 32, 8, 0, 1, 5), (4, 4, 16, 4, 11, 2, 0), (14, 2, 64, 16, 0, 4, 2100), (5, 1, 48, 32, 40, 1, 3),
+])
+def test_paged_attention_of_a_decode_step_without_a_tile_list(ops, dtype, general, nh, nkv, hd, page, window, splits, wide):
+    """One new token per request and no tile list (the kernel takes tile i for the token of request i and
+    asks for length, block table and query at once): the same bits as with the list, for short and long
+    contexts, a first token, and a block table wider than the kernel keeps in shared memory."""
+    g = torch.Generator().manual_seed(6)
+    ctxs = [150, 0, 70, 33, 1, 299]
+    R = len(ctxs)
+    max_blocks = (max(ctxs) + page) // page + 1 + wide
+    pages = R * ((max(ctxs) + page) // page + 1) + 1
+    bt = torch.zeros(R, max_blocks, dtype=torch.int32)
+    used = (max(ctxs) + page) // page + 1
+    bt[:, :used] = (torch.randperm(pages - 1, generator=g)[: R * used] + 1).view(R, used).int()
+    q = torch.randn(R, nh * hd, generator=g).to(dtype).cuda()
+    kp = torch.randn(pages, nkv, page, hd, generator=g).to(dtype).cuda()
+    vp = torch.randn(pages, nkv, hd, page, generator=g).to(dtype).cuda()
+    indptr = torch.arange(R + 1, dtype=torch.int32).cuda()
+    ctx_t = torch.tensor(ctxs, dtype=torch.int32).cuda()
+    tiles = torch.arange(R, dtype=torch.int32).cuda()
+    zeros = torch.zeros(R, dtype=torch.int32).cuda()
+    tq = ops.attention_tile_tokens(nh, nkv)
+    common = (nh, nkv, hd, page, window, 1.0 / math.sqrt(hd), splits)
+    listed = torch.empty(R, nh * hd, dtype=dtype, device="cuda")
+    ops.paged_attention(q, listed, kp, vp, bt.cuda(), indptr, ctx_t, tiles, zeros, R, tq, *common, general=general)
+    bare = torch.full_like(listed, float("nan"))
+    ops.paged_attention(q, bare, kp, vp, bt.cuda(), None, ctx_t, None, None, R, tq, *common, general=general)
+    assert torch.equal(bare, listed) and bool(torch.isfinite(bare.float()).all())
+    with pytest.raises(ops.KernelError, match="exactly one token"):
+        ops.paged_attention(q, bare, kp, vp, bt.cuda(), None, ctx_t, None, None, R - 1, tq, *common, general=general)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_of_some_requests_leaves_the_other_rows_alone(ops, dtype):
     """Tiles of two of four requests, keys split over work-groups: with the tokens of those

@@ -82,10 +82,12 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
     const int gcount = min(a.gcap, group - g0);
     const int split = blockIdx.z;
 
-    const int req = a.tile_req[tile];
-    const int tok0 = a.tile_tok0[tile];
-    const int first = a.req_indptr[req];
-    const int n_new = a.req_indptr[req + 1] - first;
+    // without a tile list (a step in which every request decodes one token): tile i is the token of request i
+    const bool one_each = a.tile_req == nullptr;
+    const int req = one_each ? tile : a.tile_req[tile];
+    const int tok0 = one_each ? 0 : a.tile_tok0[tile];
+    const int first = one_each ? req : a.req_indptr[req];
+    const int n_new = one_each ? 1 : a.req_indptr[req + 1] - first;
     const int ctx = a.ctx_lens[req];
     const int ntok = min(a.tq, n_new - tok0);                // tokens of this tile
 
@@ -260,10 +262,19 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
     const int gcount = min(a.gcap, group - g0);
     const int split = blockIdx.z;
 
-    const int req = a.tile_req[tile];
-    const int tok0 = a.tile_tok0[tile];
-    const int first = a.req_indptr[req];
-    const int n_new = a.req_indptr[req + 1] - first;
+    // Without a tile list (a step in which every request decodes one token) tile i is the token of request
+    // i: nothing has to be looked up before the request's length, its block table and the query are
+    // requested, all three at once; with a list each of these waits for the one before it.
+    const bool one_each = a.tile_req == nullptr;
+    const int req = one_each ? tile : a.tile_req[tile];
+    __shared__ int bt_s[ATM_BT_MAX];
+    const int* bt_g = a.block_table + (size_t)req * a.bt_stride;
+    const bool bt_whole = a.bt_stride <= ATM_BT_MAX;        // the whole row, before the length says which part is needed
+    if (bt_whole)
+        for (int i = threadIdx.x; i < a.bt_stride; i += 256) bt_s[i] = bt_g[i];
+    const int tok0 = one_each ? 0 : a.tile_tok0[tile];
+    const int first = one_each ? req : a.req_indptr[req];
+    const int n_new = one_each ? 1 : a.req_indptr[req + 1] - first;
     const int ctx = a.ctx_lens[req];
     const int ntok = min(a.tq, n_new - tok0);
 
@@ -299,13 +310,12 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
     // The block-table entries of the keys this work-group reads go to shared memory first: a
     // page lookup in the loop is then a shared-memory read instead of a memory access that the
     // key and value loads would have to wait for (two memory latencies in a row per chunk).
-    __shared__ int bt_s[ATM_BT_MAX];
-    const int* bt_g = a.block_table + (size_t)req * a.bt_stride;
-    const int blk0 = (ch_begin * 32) / page;
+    const int blk0 = bt_whole ? 0 : (ch_begin * 32) / page;
     const int blk_n = ch_begin < ch_end ? (min(ch_end * 32, key_hi) - 1) / page - blk0 + 1 : 0;
-    const bool bt_local = blk_n <= ATM_BT_MAX;
+    const bool bt_local = bt_whole || blk_n <= ATM_BT_MAX;
     if (bt_local) {
-        for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
+        if (!bt_whole)
+            for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
         __syncthreads();
     }
 #define ATM_PAGE_OF(blk) (bt_local ? bt_s[(blk) - blk0] : bt_g[(blk)])
@@ -1164,6 +1174,8 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
     TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
     TL_REQUIRE(page > 0 && bt_stride > 0 && tq > 0 && splits > 0 && window >= 0, "attention: bad page/table/tile sizes");
     TL_REQUIRE(splits == 1 || (part_o && part_ml), "attention: splits > 1 needs scratch");
+    TL_REQUIRE((tile_req && tile_tok0 && req_indptr) || (!tile_req && !tile_tok0 && tiles == tokens),
+               "attention: without a tile list every request brings one token (tiles %d, tokens %d)", tiles, tokens);
     const int group = heads / kv_heads;
     const int gcap = group < AT_ROWS ? group : AT_ROWS;
     TL_REQUIRE(tq * gcap <= AT_ROWS, "attention: tile of %d tokens x %d heads exceeds %d rows", tq, gcap, AT_ROWS);

@@ -395,16 +395,25 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
     ``ctx_lens[r] + i``.  ``window`` 0: all keys.  bfloat16 with pages of a multiple of 4
     tokens runs on the matrix cores; ``general=True`` forces the general kernel.  When the
     tiles cover only some of the step's tokens and ``splits > 1``, ``merge_tokens = (int32
-    indices of those tokens, their number)`` keeps the merge of the parts to their rows."""
+    indices of those tokens, their number)`` keeps the merge of the parts to their rows.
+    ``tile_req = tile_tok0 = None``: every request brings exactly one token, token ``i`` that of
+    request ``i`` (a decode step); the kernel then looks nothing up before it asks for the
+    request's length, block table and query."""
     T = q.shape[0]
     if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
         raise KernelError("paged_attention: q/out shapes or dtypes do not fit")
     _check_planes("paged_attention", k_plane, v_plane, q.dtype, num_kv_heads, page_size, head_dim)
-    for name, t in (("block_table", block_table), ("req_indptr", req_indptr), ("ctx_lens", ctx_lens),
-                    ("tile_req", tile_req), ("tile_tok0", tile_tok0)):
+    for name, t in (("block_table", block_table), ("ctx_lens", ctx_lens)):
         _i32(t, name)
-    if tile_req.numel() < num_tiles or tile_tok0.numel() < num_tiles:
-        raise KernelError("paged_attention: tile arrays shorter than the number of tiles")
+    if tile_req is None:        # every request brings one token: tile i is the token of request i
+        if tile_tok0 is not None or num_tiles != T or ctx_lens.numel() < T or block_table.shape[0] < T:
+            raise KernelError("paged_attention: without a tile list every request brings exactly one token")
+        req_indptr = None
+    else:
+        for name, t in (("req_indptr", req_indptr), ("tile_req", tile_req), ("tile_tok0", tile_tok0)):
+            _i32(t, name)
+        if tile_req.numel() < num_tiles or tile_tok0.numel() < num_tiles:
+            raise KernelError("paged_attention: tile arrays shorter than the number of tiles")
     if merge_tokens is not None:
         _i32(merge_tokens[0], "merge_tokens", merge_tokens[1])
     part_o = part_ml = None

@@ -174,6 +174,8 @@ class GQAttention(Mixer):
                                     self._splits(ctx, short[2], short[5]), merge_tokens=(short[3], short[4]))
         else:
             tile_req, tile_tok0, tiles = ctx.tiles(self.tile_tokens)
+            if ctx.decode_only and tiles == T:      # one token per request: no tile list to look up
+                tile_req = tile_tok0 = None
             ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
                                 tile_req, tile_tok0, tiles, self.tile_tokens, *common, self._splits(ctx, tiles))
         if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, self.q_width):

@@ -415,7 +415,10 @@ def test_projection_with_rotation_and_cache_write_in_its_epilogue(ops, M, nh, nk
     got = torch.full((T, width), float("nan"), dtype=torch.bfloat16, device="cuda")
     gk, gv = planes()
     fused = ops.linear_rope_cache_write(x, w, b, got, nh, nkv, hd, positions, inv_freq, token_req, bt, gk, gv, page)
-    assert fused
+    # from 9 rows on the library declines where the product split over K plus the rotation kernel is ahead
+    assert fused == (M <= 8 or not ops.linear_partials_pay(M, width, hidden))
+    if not fused:
+        return
     # against the exact product and rotation: the fused kernel rounds once, to bfloat16, at the end
     # (half an ulp, 2^-9 of the value; 2^-8 allowed), on top of the 32-bit sums' own error
     exact = x.double().cpu() @ w.double().cpu().T + (b.double().cpu() if bias else 0.0)

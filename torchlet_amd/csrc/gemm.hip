@@ -1250,6 +1250,8 @@ static void launch_skinny_rope(const void* x, const void* w, const void* bias, i
     kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo, 0, 0, ra);
 }
 
+extern "C" int tl_gemm_partials_pay(int M, int N, int K);
+
 extern "C" int tl_gemm_rope(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                             int ldx, int ldo, const void* positions, const void* inv_freq, const void* token_req,
                             const void* block_table, int bt_stride, void* k_plane, void* v_plane, int page,
@@ -1260,7 +1262,9 @@ extern "C" int tl_gemm_rope(const void* x, const void* w, const void* bias, int 
                "gemm_rope: the cache write needs both planes, the block table and the requests of the rows");
     TL_REQUIRE(N == (q_heads + (k_plane ? 2 * kv_heads : 0)) * head_dim, "gemm_rope: %d output columns do not match the heads", N);
     const int strips = (N + 15) / 16, ks = strips >= 1024 ? 16 : 8;
-    if (M > 16 || !skinny_fits(x, w, M, K, ldx) || N % 16 || ldo % 4 || ((uintptr_t)out % 8) || K / 64 / ks >= 16 ||
+    // (from 9 rows on the product split over K on the tile kernel plus the rotation kernel that adds its slabs up
+    // is ahead where that split is to be had: 4608 x 3584 at 16 rows 14.5 against 17.0 us, at 8 rows 14.8 against 14.0)
+    if (M > 16 || (M > 8 && tl_gemm_partials_pay(M, N, K)) || !skinny_fits(x, w, M, K, ldx) || N % 16 || ldo % 4 || ((uintptr_t)out % 8) || K / 64 / ks >= 16 ||
         (k_plane && (((uintptr_t)k_plane % 8) || head_dim % 4)))
         return TL_NOT_FUSED;
     RopeArgs ra;

@@ -443,6 +443,76 @@ def test_projection_with_rotation_and_cache_write_in_its_epilogue(ops, M, nh, nk
     assert torch.equal(q_only, got[:, : nh * hd])
 
 
+@pytest.mark.parametrize("H,I", [(96, 200), (3584, 1000), (1032, 300), (5120, 512), (8192, 96)])
+@pytest.mark.parametrize("pending", ["none", "row", "slabs"])
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
+def test_gate_up_product_of_one_row_that_makes_its_norm_itself(ops, H, I, pending, wdtype):
+    """``linear_swiglu_normed`` against the norm's own kernel followed by ``linear_swiglu``: the new
+    residual to the bit, the product within the rounding of one more order of summation."""
+    g = torch.Generator().manual_seed(H + I)
+    res = torch.randn(1, H, generator=g).cuda()
+    w = (1 + 0.1 * torch.randn(H, generator=g)).to(wdtype).cuda()
+    pend = {"none": None, "row": torch.randn(1, H, generator=g).to(torch.bfloat16).cuda(),
+            "slabs": torch.randn(3, 1, H, generator=g).cuda()}[pending]
+    gate = (torch.randn(I, H, generator=g) / math.sqrt(H)).to(torch.bfloat16).cuda()
+    up = (torch.randn(I, H, generator=g) / math.sqrt(H)).to(torch.bfloat16).cuda()
+    gu = ops.interleave_gate_up(gate, up)
+    r0, h = res.clone(), torch.empty(1, H, dtype=torch.bfloat16, device="cuda")
+    ops.add_rmsnorm(r0, pend, w, 1e-5, h)
+    z0 = torch.empty(1, I, dtype=torch.bfloat16, device="cuda")
+    ops.linear_swiglu(h, gu, z0)
+    z1 = torch.full((1, I), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rout = torch.full_like(res, float("nan"))
+    assert ops.linear_swiglu_normed(res, pend, w, 1e-5, rout, gu, z1)
+    assert torch.equal(rout, r0)
+    torch.testing.assert_close(z1.float(), z0.float(), **_tol(torch.bfloat16))
+    # what it is not built for it declines, leaving everything alone
+    long = torch.randn(1, 16384 + 64, generator=g).cuda()
+    gul = torch.zeros(64, 16384 + 64, dtype=torch.bfloat16, device="cuda")
+    zl = torch.empty(1, 32, dtype=torch.bfloat16, device="cuda")
+    assert not ops.linear_swiglu_normed(long, None, torch.ones(16384 + 64, dtype=wdtype, device="cuda"), 1e-5, torch.empty_like(long), gul, zl)
+    assert not ops.linear_swiglu_normed(torch.randn(2, H).cuda(), None, w, 1e-5, torch.empty(2, H).cuda(), gu, torch.empty(2, I, dtype=torch.bfloat16, device="cuda"))
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page,hidden,bias", [(28, 4, 128, 16, 3584, True), (4, 2, 16, 8, 64, False), (14, 2, 64, 16, 896, True),
+                                                        (40, 8, 128, 32, 5120, True), (5, 5, 48, 16, 240, True)])
+@pytest.mark.parametrize("pending", ["none", "row", "slabs"])
+def test_projection_of_one_row_that_makes_its_norm_itself(ops, nh, nkv, hd, page, hidden, bias, pending):
+    """``linear_rope_cache_write_normed`` against the norm's own kernel followed by the fused projection:
+    the new residual, the rotated queries and what lands in the pages, to the bit."""
+    g = torch.Generator().manual_seed(nh + hidden)
+    width = (nh + 2 * nkv) * hd
+    res = torch.randn(1, hidden, generator=g).cuda()
+    nw = (1 + 0.1 * torch.randn(hidden, generator=g)).to(torch.bfloat16).cuda()
+    pend = {"none": None, "row": torch.randn(1, hidden, generator=g).to(torch.bfloat16).cuda(),
+            "slabs": torch.randn(4, 1, hidden, generator=g).cuda()}[pending]
+    w = (torch.randn(width, hidden, generator=g) / math.sqrt(hidden)).to(torch.bfloat16).cuda()
+    b = torch.randn(width, generator=g).to(torch.bfloat16).cuda() if bias else None
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, hd, 2).float() / hd))).cuda()
+    pos = 77
+    positions = torch.tensor([pos], dtype=torch.int32).cuda()
+    token_req = torch.zeros(1, dtype=torch.int32).cuda()
+    blocks = pos // page + 1
+    bt = (torch.arange(blocks, dtype=torch.int32) + 1).view(1, blocks).cuda()
+
+    def planes():
+        return (torch.zeros(blocks + 1, nkv, page, hd, dtype=torch.bfloat16, device="cuda"),
+                torch.zeros(blocks + 1, nkv, hd, page, dtype=torch.bfloat16, device="cuda"))
+    r0, h = res.clone(), torch.empty(1, hidden, dtype=torch.bfloat16, device="cuda")
+    ops.add_rmsnorm(r0, pend, nw, 1e-6, h)
+    k0, v0 = planes()
+    q0 = torch.empty(1, width, dtype=torch.bfloat16, device="cuda")
+    assert ops.linear_rope_cache_write(h, w, b, q0, nh, nkv, hd, positions, inv_freq, token_req, bt, k0, v0, page)
+    k1, v1 = planes()
+    q1 = torch.full((1, width), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rout = torch.full_like(res, float("nan"))
+    assert ops.linear_rope_cache_write_normed(res, pend, nw, 1e-6, rout, w, b, q1, nh, nkv, hd, positions, inv_freq,
+                                              token_req, bt, k1, v1, page)
+    assert torch.equal(rout, r0)
+    assert torch.equal(q1[:, : nh * hd], q0[:, : nh * hd]) and torch.equal(k1, k0) and torch.equal(v1, v0)
+    assert float(k1[0].abs().sum()) == 0.0
+
+
 def _attention_ref(q, k, v, window):
     """One request: q [n, heads, hd] at positions ctx..ctx+n-1, k/v [ctx+n, kvh, hd] (float64)."""
     n, heads, hd = q.shape

@@ -252,11 +252,53 @@ struct RopeArgs {
     int bt_stride, page, q_heads, kv_heads, head_dim;
 };
 
-template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false, int D = 2, bool RP = false>
+// Eight neighbouring elements as floats, from float or bfloat16 memory and back.
+__device__ __forceinline__ void load8(const float* p, float* v) {
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float* v) {
+    const uint4 t = *(const uint4*)p;
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    v[4] = __uint_as_float(t.z << 16); v[5] = __uint_as_float(t.z & 0xffff0000u);
+    v[6] = __uint_as_float(t.w << 16); v[7] = __uint_as_float(t.w & 0xffff0000u);
+}
+__device__ __forceinline__ void store8(float* p, const float* v) {
+    *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+    *(float4*)(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float* v) {
+    uint4 t;
+    t.x = (uint32_t)from_float<bf16_t>(v[0]).bits | ((uint32_t)from_float<bf16_t>(v[1]).bits << 16);
+    t.y = (uint32_t)from_float<bf16_t>(v[2]).bits | ((uint32_t)from_float<bf16_t>(v[3]).bits << 16);
+    t.z = (uint32_t)from_float<bf16_t>(v[4]).bits | ((uint32_t)from_float<bf16_t>(v[5]).bits << 16);
+    t.w = (uint32_t)from_float<bf16_t>(v[6]).bits | ((uint32_t)from_float<bf16_t>(v[7]).bits << 16);
+    *(uint4*)p = t;
+}
+
+// NF (one row, with XL): x is not read but made here, as the norm of the residual stream would make it:
+// r = residual + pending (bfloat16, or float slabs of partial sums), x = r * rsqrt(mean(r^2) + eps) * weight, all
+// in 32-bit and rounded once; the first work-group writes r out as the new residual (to another place than it
+// is read from: the others may still be reading).  Every work-group does this once for all the strips it
+// walks, while its first weights are on their way; the norm's own kernel, a launch and a trip to memory with
+// nothing else to do, is not run at all (7B sizes, one row: 4.6 us twice a layer).
+struct NormArgs {
+    const float* residual;     // [K]
+    float* residual_out;       // [K]
+    const void* pending;       // bfloat16 [K], or float [parts][part_stride], or null
+    const void* weight;        // [K], bfloat16 or float
+    size_t part_stride;
+    int parts, weight_f32;
+    float eps;
+};
+
+template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false, int D = 2, bool RP = false, bool NF = false>
 __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                               const void* __restrict__ bias, int bias_f32,
                                                               TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-                                                              int out_cols, int k_per_split, RopeArgs ra) {
+                                                              int out_cols, int k_per_split, RopeArgs ra, NormArgs na) {
+    static_assert(!NF || (XL && MT == 1), "the fused norm makes x in shared memory, for one row");
     static_assert(!SW || (R == 1 && KS % 2 == 0), "the fused gate deals a work-group's waves to a gate strip and its up strip");
     static_assert(!RP || (R == 1 && MT == 1 && !SW), "the fused rotation is built for one strip and up to 16 rows");
     // Split K (k_per_split > 0, a multiple of 64): blockIdx.y owns the columns
@@ -327,7 +369,57 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
 #pragma unroll
     for (int d = 0; d < D; ++d)
         if (d < mine) SK_ISSUE(d, d)
-    if (XL) {                                  // the weights are on their way while x is copied
+    if (NF) {                                  // the weights are on their way while x is made
+        // a thread owns up to two pieces of eight elements (the host checked K <= 16 * threads)
+        const int pieces = K / 8;
+        float r[2][8];
+        float ss = 0.f;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int i = min((int)threadIdx.x + c * KS * 64, pieces - 1) * 8;
+            load8(na.residual + i, r[c]);
+            if (na.pending && na.parts == 0) {
+                float p[8];
+                load8((const bf16_t*)na.pending + i, p);
+#pragma unroll
+                for (int v = 0; v < 8; ++v) r[c][v] += p[v];
+            }
+            for (int q = 0; q < na.parts; ++q) {
+                float p[8];
+                load8((const float*)na.pending + q * na.part_stride + i, p);
+#pragma unroll
+                for (int v = 0; v < 8; ++v) r[c][v] += p[v];
+            }
+            if ((int)threadIdx.x + c * KS * 64 < pieces) {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) ss += r[c][v] * r[c][v];
+            }
+        }
+        ss = wave_sum(ss);
+        float* sums = red;                            // free until the first strip's sums
+        if (lane == 0) sums[wave] = ss;
+        lds_barrier();
+        float total = 0.f;
+        for (int wv = 0; wv < KS; ++wv) total += sums[wv];
+        const float inv = rsqrtf(total / (float)K + na.eps);
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int pc = (int)threadIdx.x + c * KS * 64;
+            if (pc < pieces) {
+                float g[8];
+                if (na.weight_f32) load8((const float*)na.weight + pc * 8, g);
+                else load8((const bf16_t*)na.weight + pc * 8, g);
+                float o[8];
+#pragma unroll
+                for (int v = 0; v < 8; ++v) o[v] = r[c][v] * inv * g[v];
+                store8(xs + pc * 8, o);
+                if (blockIdx.x == 0 && blockIdx.y == 0) {
+                    store8(na.residual_out + pc * 8, r[c]);
+                }
+            }
+        }
+        lds_barrier();
+    } else if (XL) {                           // the weights are on their way while x is copied
         const int pieces = K / 8;                     // 16-byte pieces per row
         for (int i = threadIdx.x; i < M * pieces; i += KS * 64) {
             const int row = i / pieces, pc = i % pieces;
@@ -530,11 +622,11 @@ static void launch_skinny_d(const void* x, const void* w, const void* bias, int 
         if (allowed == hipSuccess) {
             const int most = x_bytes <= SKINNY_XL_MAX_BYTES ? 512 : 256;      // a larger x leaves room for one work-group only
             dim3 few(strips < most ? strips : most);
-            kernel<<<few, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{});
+            kernel<<<few, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{}, NormArgs{});
             return;
         }
     }
-    gemm_skinny_kernel<R, MT, KS, TOut, SW, false, D><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{});
+    gemm_skinny_kernel<R, MT, KS, TOut, SW, false, D><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{}, NormArgs{});
 }
 
 // A wave with many K steps ahead of it (a long K: the down projection) keeps as many in flight as
@@ -1247,7 +1339,7 @@ static void launch_skinny_rope(const void* x, const void* w, const void* bias, i
     const size_t lds = (size_t)KS * 1024 + (XL ? (size_t)M * (K + 8) * 2 : 0);
     auto kernel = gemm_skinny_kernel<1, 1, KS, bf16_t, false, XL, 2, true>;
     if (XL) { static hipError_t allowed = allow_lds(kernel, 96 * 1024); (void)allowed; }
-    kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo, 0, 0, ra);
+    kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo, 0, 0, ra, NormArgs{});
 }
 
 extern "C" int tl_gemm_partials_pay(int M, int N, int K);
@@ -1275,6 +1367,75 @@ extern "C" int tl_gemm_rope(const void* x, const void* w, const void* bias, int 
     if (ks == 8) { if (xl) launch_skinny_rope<8, true>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); else launch_skinny_rope<8, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); }
     else { if (xl) launch_skinny_rope<16, true>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); else launch_skinny_rope<16, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); }
     TL_CHECK_LAUNCH("gemm_rope");
+    return TL_OK;
+}
+
+// What a fused norm needs to be right: whole 16-byte pieces everywhere, two pieces per thread at most.
+static bool norm_fits(const NormArgs& na, int K, int threads) {
+    return K % 8 == 0 && K <= 16 * threads && na.residual && na.residual_out && na.residual != na.residual_out && na.weight &&
+           ((uintptr_t)na.residual % 16) == 0 && ((uintptr_t)na.residual_out % 16) == 0 && ((uintptr_t)na.weight % 16) == 0 &&
+           ((uintptr_t)na.pending % 16) == 0 && (na.parts == 0 || na.part_stride % 4 == 0) && na.parts >= 0 && na.parts <= 64;
+}
+
+static NormArgs norm_args(const void* residual, void* residual_out, const void* pending, int parts, long part_stride,
+                          const void* weight, int weight_f32, float eps) {
+    NormArgs na;
+    na.residual = (const float*)residual; na.residual_out = (float*)residual_out; na.pending = pending;
+    na.weight = weight; na.part_stride = (size_t)part_stride; na.parts = parts; na.weight_f32 = weight_f32; na.eps = eps;
+    return na;
+}
+
+// tl_gemm_rope for one row whose x is the norm of the residual stream, made inside the kernel (see NormArgs):
+// pending is bfloat16 [K] (parts == 0), float [parts][part_stride] or null.  Returns TL_NOT_FUSED (nothing
+// launched) for shapes it is not built for; the caller then runs the norm and tl_gemm_rope.
+extern "C" int tl_gemm_rope_normed(const void* residual, void* residual_out, const void* pending, int parts, long part_stride,
+                                   const void* norm_weight, int norm_weight_f32, float eps,
+                                   const void* w, const void* bias, int bias_f32, void* out, int N, int K, int ldo,
+                                   const void* positions, const void* inv_freq, const void* token_req,
+                                   const void* block_table, int bt_stride, void* k_plane, void* v_plane, int page,
+                                   int q_heads, int kv_heads, int head_dim, hipStream_t stream) {
+    TL_REQUIRE(N > 0 && K > 0 && ldo >= q_heads * head_dim, "gemm_rope_normed: bad sizes N=%d K=%d", N, K);
+    TL_REQUIRE(positions && inv_freq && head_dim % 4 == 0 && q_heads >= 0 && kv_heads >= 0, "gemm_rope_normed: needs positions, frequencies and a head size that is a multiple of 4");
+    TL_REQUIRE((k_plane == nullptr) == (v_plane == nullptr) && (!k_plane || (token_req && block_table && page > 0 && bt_stride > 0)),
+               "gemm_rope_normed: the cache write needs both planes, the block table and the request of the row");
+    TL_REQUIRE(N == (q_heads + (k_plane ? 2 * kv_heads : 0)) * head_dim, "gemm_rope_normed: %d output columns do not match the heads", N);
+    const NormArgs na = norm_args(residual, residual_out, pending, parts, part_stride, norm_weight, norm_weight_f32, eps);
+    const int strips = (N + 15) / 16, ks = strips >= 1024 ? 16 : 8;
+    if (!norm_fits(na, K, ks * 64) || ((uintptr_t)w % 16) || N % 16 || ldo % 4 || ((uintptr_t)out % 8) || K / 64 / ks >= 16 ||
+        (k_plane && (((uintptr_t)k_plane % 8) || head_dim % 4)))
+        return TL_NOT_FUSED;
+    RopeArgs ra;
+    ra.positions = (const int*)positions; ra.inv_freq = (const float*)inv_freq; ra.token_req = (const int*)token_req;
+    ra.block_table = (const int*)block_table; ra.k_plane = (bf16_t*)k_plane; ra.v_plane = (bf16_t*)v_plane;
+    ra.bt_stride = bt_stride; ra.page = page > 0 ? page : 1; ra.q_heads = q_heads; ra.kv_heads = k_plane ? kv_heads : 0; ra.head_dim = head_dim;
+    dim3 grid(strips);
+    const size_t lds = (size_t)ks * 1024 + (size_t)(K + 8) * 2;
+    if (ks == 8)
+        gemm_skinny_kernel<1, 1, 8, bf16_t, false, true, 2, true, true><<<grid, dim3(8 * 64), lds, stream>>>(
+            nullptr, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, 1, N, K, K, ldo, 0, 0, ra, na);
+    else
+        gemm_skinny_kernel<1, 1, 16, bf16_t, false, true, 2, true, true><<<grid, dim3(16 * 64), lds, stream>>>(
+            nullptr, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, 1, N, K, K, ldo, 0, 0, ra, na);
+    TL_CHECK_LAUNCH("gemm_rope_normed");
+    return TL_OK;
+}
+
+// tl_gemm_swiglu for one row whose x is the norm of the residual stream, made inside the kernel.  Returns
+// TL_NOT_FUSED (nothing launched) for shapes it is not built for.
+extern "C" int tl_gemm_swiglu_normed(const void* residual, void* residual_out, const void* pending, int parts, long part_stride,
+                                     const void* norm_weight, int norm_weight_f32, float eps,
+                                     const void* w, void* out, int I, int K, hipStream_t stream) {
+    TL_REQUIRE(I > 0 && K > 0, "gemm_swiglu_normed: bad sizes I=%d K=%d", I, K);
+    const NormArgs na = norm_args(residual, residual_out, pending, parts, part_stride, norm_weight, norm_weight_f32, eps);
+    const int N = ((I + 31) / 32) * 64;          // rows of the interleaved matrix
+    if (!norm_fits(na, K, 16 * 64) || ((uintptr_t)w % 16) || K / 64 / 16 >= 16)
+        return TL_NOT_FUSED;
+    const int strips = N / 32;
+    dim3 grid(strips < 512 ? strips : 512);       // every work-group makes x once and walks its strips
+    const size_t lds = (size_t)16 * 1024 + (size_t)(K + 8) * 2;
+    gemm_skinny_kernel<1, 1, 16, bf16_t, true, true, 2, false, true><<<grid, dim3(16 * 64), lds, stream>>>(
+        nullptr, (const bf16_t*)w, nullptr, 0, (bf16_t*)out, 1, N, K, K, I, I, 0, RopeArgs{}, na);
+    TL_CHECK_LAUNCH("gemm_swiglu_normed");
     return TL_OK;
 }
 
@@ -1393,14 +1554,14 @@ extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, 
     dim3 grid((N + 63) / 64, P), block(8 * 64);
     const size_t red_bytes = (size_t)8 * 4 * (M <= 16 ? 1 : (M <= 32 ? 2 : 4)) * 1024;
     if (M <= 16)
-        gemm_skinny_kernel<4, 1, 8, float, false, false, skinny_depth<4, 1, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{});
+        gemm_skinny_kernel<4, 1, 8, float, false, false, skinny_depth<4, 1, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{}, NormArgs{});
     else if (M <= 32)
-        gemm_skinny_kernel<4, 2, 8, float, false, false, skinny_depth<4, 2, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{});
+        gemm_skinny_kernel<4, 2, 8, float, false, false, skinny_depth<4, 2, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{}, NormArgs{});
     else {
         auto kernel = gemm_skinny_kernel<4, 4, 8, float, false, false, skinny_depth<4, 4, 8>()>;
         static hipError_t allowed = allow_lds(kernel, 128 * 1024);
         TL_REQUIRE(allowed == hipSuccess, "gemm_partials: cannot get %zu bytes of shared memory", red_bytes);
-        kernel<<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{});
+        kernel<<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{}, NormArgs{});
     }
     TL_CHECK_LAUNCH("gemm_partials");
     return TL_OK;

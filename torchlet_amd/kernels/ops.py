@@ -365,6 +365,86 @@ def linear_rope_cache_write(x: torch.Tensor, weight: torch.Tensor, bias: torch.T
     return True
 
 
+def _norm_args(what: str, residual: torch.Tensor, pending: torch.Tensor | None, weight: torch.Tensor, eps: float,
+               residual_out: torch.Tensor):
+    """The arguments that describe ``norm(residual + pending)`` of one row to a kernel that makes it itself."""
+    H = residual.shape[-1]
+    if residual.dtype != torch.float32 or residual_out.dtype != torch.float32 or residual.numel() != H or residual_out.numel() != H \
+            or not residual.is_contiguous() or not residual_out.is_contiguous():
+        raise KernelError(f"{what}: the residual and its successor must be one contiguous float32 row")
+    parts = part_stride = 0
+    if pending is not None:
+        if pending.dim() == 3:
+            if pending.dtype != torch.float32 or pending.shape[1:] != (1, H) or not pending.is_contiguous():
+                raise KernelError(f"{what}: partial sums {pending.dtype} {tuple(pending.shape)} are not float32 [P, 1, {H}]")
+            parts, part_stride = pending.shape[0], pending.stride(0)
+        elif pending.dtype != torch.bfloat16 or pending.numel() != H or not pending.is_contiguous():
+            raise KernelError(f"{what}: pending {pending.dtype} {tuple(pending.shape)} is not a bfloat16 row of {H}")
+    wf = _vec(weight, H, f"{what} norm weight")
+    return (_ptr(residual), _ptr(residual_out), _ptr(pending), c_int(parts), ctypes.c_long(part_stride), _ptr(weight), c_int(wf),
+            c_float(eps))
+
+
+def linear_rope_cache_write_normed(residual: torch.Tensor, pending: torch.Tensor | None, norm_weight: torch.Tensor, eps: float,
+                                   residual_out: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
+                                   out: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int, positions: torch.Tensor,
+                                   inv_freq: torch.Tensor, token_req: torch.Tensor | None = None,
+                                   block_table: torch.Tensor | None = None, k_plane: torch.Tensor | None = None,
+                                   v_plane: torch.Tensor | None = None, page_size: int = 0) -> bool:
+    """:func:`linear_rope_cache_write` for ONE row whose input is ``norm(residual + pending)`` (see
+    :func:`add_rmsnorm`), made inside the kernel: ``residual [1, K]`` float32, ``pending`` bfloat16
+    ``[1, K]``, float32 slabs ``[P, 1, K]`` or ``None``; the sum goes to ``residual_out`` (another
+    tensor than ``residual``).  Returns ``False`` without doing anything for shapes it is not built for."""
+    K = residual.shape[-1]
+    N = weight.shape[0]
+    if weight.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or residual.shape[0] != 1:
+        return False
+    if out.stride(1) != 1 or not weight.is_contiguous() or weight.shape[1] != K or out.shape[0] != 1:
+        raise KernelError("linear_rope_cache_write_normed: shapes or strides do not fit")
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() != head_dim // 2:
+        raise KernelError("linear_rope_cache_write_normed: inv_freq must be float32 [head_dim/2]")
+    _i32(positions, "positions", 1)
+    bt_stride = 0
+    if k_plane is not None:
+        _i32(token_req, "token_req", 1)
+        _i32(block_table, "block_table")
+        bt_stride = block_table.stride(0)
+        _check_planes("linear_rope_cache_write_normed", k_plane, v_plane, torch.bfloat16, kv_heads, page_size, head_dim)
+    if N != (q_heads + (2 * kv_heads if k_plane is not None else 0)) * head_dim or out.shape[1] < q_heads * head_dim:
+        raise KernelError("linear_rope_cache_write_normed: the projection's rows do not match the heads")
+    bf = _vec(bias, N, "linear bias")
+    lib = _lib("gemm")
+    rc = lib.tl_gemm_rope_normed(*_norm_args("linear_rope_cache_write_normed", residual, pending, norm_weight, eps, residual_out),
+                                 _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(N), c_int(K), c_int(out.stride(0)),
+                                 _ptr(positions), _ptr(inv_freq), _ptr(token_req), _ptr(block_table), c_int(bt_stride),
+                                 _ptr(k_plane), _ptr(v_plane), c_int(page_size), c_int(q_heads), c_int(kv_heads),
+                                 c_int(head_dim), _stream())
+    if rc == 100:          # not built for this shape
+        return False
+    _check(lib, rc)
+    return True
+
+
+def linear_swiglu_normed(residual: torch.Tensor, pending: torch.Tensor | None, norm_weight: torch.Tensor, eps: float,
+                         residual_out: torch.Tensor, gate_up: torch.Tensor, out: torch.Tensor) -> bool:
+    """:func:`linear_swiglu` for ONE row whose input is ``norm(residual + pending)``, made inside the
+    kernel (see :func:`linear_rope_cache_write_normed`).  Returns ``False`` without doing anything
+    for shapes it is not built for."""
+    K = residual.shape[-1]
+    I = out.shape[1]
+    if gate_up.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or residual.shape[0] != 1:
+        return False
+    if gate_up.shape != (-(-I // 32) * 64, K) or out.shape[0] != 1 or not gate_up.is_contiguous() or not out.is_contiguous():
+        raise KernelError(f"linear_swiglu_normed: shapes w{tuple(gate_up.shape)} out{tuple(out.shape)} do not fit a row of {K}")
+    lib = _lib("gemm")
+    rc = lib.tl_gemm_swiglu_normed(*_norm_args("linear_swiglu_normed", residual, pending, norm_weight, eps, residual_out),
+                                   _ptr(gate_up), _ptr(out), c_int(I), c_int(K), _stream())
+    if rc == 100:
+        return False
+    _check(lib, rc)
+    return True
+
+
 def _check_planes(what, k_plane, v_plane, dtype, kv_heads, page_size, head_dim) -> None:
     for p, shape in ((k_plane, (kv_heads, page_size, head_dim)), (v_plane, (kv_heads, head_dim, page_size))):
         if p.dtype != dtype or p.dim() != 4 or tuple(p.shape[1:]) != shape or not p.is_contiguous():

@@ -17,7 +17,7 @@ import torch
 
 from ..config.base import ConfigError
 from ..kernels import ops
-from .base import MIXERS, POSITION_ENCODINGS, Mixer, PagedNeed, WeightSpec
+from .base import MIXERS, POSITION_ENCODINGS, LazyNorm, Mixer, PagedNeed, WeightSpec
 
 _TARGET_WORKGROUPS = 512     # enough work-groups to fill 256 compute units twice
 _MIN_KEYS_PER_SPLIT = 256
@@ -111,13 +111,17 @@ class GQAttention(Mixer):
         by_keys = max(1, longest // _MIN_KEYS_PER_SPLIT)
         return max(1, min(by_fill, by_keys, 64))
 
+    takes_lazy_norm = True
+
     def forward(self, h, ctx, cache):
-        T = h.shape[0]
+        lazy = h if isinstance(h, LazyNorm) else None      # one row whose norm the projection's kernel can make itself
+        device = lazy.residual.device if lazy is not None else h.device
+        T = 1 if lazy is not None else h.shape[0]
         writes = cache.writable
         width = self.q_width + (2 * self.kv_width if writes else 0)
         w = self.w_qkv if writes else self.w_qkv[: self.q_width]
         b = self.b_qkv if (self.b_qkv is None or writes) else self.b_qkv[: self.q_width]
-        qkv = torch.empty((T, width), dtype=self.dtype, device=h.device)
+        qkv = torch.empty((T, width), dtype=self.dtype, device=device)
 
         # the cache hands out two planes of [pages, kv_heads, page, head_dim]; this mixer keeps the
         # values of a page transposed, [kv_heads, head_dim, page], as its kernels read them
@@ -127,8 +131,19 @@ class GQAttention(Mixer):
         kv_heads = self.kv_heads if writes else 0
         inv_freq = self.position.fused_inv_freq() if hasattr(self.position, "fused_inv_freq") else None
         cache_args = (ctx.token_req, table, k_plane, v_plane, cache.page_size) if writes else (None, None, None, None, 0)
-        fused = self.pair_layout and ops.linear_rope_cache_write(h, w, b, qkv, self.heads, self.kv_heads, self.head_dim,
-                                                                 ctx.positions, inv_freq, *cache_args)
+        fused = False
+        if lazy is not None:
+            if self.pair_layout:
+                residual_out = torch.empty_like(lazy.residual)
+                fused = ops.linear_rope_cache_write_normed(lazy.residual, lazy.pending, lazy.norm.weight, lazy.norm.eps,
+                                                           residual_out, w, b, qkv, self.heads, self.kv_heads, self.head_dim,
+                                                           ctx.positions, inv_freq, *cache_args)
+                if fused:
+                    lazy.done(residual_out)
+            if not fused:
+                h = lazy.value()
+        fused = fused or (self.pair_layout and ops.linear_rope_cache_write(h, w, b, qkv, self.heads, self.kv_heads, self.head_dim,
+                                                                           ctx.positions, inv_freq, *cache_args))
         if not fused and self.dtype == torch.bfloat16 and (inv_freq is not None or self.position is None) \
                 and ops.linear_partials_pay(T, width, self.hidden):
             # few rows against a narrow matrix: K split over work-groups; the rotation kernel adds the slabs up
@@ -144,7 +159,7 @@ class GQAttention(Mixer):
                 ops.rope_cache_write(qkv, self.heads, kv_heads, self.head_dim, self.heads + kv_heads, ctx.positions, inv_freq,
                                      *cache_args, pairs=self.pair_layout)
 
-        out = torch.empty((T, self.q_width), dtype=self.dtype, device=h.device)
+        out = torch.empty((T, self.q_width), dtype=self.dtype, device=device)
         q = qkv[:, : self.q_width]
         common = (self.heads, self.kv_heads, self.head_dim, cache.page_size, self.window or 0, self.scale)
         rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size, -(-ctx.max_total_len // cache.page_size))
@@ -181,6 +196,6 @@ class GQAttention(Mixer):
         if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, self.q_width):
             # few rows against a narrow matrix: K split over work-groups; the next norm adds the slabs up
             return ops.linear_partials(out, self.w_o)
-        y = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
+        y = torch.empty((T, self.hidden), dtype=self.dtype, device=device)
         ops.linear(out, self.w_o, None, y)
         return y

@@ -108,6 +108,36 @@ class Stream:
         self.pending = pending
 
 
+class LazyNorm:
+    """A norm that has not run yet, handed to the part that reads its output: ``norm(residual + pending)`` of
+    the stream, described by what a kernel needs to make it itself (``residual``, ``pending``, ``weight``,
+    ``eps``).  A consumer whose kernel did so calls :meth:`done` with the new residual it wrote; any other
+    calls :meth:`value`, which runs the norm the usual way (once).  The norm's own kernel is a launch and a
+    trip to memory that a step of one token can do without."""
+
+    def __init__(self, norm, stream: "Stream"):
+        self.norm = norm
+        self.stream = stream
+        self._value = None
+
+    @property
+    def residual(self):
+        return self.stream.residual
+
+    @property
+    def pending(self):
+        return self.stream.pending
+
+    def value(self) -> torch.Tensor:
+        if self._value is None:
+            self._value = self.norm.forward(self.stream)
+        return self._value
+
+    def done(self, residual_out: torch.Tensor) -> None:
+        self.stream.residual = residual_out
+        self.stream.pending = None
+
+
 # ----------------------------------------------------------------------- part kinds
 
 class Norm(Part):
@@ -116,6 +146,11 @@ class Norm(Part):
         return ``norm(residual)`` in the activation dtype.  With ``rows`` (int32 indices)
         only those rows are read and returned, and the stream is left untouched."""
         raise NotImplementedError
+
+    def lazy(self, stream: Stream) -> "LazyNorm | None":
+        """A :class:`LazyNorm` of the stream where a consumer's kernel could make this norm itself (the
+        norm says for which steps that is worth offering), else ``None``."""
+        return None
 
 
 class PositionEncoding(Part):

@@ -34,8 +34,9 @@ class PreNormBlock(Block):
             part.load_weights({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
 
     def forward(self, stream: Stream, ctx, cache) -> Stream:
-        h = self.mixer_norm.forward(stream)
+        # a part that says it takes a norm that has not run yet (``takes_lazy_norm``) may get one, see LazyNorm
+        h = (self.mixer_norm.lazy(stream) if getattr(self.mixer, "takes_lazy_norm", False) else None) or self.mixer_norm.forward(stream)
         stream.pending = self.mixer.forward(h, ctx, cache)
-        h = self.ffn_norm.forward(stream)
+        h = (self.ffn_norm.lazy(stream) if getattr(self.ffn, "takes_lazy_norm", False) else None) or self.ffn_norm.forward(stream)
         stream.pending = self.ffn.forward(h, ctx)
         return stream

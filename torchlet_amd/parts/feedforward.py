@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import FEED_FORWARDS, FeedForward, WeightSpec
+from .base import FEED_FORWARDS, FeedForward, LazyNorm, WeightSpec
 
 
 # The down product returns partial sums over slices of K where the kernel library finds that it
@@ -47,7 +47,20 @@ class SwiGLU(FeedForward):
             self.gate_up = self._place(torch.cat((tensors["gate_proj.weight"], tensors["up_proj.weight"]), dim=0), "matrix")
         self.down = self._place(tensors["down_proj.weight"], "matrix")
 
+    takes_lazy_norm = True
+
     def forward(self, h, ctx):
+        lazy = h if isinstance(h, LazyNorm) else None
+        if lazy is not None:
+            # one row: the gate/up kernel makes the norm itself while its first weights arrive
+            if self.fused_gate:
+                z = torch.empty((1, self.inter), dtype=self.dtype, device=lazy.residual.device)
+                residual_out = torch.empty_like(lazy.residual)
+                if ops.linear_swiglu_normed(lazy.residual, lazy.pending, lazy.norm.weight, lazy.norm.eps, residual_out,
+                                            self.gate_up, z):
+                    lazy.done(residual_out)
+                    return self._down(z, 1)
+            h = lazy.value()
         T = h.shape[0]
         z = torch.empty((T, self.inter), dtype=self.dtype, device=h.device)
         if self.fused_gate:
@@ -56,9 +69,12 @@ class SwiGLU(FeedForward):
             gu = torch.empty((T, 2 * self.inter), dtype=self.dtype, device=h.device)
             ops.linear(h, self.gate_up, None, gu)
             ops.swiglu(gu, z)
+        return self._down(z, T)
+
+    def _down(self, z, T):
         if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, self.inter):
             # few rows, long K, narrow matrix: split K over work-groups; the next norm adds the slabs up
             return ops.linear_partials(z, self.down)
-        y = torch.empty((T, self.hidden), dtype=self.dtype, device=h.device)
+        y = torch.empty((T, self.hidden), dtype=self.dtype, device=z.device)
         ops.linear(z, self.down, None, y)
         return y

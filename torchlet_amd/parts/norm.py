@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import NORMS, Norm, Stream, WeightSpec
+from .base import NORMS, LazyNorm, Norm, Stream, WeightSpec
 
 
 @NORMS.register("rmsnorm")
@@ -34,3 +34,9 @@ class RMSNorm(Norm):
         if rows is None:
             stream.pending = None
         return out
+
+    def lazy(self, stream: Stream) -> LazyNorm | None:
+        # one row in bfloat16: the kernels that read the norm's output can make it while their weights arrive
+        if self.dtype == torch.bfloat16 and stream.residual.shape[0] == 1 and stream.residual.is_cuda:
+            return LazyNorm(self, stream)
+        return None

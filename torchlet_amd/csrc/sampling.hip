@@ -6,6 +6,8 @@
 // of the row's 32-bit key and the index i, so a draw depends on nothing but (key, logits):
 // not on the batch, the row's place in it, or the grid.
 #include "common.h"
+#include "sampling.h"
+#include <mutex>
 
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
     x ^= x >> 16; x *= 0x7feb352du;
@@ -82,7 +84,22 @@ __global__ __launch_bounds__(TL_WAVE) void sample_pick_kernel(const float* __res
 // Chunks a row of `vocab` columns is scanned in: about a thousand columns each, 128 at most.
 extern "C" int tl_sample_chunks(int vocab) {
     const int c = (vocab + 1023) / 1024;
-    return c < 1 ? 1 : (c > 128 ? 128 : c);
+    return c < 1 ? 1 : (c > TL_SAMPLE_MAX_CHUNKS ? TL_SAMPLE_MAX_CHUNKS : c);
+}
+
+// Both stages; `candidates` holds rows * chunks floats, then rows * chunks ints.
+static int launch_sample(const void* logits, int rows, int vocab, int ld, const void* temperature, const void* keys,
+                         void* out, void* candidates, hipStream_t stream) {
+    const int chunks = tl_sample_chunks(vocab);
+    const int per = (vocab + chunks - 1) / chunks;
+    float* part_v = (float*)candidates;
+    int* part_i = (int*)candidates + (size_t)rows * chunks;
+    sample_scan_kernel<<<dim3(chunks, rows), dim3(SAMPLE_THREADS), 0, stream>>>((const float*)logits, vocab, ld, per,
+        (const float*)temperature, (const int*)keys, part_v, part_i);
+    TL_CHECK_LAUNCH("sample_scan");
+    sample_pick_kernel<<<dim3(rows), dim3(TL_WAVE), 0, stream>>>(part_v, part_i, chunks, vocab, (int*)out);
+    TL_CHECK_LAUNCH("sample_pick");
+    return TL_OK;
 }
 
 // temperature: float[rows] or null (all greedy); keys: int32[rows] bit patterns or null.
@@ -92,14 +109,52 @@ extern "C" int tl_sample(const void* logits, int rows, int vocab, int ld, const 
     TL_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "sample: bad sizes rows=%d vocab=%d ld=%d", rows, vocab, ld);
     TL_REQUIRE(scratch != nullptr || rows == 0, "sample: no scratch buffer");
     if (rows == 0) return TL_OK;
-    const int chunks = tl_sample_chunks(vocab);
-    const int per = (vocab + chunks - 1) / chunks;
-    float* part_v = (float*)scratch;
-    int* part_i = (int*)scratch + (size_t)rows * chunks;
-    sample_scan_kernel<<<dim3(chunks, rows), dim3(SAMPLE_THREADS), 0, stream>>>((const float*)logits, vocab, ld, per,
-        (const float*)temperature, (const int*)keys, part_v, part_i);
-    TL_CHECK_LAUNCH("sample_scan");
-    sample_pick_kernel<<<dim3(rows), dim3(TL_WAVE), 0, stream>>>(part_v, part_i, chunks, vocab, (int*)out);
-    TL_CHECK_LAUNCH("sample_pick");
+    return launch_sample(logits, rows, vocab, ld, temperature, keys, out, scratch, stream);
+}
+
+// ---------------------------------------------------------------- the entry point that allocates nothing
+// The candidates' array of tl_sample_static, held by the library on every GPU it runs on.  In host code
+// this name is only a stand-in for the symbol: the array's address on a GPU comes from
+// hipGetSymbolAddress, asked once per device with that device current, and is what kernels are given.
+static __device__ __align__(256) unsigned char scratch[(size_t)TL_SAMPLE_STATIC_MAX_ROWS * TL_SAMPLE_MAX_CHUNKS * 8];
+
+#define TL_MAX_DEVICES 64
+static void* scratch_of_device[TL_MAX_DEVICES];      // null: not asked for yet
+static std::mutex scratch_mutex;
+
+// The address of `scratch` on the device that is current in this thread.
+static int scratch_here(void** address) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) {
+        tl_set_error("sample_static: hipGetDevice failed: %s", hipGetErrorString(e));
+        return TL_ERR_HIP;
+    }
+    TL_REQUIRE(device >= 0 && device < TL_MAX_DEVICES, "sample_static: device %d is beyond the %d this library keeps track of",
+               device, TL_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_of_device[device] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            tl_set_error("sample_static: hipGetSymbolAddress failed on device %d: %s", device, hipGetErrorString(e));
+            return TL_ERR_HIP;
+        }
+        scratch_of_device[device] = ptr;
+    }
+    *address = scratch_of_device[device];
     return TL_OK;
+}
+
+extern "C" int tl_sample_static(const void* logits, int rows, int vocab, int ld, const void* temperature,
+                                const void* keys, void* out, hipStream_t stream) {
+    TL_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "sample_static: bad sizes rows=%d vocab=%d ld=%d", rows, vocab, ld);
+    TL_REQUIRE(rows <= TL_SAMPLE_STATIC_MAX_ROWS, "sample_static: %d rows, but the library's own array holds the candidates of %d at most",
+               rows, TL_SAMPLE_STATIC_MAX_ROWS);
+    if (rows == 0) return TL_OK;
+    TL_REQUIRE(logits != nullptr && out != nullptr, "sample_static: logits and out must be given");
+    void* ptr = nullptr;
+    const int rc = scratch_here(&ptr);
+    if (rc != TL_OK) return rc;
+    return launch_sample(logits, rows, vocab, ld, temperature, keys, out, ptr, stream);
 }

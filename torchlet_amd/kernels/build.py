@@ -28,7 +28,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-HEADERS = ["common.h"]
+HEADERS = sorted(p.name for p in CSRC.glob("*.h"))      # every header is part of every library's stamp
 
 # head sizes compiled by build_all(): what the tests, the smoke run and the benchmark use
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)

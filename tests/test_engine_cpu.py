@@ -250,3 +250,38 @@ def test_shutdown_gives_up_unfinished_requests_and_frees_their_pages(cpu_ops, mo
     engine.add_request(again)
     engine.run_until_done()
     assert len(again.output_tokens) == 2
+
+
+def test_requests_are_added_all_or_none(cpu_ops, model_folders):
+    """A call that brings one bad request leaves nothing waiting (``LLM.generate`` adds through this)."""
+    engine = Engine(runner_for(model_folders["A"], "A"), max_tokens_per_step=24)
+    good = Request(prompt_tokens=[1, 2, 3], max_new_tokens=4)
+    for bad in (Request(prompt_tokens=[1] * 126, max_new_tokens=4),        # passes max_position_embeddings (128)
+                Request(prompt_tokens=[1, 256], max_new_tokens=4),         # outside the vocabulary
+                Request(prompt_tokens=[], max_new_tokens=4)):
+        with pytest.raises(ValueError):
+            engine.add_requests([good, bad])
+        assert not engine.has_work()
+    engine.add_requests([good])
+    assert engine.has_work()
+    engine.run_until_done()
+    assert len(good.output_tokens) == 4 and engine.runner.cache.live_requests() == []
+
+
+def test_chat_template_runs_in_a_sandbox():
+    import jinja2
+
+    from torchlet_amd.llm import render_chat_template
+
+    ok = "{% for m in messages %}<|im_start|>{{ m['role'] }}\n{{ m['content'] }}<|im_end|>\n{% endfor %}" \
+         "{% if add_generation_prompt %}<|im_start|>assistant\n{% endif %}"
+    assert render_chat_template(ok, "hi") == "<|im_start|>user\nhi<|im_end|>\n<|im_start|>assistant\n"
+    for evil in ("{{ messages.__class__.__mro__ }}", "{{ ''.__class__.__base__.__subclasses__() }}",
+                 "{% set _ = messages.append(1) %}"):
+        with pytest.raises(jinja2.exceptions.SecurityError):
+            render_chat_template(evil, "hi")
+    assert render_chat_template("{{ raise_exception.__globals__ }}", "hi") == ""      # a function's globals: not there
+    with pytest.raises(jinja2.exceptions.UndefinedError):
+        render_chat_template("{{ raise_exception.__globals__['__builtins__'] }}", "hi")
+    with pytest.raises(jinja2.exceptions.TemplateError, match="no system turn"):
+        render_chat_template("{{ raise_exception('no system turn') }}", "hi")

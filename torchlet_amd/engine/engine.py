@@ -47,11 +47,25 @@ class Engine:
         self.steps_ahead = 0              # steps that were enqueued before their tokens were known
         self._ahead: _Launched | None = None
 
-    def add_request(self, req: Request) -> None:
+    def validate(self, req: Request) -> None:
+        """Raise ``ValueError`` for a request that could never run (the scheduler's rules, and token ids
+        outside the vocabulary); nothing is kept of it."""
         bad = [t for t in req.prompt_tokens if not 0 <= t < self.runner.vocab_size]
         if bad:
             raise ValueError(f"request {req.req_id}: token id {bad[0]} outside the vocabulary of {self.runner.vocab_size}")
+        self.scheduler.validate(req)
+
+    def add_request(self, req: Request) -> None:
+        self.validate(req)
         self.scheduler.add_request(req)
+
+    def add_requests(self, reqs: list[Request]) -> None:
+        """All of them or none: every request is checked before the first one is queued, so a call that
+        fails leaves nothing waiting."""
+        for r in reqs:
+            self.validate(r)
+        for r in reqs:
+            self.scheduler.add_request(r)
 
     def has_work(self) -> bool:
         return self.scheduler.has_work()

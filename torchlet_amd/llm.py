@@ -99,8 +99,7 @@ class LLM:
         if max_new_tokens <= 0:
             return ["" if isinstance(x, str) else [] for x in inputs]
         reqs = self._requests(inputs, max_new_tokens, temperature, seed, stop_token_ids)
-        for r in reqs:
-            self.engine.add_request(r)
+        self.engine.add_requests(reqs)          # all or none: a bad request leaves nothing queued
         self.engine.run_until_done()
         return self._outputs(inputs, reqs)
 
@@ -112,8 +111,7 @@ class LLM:
         if max_new_tokens <= 0:
             return ["" if isinstance(x, str) else [] for x in inputs]
         reqs = self._requests(inputs, max_new_tokens, kw.get("temperature", 0.0), kw.get("seed"), kw.get("stop_token_ids"))
-        for r in reqs:
-            self.engine.add_request(r)
+        self.engine.add_requests(reqs)
         while any(r.finish_reason is None for r in reqs):
             try:
                 self.engine.step()
@@ -161,18 +159,30 @@ class _Tokenizer:
         return ids
 
     def encode_chat(self, user_text: str):
-        if self.template:
-            import jinja2
-            env = jinja2.Environment(trim_blocks=True, lstrip_blocks=True)
-            text = env.from_string(self.template).render(
-                messages=[{"role": "user", "content": user_text}], add_generation_prompt=True,
-                bos_token=self._token_text("bos_token") or "", eos_token=self._token_text("eos_token") or "")
-        else:
-            text = user_text
+        text = render_chat_template(self.template, user_text, self._token_text("bos_token") or "",
+                                    self._token_text("eos_token") or "") if self.template else user_text
         return text, self.tok.encode(text, add_special_tokens=False).ids
 
     def decode(self, ids) -> str:
         return self.tok.decode(list(ids), skip_special_tokens=True)
+
+
+def render_chat_template(template: str, user_text: str, bos_token: str = "", eos_token: str = "") -> str:
+    """One user turn with the generation prompt through a model folder's chat template.  The template
+    is text from the model folder and is not trusted: it runs in jinja2's immutable sandbox, where
+    reaching for ``__class__``, ``__globals__`` and the like, or changing a passed object, raises
+    ``jinja2.exceptions.SecurityError`` (the reference goes through ``apply_chat_template``, llm.py:87-96,
+    which renders in the same kind of sandbox)."""
+    import jinja2
+    from jinja2.sandbox import ImmutableSandboxedEnvironment
+
+    def raise_exception(message):
+        raise jinja2.exceptions.TemplateError(message)
+
+    env = ImmutableSandboxedEnvironment(trim_blocks=True, lstrip_blocks=True)
+    env.globals["raise_exception"] = raise_exception
+    return env.from_string(template).render(messages=[{"role": "user", "content": user_text}], add_generation_prompt=True,
+                                            bos_token=bos_token, eos_token=eos_token)
 
 
 def _load_tokenizer(folder: Path):

@@ -281,7 +281,7 @@ def test_chat_template_runs_in_a_sandbox():
         with pytest.raises(jinja2.exceptions.SecurityError):
             render_chat_template(evil, "hi")
     assert render_chat_template("{{ raise_exception.__globals__ }}", "hi") == ""      # a function's globals: not there
-    with pytest.raises(jinja2.exceptions.UndefinedError):
+    with pytest.raises(jinja2.exceptions.SecurityError):
         render_chat_template("{{ raise_exception.__globals__['__builtins__'] }}", "hi")
     with pytest.raises(jinja2.exceptions.TemplateError, match="no system turn"):
         render_chat_template("{{ raise_exception('no system turn') }}", "hi")

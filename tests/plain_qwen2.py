@@ -48,12 +48,14 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
 def rope_angles(positions: torch.Tensor, head_dim: int, theta: float) -> torch.Tensor:
     """Angles ``[len(positions), head_dim/2]``: ``pos * theta**(-2j/head_dim)``.
 
-    The inverse frequencies and the product are taken in float32, as the reference's
-    table is (v00_full_recompute/layer/rope.py:29-35), then widened.
+    The inverse frequencies and the product are taken in float32 on the host, as the reference's
+    table is when its module is constructed (v00_full_recompute/layer/rope.py:29-35), then moved to
+    where the positions are and widened by the caller.  (A power taken by another device's routine
+    may differ in its last bit, which a position of several thousand turns into 1e-4 of an angle.)
     """
-    j = torch.arange(0, head_dim, 2, dtype=torch.float32, device=positions.device)
+    j = torch.arange(0, head_dim, 2, dtype=torch.float32)
     inv_freq = 1.0 / (theta ** (j / head_dim))
-    return torch.outer(positions.to(torch.float32), inv_freq)
+    return torch.outer(positions.to(device="cpu", dtype=torch.float32), inv_freq).to(positions.device)
 
 
 def rotate_half(x: torch.Tensor) -> torch.Tensor:

@@ -110,6 +110,26 @@ def expected_logits(folder, requests):
     return {r: plain_qwen2.forward(cfg, weights, t) for r, t in requests.items()}
 
 
+def bounds_from_plain(cfg, tensors, requests):
+    """The plain implementation as its own yardstick, on the device of ``tensors``:
+    ``(expected, noise, noise16, rms16)``.  ``expected``: float64 logits of every request (on the host);
+    ``noise``: how far the plain implementation's own 32-bit evaluation lies from them at most (rounding
+    that depends on the order of summation only); ``noise16`` and ``rms16``: how far, at most and in the
+    root mean square, it moves when evaluated in 64-bit but with every tensor that separate kernels hand
+    to each other through memory rounded to bfloat16."""
+    w64 = {k: v.double() for k, v in tensors.items()}
+    expected = {r: plain_qwen2.forward(cfg, w64, t).cpu() for r, t in requests.items()}
+    rounded = lambda t: t.to(torch.bfloat16).double()
+    moved = {r: plain_qwen2.forward(cfg, w64, t, stored=rounded).cpu() - expected[r] for r, t in requests.items()}
+    del w64
+    w32 = {k: v.float() for k, v in tensors.items()}
+    noise = max(float((plain_qwen2.forward(cfg, w32, t).cpu().double() - expected[r]).abs().max()) for r, t in requests.items())
+    del w32
+    noise16 = max(float(m.abs().max()) for m in moved.values())
+    rms16 = float(torch.cat([m.flatten() for m in moved.values()]).pow(2).mean().sqrt())
+    return expected, noise, noise16, rms16
+
+
 def _rows(steps, outputs, expected, what=""):
     """Every wanted row of a replay beside the plain implementation's logits of its request
     at its absolute position: ``(got, ref, place)``."""

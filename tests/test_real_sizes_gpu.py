@@ -54,18 +54,7 @@ def sized(request):
     tensors = random_tensors(config, seed=seed, dtype=torch.bfloat16, device="cuda")
     requests = scenarios.make_requests(d["vocab_size"], LENGTHS, seed=5)
     cfg = plain.PlainConfig(d)
-    w64 = {k: v.double() for k, v in tensors.items()}
-    expected = {r: plain.forward(cfg, w64, t).cpu() for r, t in requests.items()}
-    del w64
-    w32 = {k: v.float() for k, v in tensors.items()}
-    noise = max(float((plain.forward(cfg, w32, t).cpu().double() - expected[r]).abs().max()) for r, t in requests.items())
-    del w32
-    w64 = {k: v.double() for k, v in tensors.items()}
-    rounded = lambda t: t.to(torch.bfloat16).double()
-    moved = {r: plain.forward(cfg, w64, t, stored=rounded).cpu() - expected[r] for r, t in requests.items()}
-    noise16 = max(float(m.abs().max()) for m in moved.values())
-    rms16 = float(torch.cat([m.flatten() for m in moved.values()]).pow(2).mean().sqrt())
-    del w64, moved
+    expected, noise, noise16, rms16 = scenarios.bounds_from_plain(cfg, tensors, requests)
     torch.cuda.empty_cache()
     print(f"{request.param}: 32-bit noise {noise:.3e}, bfloat16 roundings move the logits by {noise16:.3e} at most, {rms16:.3e} rms", flush=True)
     yield request.param, config, tensors, requests, expected, (noise, noise16, rms16)

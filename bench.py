@@ -122,7 +122,8 @@ def fill_context(runner, req_ids, context: int):
             raise RuntimeError("cache pool too small for the benchmark")
         cache.commit(r, context)
     for g in cache.groups:
-        g.tensor.normal_(0.0, 0.5)
+        for plane in g.tensors:
+            plane.normal_(0.0, 0.5)
 
 
 def time_decode(model, batch: int, steps: int, warmup: int, context: int = CONTEXT):

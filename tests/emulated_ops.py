@@ -22,11 +22,11 @@ def load(names):
     pass
 
 
-def embedding(token_ids, table, out):
-    out.copy_(table.float()[token_ids.long()])
+def embedding(token_ids, table, out, scale=1.0):
+    out.copy_(table.float()[token_ids.long()] * scale)
 
 
-def add_rmsnorm(residual, pending, weight, eps, out, rows=None):
+def add_rmsnorm(residual, pending, weight, eps, out, rows=None, gain=1.0):
     if pending is not None and pending.dim() == 3:
         pending = pending.sum(0)
     if rows is None:
@@ -36,7 +36,7 @@ def add_rmsnorm(residual, pending, weight, eps, out, rows=None):
     else:
         idx = rows.long()
         r = residual[idx] + (pending[idx].float() if pending is not None else 0)
-    y = r * torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    y = r * (torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + eps) * gain) * weight.float()
     out.copy_(y.to(out.dtype))
 
 

@@ -166,3 +166,52 @@ def rms_error(steps, outputs, expected) -> float:
         total += float((got - ref).pow(2).sum())
         count += ref.numel()
     return (total / max(count, 1)) ** 0.5
+
+
+def check_steps_ahead_on_a_random_workload(model, page_size, seed, use_graphs=False):
+    """A random workload (arrivals at random steps, lengths, temperatures, stop tokens, a pool so small
+    that requests are preempted) through the whole engine, with and without steps enqueued ahead of
+    their tokens: every request generates the same tokens and ends for the same reason, no page is
+    lost, and every pool ends full.  Returns the engine of the run with steps ahead."""
+    from torchlet_amd.engine.config import EngineConfig
+    from torchlet_amd.engine.loading import make_engine
+    from torchlet_amd.engine.request import Request
+
+    rnd = random.Random(seed)
+    vocab = model.spec.vocab_size
+    n = rnd.randrange(3, 7)
+    lengths = [rnd.randrange(1, 40) for _ in range(n)]
+    prompts = list(make_requests(vocab, lengths, seed=seed).values())
+    news = [rnd.randrange(1, 20) for _ in range(n)]
+    temps = [rnd.choice([0.0, 0.0, 0.7, 1.3]) for _ in range(n)]
+    arrive = sorted(rnd.randrange(0, 25) for _ in range(n))
+    stop = frozenset(rnd.sample(range(vocab), 24))
+    pages = rnd.choice([6, 8, 30]) * 16 // page_size          # few of them force preemptions
+    budget = rnd.choice([8, 24, 64])
+    slots = rnd.choice([2, 4])
+    dtype = "float32" if model.dtype == torch.float32 else "bfloat16"
+
+    def run(lookahead):
+        e = make_engine(model, EngineConfig(page_size=page_size, num_pages=pages, max_slots=slots, max_tokens_per_step=budget,
+                                            dtype=dtype, use_graphs=use_graphs, lookahead=lookahead, seed=3))
+        reqs = [Request(prompt_tokens=p, seed=i, max_new_tokens=m, temperature=t, stop_token_ids=stop)
+                for i, (p, m, t) in enumerate(zip(prompts, news, temps))]
+        step = 0
+        while step <= max(arrive) or e.has_work():
+            for i, a in enumerate(arrive):
+                if a == step:
+                    e.add_request(reqs[i])
+            if e.has_work():
+                e.step()
+            e.runner.cache.check()
+            step += 1
+        assert e.runner.cache.live_requests() == [] and e._ahead is None
+        assert e.runner.cache.free_pages() == e.runner.cache.capacity()
+        return e, [(r.output_tokens, r.finish_reason) for r in reqs]
+
+    e0, plain = run(False)
+    e1, ahead = run(True)
+    assert ahead == plain, f"seed {seed}: steps enqueued ahead changed what was generated"
+    assert all(reason in ("stop", "length") for _, reason in plain)
+    assert e0.steps_ahead == 0
+    return e1

@@ -36,7 +36,7 @@ def test_pool_is_lifo_and_guards_misuse():
 def test_layers_with_equal_needs_share_a_group_and_shared_caches_follow_their_owner():
     m = manager([(FULL, None, None), (WIN, None, None), (FULL, None, None), (None, None, 1)], device="cpu")
     assert len(m.groups) == 2 and m.groups[0].runs == [0, 2] and m.groups[1].runs == [1]
-    assert m.groups[0].tensor.shape == (2, 2, 10, 2, 8, 16)
+    assert [tuple(t.shape) for t in m.groups[0].tensors] == [(2, 10, 2, 8, 16)] * 2
     c0, c2, c3 = m.layer_cache(0), m.layer_cache(2), m.layer_cache(3)
     assert c0.group == c2.group == 0 and c0.writable and c0.planes[0].data_ptr() != c2.planes[0].data_ptr()
     assert c3.group == 1 and not c3.writable and c3.planes[0].data_ptr() == m.layer_cache(1).planes[0].data_ptr()
@@ -99,7 +99,8 @@ def test_state_slots_are_zeroed_when_handed_out():
     m = manager([(None, StateNeed((4,)), None), (FULL, StateNeed((2, 2), torch.float32), None)], device="cpu")
     s = m.add_request("a")
     c0, c1 = m.layer_cache(0), m.layer_cache(1)
-    assert c0.group is None and c0.state.shape == (3, 4) and c1.state.shape == (3, 2, 2) and c1.group == 0
+    # three slots and the row of the padding requests of fixed-shape steps, which belongs to no request
+    assert c0.group is None and c0.state.shape == (4, 4) and c1.state.shape == (4, 2, 2) and c1.group == 0 and m.pad_slot == 3
     c0.state[s] = 7.0
     m.release("a")
     assert m.add_request("b") == s             # slots are reused, last freed first
@@ -139,3 +140,48 @@ def test_random_orders_never_lose_or_share_a_page(seed):
     for r in list(live):
         m.release(r)
     assert m.free_pages() == [23, 23] and m.free_slots() == 5
+
+
+def test_planes_of_different_widths_and_an_element_type_of_their_own():
+    """A mixer may keep planes that differ in heads and width (a compressed latent beside a small rotated
+    part) and in element type; runs with the same such need still share a group."""
+    latent = PagedNeed(num_heads=1, head_dim=0, planes=((1, 24), (1, 8), (3, 2)), dtype=torch.float32)
+    m = CacheManager([(latent, None, None), (FULL, None, None), (latent, None, None)], page_size=4, num_pages=6,
+                     max_requests=2, dtype=torch.bfloat16, device="cpu")
+    assert len(m.groups) == 2 and m.groups[0].runs == [0, 2]
+    assert [tuple(t.shape) for t in m.groups[0].tensors] == [(2, 6, 1, 4, 24), (2, 6, 1, 4, 8), (2, 6, 3, 4, 2)]
+    assert {t.dtype for t in m.groups[0].tensors} == {torch.float32} and m.groups[1].tensors[0].dtype == torch.bfloat16
+    c = m.layer_cache(2)
+    assert [tuple(p.shape) for p in c.planes] == [(6, 1, 4, 24), (6, 1, 4, 8), (6, 3, 4, 2)]
+    assert c.planes[0].data_ptr() == m.groups[0].tensors[0][1].data_ptr()
+    assert m.bytes_per_page() == 2 * 4 * (24 + 8 + 6) * 4 + 2 * (2 * 4 * 16) * 2
+    assert FULL.plane_shapes == ((2, 16), (2, 16))
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_a_windowed_groups_pool_is_sized_by_the_window_when_steps_are_bounded(seed):
+    """With steps of at most 12 tokens a request holds at most (20 + 12 - 2) // 4 + 2 = 9 pages of a group
+    with a window of 20 at pages of 4: three slots need 27 pages and the sentinel, however many pages the
+    full-attention group has; sequences far longer than that pool still fit, and nothing is lost."""
+    rng = random.Random(seed)
+    m = CacheManager([(FULL, None, None), (WIN, None, None)], page_size=4, num_pages=200, max_requests=3, max_step_tokens=12)
+    assert m.capacity() == [199, 27] and m.pages_for(400) == [100, 9]
+    lengths: dict[str, int] = {}
+    for step in range(400):
+        if len(lengths) < 3 and rng.random() < 0.3:
+            r = f"r{step}"
+            m.add_request(r)
+            lengths[r] = 0
+        for r in list(lengths):
+            n = rng.choice([1, 1, 1, 5, 12])
+            if lengths[r] + n > 260 or rng.random() < 0.02:
+                m.release(r)
+                del lengths[r]
+                continue
+            assert m.reserve(r, lengths[r] + n), "a bounded step must always find its pages in the windowed pool"
+            lengths[r] += n
+            m.commit(r, lengths[r])
+        m.check()
+    for r in lengths:
+        m.release(r)
+    assert m.free_pages() == [199, 27]

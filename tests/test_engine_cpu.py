@@ -162,43 +162,18 @@ def test_a_step_enqueued_ahead_of_its_tokens_changes_nothing_that_is_generated(c
 def test_steps_ahead_under_random_arrivals_stop_tokens_and_few_pages(cpu_ops, model_folders, name, seed):
     """Random workloads (arrivals at random steps, lengths, temperatures, stop tokens, a pool so small
     that requests are preempted): with and without steps enqueued ahead, every request generates
-    the same tokens and ends for the same reason; no page is lost."""
-    import random
-    rnd = random.Random(seed)
-    cfg = json.loads((model_folders[name] / "config.json").read_text())
-    n = rnd.randrange(3, 7)
-    lengths = [rnd.randrange(1, 40) for _ in range(n)]
-    prompts = list(scenarios.make_requests(cfg["vocab_size"], lengths, seed=seed).values())
-    news = [rnd.randrange(1, 20) for _ in range(n)]
-    temps = [rnd.choice([0.0, 0.0, 0.7, 1.3]) for _ in range(n)]
-    arrive = sorted(rnd.randrange(0, 25) for _ in range(n))
-    stop = frozenset(rnd.sample(range(cfg["vocab_size"]), 24))
-    pages = rnd.choice([6, 8, 30])                           # pages of 16 tokens; few of them force preemptions
-    budget = rnd.choice([8, 24, 64])
+    the same tokens and ends for the same reason; no page is lost.  (The same runs on the GPU, with
+    decode steps replayed as graphs, in test_generate_gpu.py.)"""
+    _, model = load_model(model_folders[name], "float32", device="cpu")
+    scenarios.check_steps_ahead_on_a_random_workload(model, tiny_models.PAGE_SIZES[name], seed)
 
-    def run(lookahead):
-        e = Engine(runner_for(model_folders[name], name, pages=pages, slots=rnd_slots), max_tokens_per_step=budget, seed=3,
-                   lookahead=lookahead)
-        reqs = [Request(prompt_tokens=p, seed=i, max_new_tokens=m, temperature=t, stop_token_ids=stop)
-                for i, (p, m, t) in enumerate(zip(prompts, news, temps))]
-        step = 0
-        while step <= max(arrive) or e.has_work():
-            for i, a in enumerate(arrive):
-                if a == step:
-                    e.add_request(reqs[i])
-            if e.has_work():
-                e.step()
-            e.runner.cache.check()
-            step += 1
-        assert e.runner.cache.live_requests() == [] and e._ahead is None
-        assert all(f == pages - 1 for f in e.runner.cache.free_pages())
-        return e, [(r.output_tokens, r.finish_reason) for r in reqs]
 
-    rnd_slots = rnd.choice([2, 4])
-    e0, plain = run(False)
-    e1, ahead = run(True)
-    assert ahead == plain
-    assert all(reason in ("stop", "length") for _, reason in plain)
+def test_max_model_len_bounds_the_step_function(cpu_ops, model_folders):
+    _, model = load_model(model_folders["A"], "float32", device="cpu")
+    runner = make_runner(model, page_size=16, num_pages=20, max_requests=2, max_model_len=30)
+    assert runner.step([StepEntry("a", [1] * 30, [29])].copy()).shape == (1, 256)
+    with pytest.raises(ValueError, match="max_model_len"):
+        runner.step([StepEntry("a", [1], [0])])
 
 
 def test_draw_keys_differ_in_every_argument():

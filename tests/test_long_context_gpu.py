@@ -281,8 +281,9 @@ def test_every_split_at_long_contexts(long_model, dtype):
         need = scenarios.max_tokens_needed(steps, unit=page)
         runner = make_runner(model, page_size=page, num_pages=-(-need // page) + 1, max_requests=4)
         for g in runner.cache.groups:
-            g.tensor.fill_(float("nan"))            # whatever an earlier request left in a page must not matter
-            g.tensor[:, :, 0] = 0                   # but the sentinel page, which masked places may read
+            for plane in g.tensors:
+                plane.fill_(float("nan"))           # whatever an earlier request left in a page must not matter
+                plane[:, 0] = 0                     # but the sentinel page, which masked places may read
         print(f"{name} {dtype} {mode}: {len(steps)} steps, {need} tokens of cache", flush=True)
         out = {}
         for s in steps:

@@ -235,7 +235,7 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path):
         assert "model.layers.1.mix.decay" in tensors
         model = build_model(cfg, "float32", tensors=tensors)
         runner = make_runner(model, page_size=16, num_pages=2, max_requests=2)
-        assert runner.cache.groups == [] and runner.caches[0].state.shape == (2, 24)
+        assert runner.cache.groups == [] and runner.caches[0].state.shape == (3, 24)
         seqs = {"a": torch.randint(0, 40, (23,)).tolist(), "b": torch.randint(0, 40, (9,)).tolist()}
         whole = {k: runner.step([StepEntry(k, v, list(range(len(v))))]).cpu() for k, v in seqs.items()}
         for k in seqs:

@@ -29,7 +29,8 @@ def _run_in_process(folder, dtype, steps, page_size, max_tokens, max_requests=4,
     runner = make_runner(model, page_size=page_size, num_pages=-(-max_tokens // page_size) + 1, max_requests=max_requests)
     if poison:      # every page but the sentinel (page 0), which nothing ever writes and released entries point to
         for group in runner.cache.groups:
-            group.tensor[:, :, 1:].fill_(float("nan"))          # [runs, planes, pages, heads, page, head size]
+            for plane in group.tensors:
+                plane[:, 1:].fill_(float("nan"))                     # [runs, pages, heads, page, head size]
     out = {}
     for s in steps:
         logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
@@ -41,7 +42,7 @@ def _run_in_process(folder, dtype, steps, page_size, max_tokens, max_requests=4,
     assert runner.cache.live_requests() == []
     if poison:
         for group in runner.cache.groups:
-            assert not bool(group.tensor[:, :, 0].any()), "the sentinel page was written"
+            assert not any(bool(plane[:, 0].any()) for plane in group.tensors), "the sentinel page was written"
     return out
 
 

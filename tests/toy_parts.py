@@ -12,8 +12,10 @@ def run_toy_mix(dtype, device, tolerance):
     """Parts defined here -- a feed-forward that routes every token to one of three experts, and
     a rotary encoding that pairs neighbouring dimensions -- are registered and put into a model
     beside the framework's own parts; the first layer runs a second time at the end, reading the
-    keys and values of its first run.  Whole requests and requests cut into portions beside
-    other requests agree with each other and with a plain computation written out below."""
+    keys and values of its first run.  The model also uses what the model specification offers beyond
+    the one architecture's needs: a factor on the embedding rows, a factor on the logits, a bias on the
+    output head, and a score scale of its own in one layer's attention.  Whole requests and requests cut
+    into portions beside other requests agree with each other and with a plain computation written out below."""
     from torchlet_amd.config import (AttentionSpec, BlockSpec, ModelConfig, ModelSpec, PartSpec, RMSNormSpec, RotarySpec,
                                      RunEntry, SwiGLUSpec)
     from torchlet_amd.engine.batch import StepEntry
@@ -24,6 +26,7 @@ def run_toy_mix(dtype, device, tolerance):
     from torchlet_amd.weights.random_init import random_tensors
 
     H, HEADS, KVH, HD, INTER, EXPERTS, VOCAB, THETA = 48, 4, 2, 16, 40, 3, 50, 100.0
+    EMBED_SCALE, LOGIT_SCALE, SCORE_SCALE = 1.7, 0.6, 0.31
 
     @dataclass(frozen=True)
     class PairRotarySpec(PartSpec):
@@ -100,14 +103,15 @@ def run_toy_mix(dtype, device, tolerance):
 
         def to_spec(self):
             norm = RMSNormSpec(dim=H, eps=1e-5)
-            attn = lambda pos: AttentionSpec(hidden=H, num_heads=HEADS, num_kv_heads=KVH, head_dim=HD, qkv_bias=False, position=pos)
+            attn = lambda pos, scale=None: AttentionSpec(hidden=H, num_heads=HEADS, num_kv_heads=KVH, head_dim=HD, qkv_bias=False,
+                                                         position=pos, scale=scale)
             first = BlockSpec(mixer=attn(PairRotarySpec(head_dim=HD, theta=THETA)), mixer_norm=norm, ffn_norm=norm,
                               ffn=SwiGLUSpec(hidden=H, intermediate=INTER))
-            second = BlockSpec(mixer=attn(RotarySpec(head_dim=HD, theta=THETA, max_positions=4096)), mixer_norm=norm, ffn_norm=norm,
-                               ffn=Top1Spec(hidden=H, intermediate=INTER, experts=EXPERTS), ffn_name="moe")
+            second = BlockSpec(mixer=attn(RotarySpec(head_dim=HD, theta=THETA, max_positions=4096), SCORE_SCALE), mixer_norm=norm,
+                               ffn_norm=norm, ffn=Top1Spec(hidden=H, intermediate=INTER, experts=EXPERTS), ffn_name="moe")
             return ModelSpec(vocab_size=self.vocab_size, hidden=H, layers=(first, second),
                              order=(RunEntry(0), RunEntry(1), RunEntry(0, cache_of=0)), final_norm=norm,
-                             tie_head=True, max_positions=4096)
+                             tie_head=True, max_positions=4096, embed_scale=EMBED_SCALE, logit_scale=LOGIT_SCALE, head_bias=True)
 
     def pair_rope(x, positions):                      # x [heads, T, hd], float64
         inv = 1.0 / (THETA ** (torch.arange(0, HD, 2, dtype=torch.float32) / HD))
@@ -118,7 +122,7 @@ def run_toy_mix(dtype, device, tolerance):
         y[..., 1::2] = b * ang.cos() + a * ang.sin()
         return y
 
-    def plain_attention(h, w, rope, kv=None, stored=lambda t: t):
+    def plain_attention(h, w, rope, kv=None, stored=lambda t: t, scale=None):
         """Returns the mixed heads' projection and the (k, v) it used; with ``kv`` given, only q is new.
         ``stored``: applied to what separate kernels hand each other through memory (see plain_qwen2)."""
         T = h.shape[0]
@@ -129,19 +133,21 @@ def run_toy_mix(dtype, device, tolerance):
             v = stored(h @ w["v_proj.weight"].T).view(T, KVH, HD).transpose(0, 1)
             kv = (k, v)
         k, v = (t.repeat_interleave(HEADS // KVH, dim=0) for t in kv)
+        if scale is not None:             # attention_weights divides the scores by sqrt(head size): undo that, put `scale` there
+            q = q * (scale * HD ** 0.5)
         ctx = stored((plain.attention_weights(q, k) @ v).transpose(0, 1).reshape(T, HEADS * HD))
         return stored(ctx @ w["o_proj.weight"].T), kv
 
     def plain_forward(w, ids, stored=lambda t: t):
         sub = lambda p: {k[len(p):]: v for k, v in w.items() if k.startswith(p)}
         l0, l1 = sub("model.layers.0."), sub("model.layers.1.")
-        x = w["model.embed_tokens.weight"][torch.tensor(ids)]
+        x = w["model.embed_tokens.weight"][torch.tensor(ids)] * EMBED_SCALE
         norm = lambda t, weight: stored(plain.rms_norm(t, weight, 1e-5))
         a, kv0 = plain_attention(norm(x, l0["input_layernorm.weight"]), sub("model.layers.0.self_attn."), pair_rope, None, stored)
         x = x + a
         x = x + plain.swiglu_ffn(norm(x, l0["post_attention_layernorm.weight"]), sub("model.layers.0.mlp."), stored)
         a, _ = plain_attention(norm(x, l1["input_layernorm.weight"]), sub("model.layers.1.self_attn."),
-                               lambda t, pos: plain.rope_apply(t, pos, THETA), None, stored)
+                               lambda t, pos: plain.rope_apply(t, pos, THETA), None, stored, SCORE_SCALE)
         x = x + a
         h = norm(x, l1["post_attention_layernorm.weight"])
         p = torch.softmax(h @ l1["moe.router.weight"].T, dim=-1)
@@ -159,7 +165,8 @@ def run_toy_mix(dtype, device, tolerance):
         a, _ = plain_attention(norm(x, l0["input_layernorm.weight"]), sub("model.layers.0.self_attn."), pair_rope, kv0, stored)
         x = x + a
         x = x + plain.swiglu_ffn(norm(x, l0["post_attention_layernorm.weight"]), sub("model.layers.0.mlp."), stored)
-        return norm(x, w["model.norm.weight"]) @ w["model.embed_tokens.weight"].T
+        last = stored(plain.rms_norm(x, w["model.norm.weight"], 1e-5) * LOGIT_SCALE)
+        return last @ w["model.embed_tokens.weight"].T + w["lm_head.bias"]
 
     gaps = []
     register_architecture(ToyConfig)
@@ -168,6 +175,7 @@ def run_toy_mix(dtype, device, tolerance):
         tensors = {k: (v * 5 if "proj" in k or "experts" in k or "router" in k else v)
                    for k, v in random_tensors(cfg, seed=4, dtype=torch.bfloat16).items()}
         assert "model.layers.1.moe.experts.2.down.weight" in tensors and "model.layers.1.moe.router.weight" in tensors
+        assert tensors["lm_head.bias"].shape == (VOCAB,) and "lm_head.weight" not in tensors
         model = build_model(cfg, dtype, device=device, tensors=tensors)
         runner = make_runner(model, page_size=8, num_pages=24, max_requests=2)
         assert len(runner.caches) == 3 and runner.caches[2].planes[0].data_ptr() == runner.caches[0].planes[0].data_ptr() and not runner.caches[2].writable

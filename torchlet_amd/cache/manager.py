@@ -3,17 +3,20 @@
 What it owns
 ------------
 * **Groups of pages.**  Every run of the layer order that owns a per-token cache declares
-  a :class:`~torchlet_amd.parts.base.PagedNeed`.  Runs with equal needs (heads, head size,
-  window) form a *group*: one pool of pages, one tensor
-  ``[runs, planes, pages, heads, page_size, head_dim]`` and one block table per request.
-  A page id addresses every run of its group, so one table row serves them all.  Page 0
-  of every group is a sentinel that is never handed out: empty table entries point to it.
+  a :class:`~torchlet_amd.parts.base.PagedNeed`.  Runs with equal needs (planes, their heads and
+  widths, element type, window) form a *group*: one pool of pages, per plane one tensor
+  ``[runs, pages, heads, page_size, width]`` and one block table per request.
+  A page id addresses every run and plane of its group, so one table row serves them all.  Page 0
+  of every group is a sentinel that is never handed out and never written: empty table entries
+  point to it.  A group with a window needs fewer pages than one that keeps everything: when the
+  most tokens of a step are known its pool is sized for what its requests can hold at once.
 * **Block tables.**  Per request and group, the list of pages in logical order.  A group
   with a window gives pages back as soon as every key in them lies behind the window of
   all future queries; their table entries fall back to the sentinel.
 * **Slots.**  A request holds one slot from admission to release.  Runs that declare a
-  :class:`~torchlet_amd.parts.base.StateNeed` get a tensor ``[slots, *shape]``; a slot's
-  rows are zeroed when it is handed out.
+  :class:`~torchlet_amd.parts.base.StateNeed` get a tensor ``[slots + 1, *shape]``; a slot's
+  rows are zeroed when it is handed out.  The last row (``pad_slot``) belongs to no request: the
+  padding rows of a step of fixed shape read and write it.
 
 Free lists are last-in-first-out (as the reference's, /root/reference/src/torchlet/
 v10_triton_paged_gqa/kvcache.py:39-66): pages freed by a finished request are the next to
@@ -82,7 +85,7 @@ class PagePool:
 class LayerCache:
     """What one run of the layer order sees of the cache."""
     group: int | None                 # index into StepContext.block_tables
-    planes: tuple                     # per plane a tensor [pages, heads, page_size, head_dim]
+    planes: tuple                     # per plane a tensor [pages, heads, page_size, width]
     page_size: int
     state: torch.Tensor | None        # [slots, *shape] of the run's StateNeed
     writable: bool                    # False: the run reads another run's cache
@@ -135,7 +138,7 @@ class _Group:
         self.runs: list[int] = []                 # indices into the run order, in order
         self.pool = PagePool(num_pages)
         self.tables: dict[object, _PageTable] = {}  # request -> page of each logical block (0: none)
-        self.tensor: torch.Tensor | None = None
+        self.tensors: list[torch.Tensor] = []     # per plane [runs, pages, heads, page_size, width]
 
 
 class _Request:
@@ -147,10 +150,13 @@ class _Request:
 
 
 class CacheManager:
-    """``plan``: per run of the layer order ``(paged_need | None, state_need | None, cache_of | None)``."""
+    """``plan``: per run of the layer order ``(paged_need | None, state_need | None, cache_of | None)``.
+    ``num_pages``: pages of a group's pool, the sentinel included.  ``max_step_tokens``: the most tokens a
+    request brings in one step, if the caller keeps to one (a scheduler's token budget); the pool of a group
+    with a window is then no larger than what ``max_requests`` requests can hold of it at once."""
 
     def __init__(self, plan, *, page_size: int, num_pages: int, max_requests: int,
-                 dtype: torch.dtype = torch.float32, device=None):
+                 dtype: torch.dtype = torch.float32, device=None, max_step_tokens: int | None = None):
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         if max_requests <= 0:
@@ -158,6 +164,8 @@ class CacheManager:
         self.page_size = page_size
         self.num_pages = num_pages
         self.max_requests = max_requests
+        self.pad_slot = max_requests             # a state row of its own for the padding rows of fixed-shape steps
+        self.max_step_tokens = max_step_tokens
         self.dtype = dtype
         self.device = device
         self.groups: list[_Group] = []
@@ -182,7 +190,7 @@ class CacheManager:
                 g = by_need.get(paged)
                 if g is None:
                     g = by_need[paged] = len(self.groups)
-                    self.groups.append(_Group(paged, num_pages))
+                    self.groups.append(_Group(paged, self._pool_size(paged)))
                 self._run_group.append(g)
                 self._run_index.append(len(self.groups[g].runs))
                 self.groups[g].runs.append(i)
@@ -191,20 +199,43 @@ class CacheManager:
         self._free_slots = list(range(max_requests - 1, -1, -1))
         if device is not None:
             for g in self.groups:
-                n = g.need
-                g.tensor = torch.zeros((len(g.runs), n.planes, num_pages, n.num_heads, page_size, n.head_dim),
-                                       dtype=dtype, device=device)
+                g.tensors = [torch.zeros((len(g.runs), g.pool.num_pages, heads, page_size, width),
+                                         dtype=g.need.dtype or dtype, device=device)
+                             for heads, width in g.need.plane_shapes]
             for s in self._state_needs:
                 self._states.append(None if s is None else
-                                    torch.zeros((max_requests, *s.shape), dtype=s.dtype, device=device))
+                                    torch.zeros((max_requests + 1, *s.shape), dtype=s.dtype, device=device))
         else:
             self._states = [None] * len(self._state_needs)
 
+    def _held_at_most(self, need: PagedNeed) -> int | None:
+        """Most pages one request can hold in a group with a window when no step brings more than
+        ``max_step_tokens`` tokens: the blocks from the first one a query can still read to the last
+        one the step writes.  ``None``: no bound (no window, or steps of any size)."""
+        if need.window is None or self.max_step_tokens is None:
+            return None
+        return (need.window + self.max_step_tokens - 2) // self.page_size + 2
+
+    def _pool_size(self, need: PagedNeed) -> int:
+        most = self._held_at_most(need)
+        if most is None:
+            return self.num_pages
+        return max(2, min(self.num_pages, self.max_requests * most + 1))
+
     # ------------------------------------------------------------------ queries
     def bytes_per_page(self) -> int:
-        size = torch.empty((), dtype=self.dtype).element_size()
-        return sum(len(g.runs) * g.need.planes * g.need.num_heads * self.page_size * g.need.head_dim * size
-                   for g in self.groups)
+        """Bytes that one more page of ``num_pages`` costs (groups whose pools are capped do not grow with it)."""
+        total = 0
+        for g in self.groups:
+            if self._held_at_most(g.need) is not None and g.pool.num_pages < self.num_pages:
+                continue
+            size = torch.empty((), dtype=g.need.dtype or self.dtype).element_size()
+            total += sum(len(g.runs) * heads * self.page_size * width * size for heads, width in g.need.plane_shapes)
+        return total
+
+    def capacity(self) -> list[int]:
+        """Per group, the pages that can be handed out (the pool without its sentinel)."""
+        return [g.pool.num_pages - 1 for g in self.groups]
 
     def has(self, req_id) -> bool:
         return req_id in self._requests
@@ -250,8 +281,13 @@ class CacheManager:
         return out
 
     def pages_for(self, length: int) -> list[int]:
-        """Per group, the pages a fresh request needs to hold ``length`` tokens in one step."""
-        return [-(-length // self.page_size) for _ in self.groups]
+        """Per group, the most pages a request holds at once on its way to ``length`` tokens."""
+        out = []
+        for g in self.groups:
+            blocks = -(-length // self.page_size)
+            most = self._held_at_most(g.need)
+            out.append(blocks if most is None else min(blocks, most))
+        return out
 
     # ------------------------------------------------------------------ lifecycle
     def add_request(self, req_id) -> int:
@@ -341,8 +377,8 @@ class CacheManager:
         if gi is None and state is None:
             return None
         planes: tuple = ()
-        if gi is not None and self.groups[gi].tensor is not None:
-            planes = tuple(self.groups[gi].tensor[self._run_index[owner]].unbind(0))
+        if gi is not None:
+            planes = tuple(t[self._run_index[owner]] for t in self.groups[gi].tensors)
         return LayerCache(group=gi, planes=planes, page_size=self.page_size, state=state, writable=(owner == run))
 
     def check(self) -> None:

@@ -54,6 +54,7 @@ class AttentionSpec(PartSpec):
     qkv_bias: bool = True
     window: int | None = None          # None: every earlier key; W: the last W keys
     position: PartSpec | None = None   # position encoding applied to q and k
+    scale: float | None = None         # factor on the scores before the softmax; None: head_dim ** -0.5
 
 
 @dataclass(frozen=True)
@@ -106,6 +107,9 @@ class ModelSpec:
     layers_prefix: str = "model.layers"
     final_norm_name: str = "model.norm"
     head_name: str = "lm_head"
+    embed_scale: float = 1.0       # factor on the embedding rows as they enter the residual stream
+    logit_scale: float = 1.0       # factor on the logits (applied to the final norm's output, in 32-bit)
+    head_bias: bool = False        # the output head has a bias vector ``<head_name>.bias``
 
     def __post_init__(self):
         for i, e in enumerate(self.order):

@@ -4,27 +4,27 @@
 #include "common.h"
 
 // ------------------------------------------------------------------ embedding
-// out[t, :] = float(table[ids[t], :]); the residual stream is 32-bit.
+// out[t, :] = float(table[ids[t], :]) * scale; the residual stream is 32-bit.
 template <typename T>
 __global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                                 float* __restrict__ out, int hidden, int vocab) {
+                                 float* __restrict__ out, int hidden, int vocab, float scale) {
     const int t = blockIdx.x;
     int id = ids[t];
     if (id < 0 || id >= vocab) id = 0;  // ids are checked on the host; never read out of bounds
     const T* src = table + (size_t)id * hidden;
     float* dst = out + (size_t)t * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]) * scale;
 }
 
 extern "C" int tl_embedding(const void* ids, const void* table, int table_dtype, void* out,
-                            int tokens, int hidden, int vocab, hipStream_t stream) {
+                            int tokens, int hidden, int vocab, float scale, hipStream_t stream) {
     TL_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes tokens=%d hidden=%d vocab=%d", tokens, hidden, vocab);
     if (tokens == 0) return TL_OK;
     dim3 grid(tokens), block(256);
     if (table_dtype == TL_DT_F32)
-        embedding_kernel<float><<<grid, block, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab);
+        embedding_kernel<float><<<grid, block, 0, stream>>>((const int*)ids, (const float*)table, (float*)out, hidden, vocab, scale);
     else if (table_dtype == TL_DT_BF16)
-        embedding_kernel<bf16_t><<<grid, block, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab);
+        embedding_kernel<bf16_t><<<grid, block, 0, stream>>>((const int*)ids, (const bf16_t*)table, (float*)out, hidden, vocab, scale);
     else TL_REQUIRE(false, "embedding: unknown dtype %d", table_dtype);
     TL_CHECK_LAUNCH("embedding");
     return TL_OK;
@@ -34,12 +34,13 @@ extern "C" int tl_embedding(const void* ids, const void* table, int table_dtype,
 // One block per output row.  r = residual[row] (+ pending[row]); if `update`, r is
 // written back to the residual; out = r * rsqrt(mean(r^2) + eps) * weight.
 // `rows` (optional) selects the source row of each output row; then nothing is written back.
+// `gain` multiplies the row's scale factor (1: the plain norm; a model with a factor on its logits puts it here).
 // The pending branch output comes either as one [rows, hidden] tensor of the activation type
 // (parts == 0) or as `parts` float slabs [parts, total_rows, hidden] of partial sums that are
 // added up here (the split-K products write such slabs).
 template <typename T>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const void* __restrict__ pending, int parts, size_t part_stride,
-                                   const void* __restrict__ weight, int weight_f32, float eps,
+                                   const void* __restrict__ weight, int weight_f32, float eps, float gain,
                                    T* __restrict__ out, const int* __restrict__ rows, int hidden) {
     __shared__ float red[16];
     const int orow = blockIdx.x;
@@ -58,7 +59,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const void* __r
         ss += r * r;
     }
     ss = block_sum(ss, red);
-    const float inv = rsqrtf(ss / (float)hidden + eps);
+    const float inv = rsqrtf(ss / (float)hidden + eps) * gain;
     T* dst = out + (size_t)orow * hidden;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float r = res[i];
@@ -98,7 +99,7 @@ template <> struct Vec4<bf16_t> {
 
 template <typename T, int IT>
 __global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const void* __restrict__ pending, int parts, size_t part_stride,
-                                       const void* __restrict__ weight, int weight_f32, float eps,
+                                       const void* __restrict__ weight, int weight_f32, float eps, float gain,
                                        T* __restrict__ out, const int* __restrict__ rows, int hidden) {
     __shared__ float red[16];
     const int orow = blockIdx.x;
@@ -155,7 +156,7 @@ __global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const void*
         }
     }
     ss = block_sum(ss, red);
-    const float inv = rsqrtf(ss / (float)hidden + eps);
+    const float inv = rsqrtf(ss / (float)hidden + eps) * gain;
     T* dst = out + (size_t)orow * hidden;
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
@@ -171,37 +172,37 @@ __global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const void*
 
 template <typename T>
 static void launch_add_rmsnorm(float* residual, const void* pending, int parts, size_t part_stride, const void* weight,
-                               int weight_f32, float eps, T* out, const int* rows, int out_rows, int hidden, hipStream_t stream) {
+                               int weight_f32, float eps, float gain, T* out, const int* rows, int out_rows, int hidden, hipStream_t stream) {
     const bool aligned = hidden % 4 == 0 && ((uintptr_t)residual % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
                          ((uintptr_t)pending % 16) == 0 && ((uintptr_t)weight % 16) == 0;
     dim3 grid(out_rows);
     if (aligned && hidden <= 1024)
-        add_rmsnorm_reg_kernel<T, 1><<<grid, 256, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 1><<<grid, 256, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, gain, out, rows, hidden);
     else if (aligned && hidden <= 2048)
-        add_rmsnorm_reg_kernel<T, 2><<<grid, 256, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 2><<<grid, 256, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, gain, out, rows, hidden);
     else if (aligned && hidden <= 4096)
-        add_rmsnorm_reg_kernel<T, 2><<<grid, 512, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 2><<<grid, 512, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, gain, out, rows, hidden);
     else if (aligned && hidden <= 8192)
-        add_rmsnorm_reg_kernel<T, 4><<<grid, 512, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 4><<<grid, 512, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, gain, out, rows, hidden);
     else if (aligned && hidden <= 16384)
-        add_rmsnorm_reg_kernel<T, 4><<<grid, 1024, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_reg_kernel<T, 4><<<grid, 1024, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, gain, out, rows, hidden);
     else
-        add_rmsnorm_kernel<T><<<grid, hidden >= 2048 ? 512 : 256, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, out, rows, hidden);
+        add_rmsnorm_kernel<T><<<grid, hidden >= 2048 ? 512 : 256, 0, stream>>>(residual, pending, parts, part_stride, weight, weight_f32, eps, gain, out, rows, hidden);
 }
 
 // parts == 0: `pending` is [rows, hidden] of the activation type (or null); parts > 0: `pending` is
 // float [parts, part_rows, hidden], slabs of partial sums to be added up.
 extern "C" int tl_add_rmsnorm(void* residual, const void* pending, int parts, int part_rows, const void* weight,
-                              int weight_f32, float eps, void* out, const void* rows, int out_rows, int hidden,
+                              int weight_f32, float eps, float gain, void* out, const void* rows, int out_rows, int hidden,
                               int act_dtype, hipStream_t stream) {
     TL_REQUIRE(parts >= 0 && parts <= 64, "add_rmsnorm: %d partial slabs", parts);
     const size_t part_stride = (size_t)part_rows * hidden;
     TL_REQUIRE(out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d hidden=%d", out_rows, hidden);
     if (out_rows == 0) return TL_OK;
     if (act_dtype == TL_DT_F32)
-        launch_add_rmsnorm<float>((float*)residual, pending, parts, part_stride, weight, weight_f32, eps, (float*)out, (const int*)rows, out_rows, hidden, stream);
+        launch_add_rmsnorm<float>((float*)residual, pending, parts, part_stride, weight, weight_f32, eps, gain, (float*)out, (const int*)rows, out_rows, hidden, stream);
     else if (act_dtype == TL_DT_BF16)
-        launch_add_rmsnorm<bf16_t>((float*)residual, pending, parts, part_stride, weight, weight_f32, eps, (bf16_t*)out, (const int*)rows, out_rows, hidden, stream);
+        launch_add_rmsnorm<bf16_t>((float*)residual, pending, parts, part_stride, weight, weight_f32, eps, gain, (bf16_t*)out, (const int*)rows, out_rows, hidden, stream);
     else TL_REQUIRE(false, "add_rmsnorm: unknown dtype %d", act_dtype);
     TL_CHECK_LAUNCH("add_rmsnorm");
     return TL_OK;
@@ -216,7 +217,9 @@ extern "C" int tl_add_rmsnorm(void* residual, const void* pending, int parts, in
 //   * write (k_plane != null): rotated k and raw v of the token go to the page
 //     block_table[token_req[t]][pos / page] at offset pos % page.  The key plane is
 //     [pages, kv_heads, page, head_dim]; the value plane holds each page transposed,
-//     [pages, kv_heads, head_dim, page], the layout the attention kernels read.
+//     [pages, kv_heads, head_dim, page], the layout the attention kernels read.  Page 0 is the
+//     sentinel that empty block-table entries point to: a token whose page is 0 (a padding row of a
+//     step of fixed shape) has its keys and values dropped, so nothing ever writes that page.
 // One pair turned by its angle, in a fixed sequence of roundings (one product, one fused
 // multiply-add per result), so that every kernel here gives the same bits for the same input.
 __device__ __forceinline__ void rope_turn(float& x1, float& x2, float c, float sn) {
@@ -252,8 +255,9 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
         const int page = block_table[(size_t)token_req[t] * bt_stride + pos / page_size];
         const int kvh = (head - q_heads) % kv_heads;
         const size_t base = ((size_t)page * kv_heads + kvh) * page_size * head_dim;
-        dst = head < q_heads + kv_heads ? k_plane + base + (size_t)(pos % page_size) * head_dim
-                                        : v_plane + base + (pos % page_size);
+        if (page != 0)
+            dst = head < q_heads + kv_heads ? k_plane + base + (size_t)(pos % page_size) * head_dim
+                                            : v_plane + base + (pos % page_size);
     }
     // With `parts` the row does not come from qkv but is the sum of float slabs of partial sums
     // [num_parts][tokens, parts_ld] plus the bias (a projection that was split over K); the rotated
@@ -275,7 +279,8 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
         return sum;
     };
     if (head >= q_heads + kv_heads) {      // value head: [head_dim, page] inside the page
-        for (int d = lane; d < head_dim; d += TL_WAVE) dst[(size_t)d * page_size] = from_float<T>(element(d));
+        if (dst)
+            for (int d = lane; d < head_dim; d += TL_WAVE) dst[(size_t)d * page_size] = from_float<T>(element(d));
         return;
     }
     const bool rotate = inv_freq && head < rot_heads;
@@ -334,6 +339,7 @@ void rope_cache_write_rows_kernel(bf16_t* __restrict__ qkv, int row_stride, int 
     bf16_t* row = qkv + (size_t)t * row_stride;
     size_t page_base = 0;
     if (k_plane) page_base = (size_t)block_table[(size_t)token_req[t] * bt_stride + pos / page_size] * kv_heads * page_size * head_dim;
+    const bool stores = k_plane && page_base != 0;                 // page 0 is the sentinel: never written
     const int off = pos % page_size;
     for (int p = threadIdx.x; p < heads * pph; p += 256) {
         const int head = p / pph, d0 = (p % pph) * 8;
@@ -341,8 +347,10 @@ void rope_cache_write_rows_kernel(bf16_t* __restrict__ qkv, int row_stride, int 
         piece.u = *(const uint4*)(row + (size_t)head * head_dim + d0);
         if (head >= q_heads + kv_heads) {                          // value head: [head_dim, page] inside the page
             bf16_t* dst = v_plane + page_base + (size_t)(head - q_heads - kv_heads) * page_size * head_dim + off;
+            if (stores) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) dst[(size_t)(d0 + e) * page_size].bits = piece.e[e];
+                for (int e = 0; e < 8; ++e) dst[(size_t)(d0 + e) * page_size].bits = piece.e[e];
+            }
             continue;
         }
         const bool rotate = inv_freq && head < rot_heads;
@@ -362,7 +370,7 @@ void rope_cache_write_rows_kernel(bf16_t* __restrict__ qkv, int row_stride, int 
             }
             *(uint4*)(row + (size_t)head * head_dim + d0) = piece.u;
         }
-        if (head >= q_heads && k_plane)
+        if (head >= q_heads && stores)
             *(uint4*)(k_plane + page_base + ((size_t)(head - q_heads) * page_size + off) * head_dim + d0) = piece.u;
     }
 }

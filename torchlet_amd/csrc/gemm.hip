@@ -565,7 +565,7 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
                     for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(val[v]).bits;
                     if (head < ra.q_heads || !ra.k_plane) {
                         *(uint2*)((bf16_t*)out + (size_t)m * ldo + n) = pk.u;
-                    } else {
+                    } else if (rp_page != 0) {         // page 0 is the sentinel (a padding row's): never written
                         const int kvh = (head - ra.q_heads) % ra.kv_heads, off = rp_pos % ra.page;
                         const size_t base = ((size_t)rp_page * ra.kv_heads + kvh) * ra.page * ra.head_dim;
                         if (head < ra.q_heads + ra.kv_heads) {

@@ -148,11 +148,14 @@ class StaticDecodeContext:
     that is refilled before every step (one copy from pinned host memory).  Because no
     address or launch size changes between steps, the model's forward pass over it can be
     captured once as a HIP graph and replayed.  Unused rows are padded with requests of
-    length zero whose block tables point at the sentinel page.
+    length zero whose block tables point at the sentinel page (the cache-write kernels drop what
+    would go to that page, so nothing writes it) and whose slot is ``pad_slot``, a state row that
+    belongs to no request.
     """
 
-    def __init__(self, *, width: int, blocks: int, num_groups: int, tile_sizes, page_size: int, device):
+    def __init__(self, *, width: int, blocks: int, num_groups: int, tile_sizes, page_size: int, device, pad_slot: int = 0):
         S = width
+        self.pad_slot = pad_slot
         self.width = S
         self.blocks = blocks
         self.num_tokens = S
@@ -201,7 +204,7 @@ class StaticDecodeContext:
         self._set("token_ids", token_ids)
         self._set("positions", ctx_lens)
         self._set("ctx_lens", ctx_lens)
-        self._set("slots", slots)
+        self._set("slots", list(slots) + [self.pad_slot] * (self.width - len(slots)))
         for g, bt in enumerate(block_tables):
             o, n = self._offsets[f"bt{g}"]
             dst = self._np[o: o + n].reshape(self.width, self.blocks)

@@ -11,6 +11,7 @@ from ..kernels import ops
 from ..models.decoder import DecoderModel
 from ..registry import load_config
 from ..weights.loader import load_folder, load_into
+from .config import EngineConfig
 from .runner import ModelRunner
 
 DTYPES = {
@@ -56,8 +57,35 @@ def load_model(folder: str | Path, dtype="bfloat16", device=None) -> tuple[Model
     return config, build_model(config, dtype, device, folder=folder)
 
 
-def make_runner(model: DecoderModel, *, page_size: int, num_pages: int, max_requests: int,
-                use_graphs: bool = False) -> ModelRunner:
-    cache = CacheManager(model.cache_plan(), page_size=page_size, num_pages=num_pages,
-                         max_requests=max_requests, dtype=model.dtype, device=model.device)
-    return ModelRunner(model, cache, use_graphs=use_graphs)
+def make_runner(model: DecoderModel, config: EngineConfig | None = None, *, page_size: int | None = None,
+                num_pages: int | None = None, max_requests: int | None = None, use_graphs: bool | None = None,
+                max_model_len: int | None = None, max_step_tokens: int | None = None) -> ModelRunner:
+    """The step function over a cache of its own, from an :class:`EngineConfig` (the keywords override its
+    fields; ``max_requests`` is its ``max_slots``).  Without ``num_pages`` the pool holds a sequence of the
+    greatest length for every slot, as far as free memory goes.  ``max_step_tokens``: the caller's bound on
+    the tokens of a step (a scheduler's budget), which sizes the pools of windowed groups; ``None`` for
+    callers that step as they like."""
+    from dataclasses import replace
+    config = config or EngineConfig(dtype="float32" if model.dtype == torch.float32 else "bfloat16")
+    given = dict(page_size=page_size, num_pages=num_pages, max_slots=max_requests, use_graphs=use_graphs, max_model_len=max_model_len)
+    config = replace(config, **{k: v for k, v in given.items() if v is not None})
+    if parse_dtype(config.dtype) != model.dtype:
+        raise ValueError(f"the engine is configured for {config.dtype}, the model was built in {model.dtype}")
+    plan = model.cache_plan()
+    if config.num_pages is None:
+        probe = CacheManager(plan, page_size=config.page_size, num_pages=2, max_requests=1, dtype=model.dtype, device=None,
+                             max_step_tokens=max_step_tokens)
+        free = torch.cuda.mem_get_info(model.device)[0] if torch.device(model.device).type == "cuda" else None
+        config = config.resolve(model.spec.max_positions, probe.bytes_per_page(), free)
+    cache = CacheManager(plan, page_size=config.page_size, num_pages=config.num_pages, max_requests=config.max_slots,
+                         dtype=model.dtype, device=model.device, max_step_tokens=max_step_tokens)
+    runner = ModelRunner(model, cache, use_graphs=config.use_graphs, max_model_len=config.max_model_len)
+    runner.config = config
+    return runner
+
+
+def make_engine(model: DecoderModel, config: EngineConfig):
+    """Scheduler, step function and sampler over a cache, all sized by ``config``."""
+    from .engine import Engine
+    runner = make_runner(model, config, max_step_tokens=config.max_tokens_per_step if config.bounded_steps else None)
+    return Engine(runner, max_tokens_per_step=config.max_tokens_per_step, seed=config.seed, lookahead=config.lookahead)

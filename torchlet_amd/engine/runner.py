@@ -35,13 +35,14 @@ class ModelRunner:
     running, so results are only ever read after an eager run or a replay (the reference
     reads its output buffer right after capture, engine.py:165-176)."""
 
-    def __init__(self, model, cache: CacheManager, use_graphs: bool = False, max_graph_width: int = 256):
+    def __init__(self, model, cache: CacheManager, use_graphs: bool = False, max_graph_width: int = 256,
+                 max_model_len: int | None = None):
         self.model = model
         self.cache = cache
         self.device = model.device
         self.caches = [cache.layer_cache(i) for i in range(len(model.spec.order))]
         self.tile_sizes = model.tile_token_sizes()
-        self.max_positions = model.spec.max_positions
+        self.max_positions = model.spec.max_positions if max_model_len is None else min(max_model_len, model.spec.max_positions)
         self.vocab_size = model.spec.vocab_size
         self.use_graphs = use_graphs and torch.device(self.device).type == "cuda" and model.graph_safe()
         self.max_graph_width = max_graph_width
@@ -98,7 +99,7 @@ class ModelRunner:
                 cache.add_request(e.req_id)
                 added.append(e.req_id)
             if cache.length(e.req_id) + len(e.tokens) > self.max_positions:
-                raise ValueError(f"request {e.req_id!r} would pass max_position_embeddings ({self.max_positions})")
+                raise ValueError(f"request {e.req_id!r} would pass max_position_embeddings or the engine's max_model_len ({self.max_positions})")
         ctx_lens = [cache.length(e.req_id) for e in entries]
         new_lens = [len(e.tokens) for e in entries]
         # all-or-nothing over the whole step: check first, then take
@@ -148,7 +149,7 @@ class ModelRunner:
         if dg is None:
             dg = self._graphs[key] = _DecodeGraph(StaticDecodeContext(
                 width=width, blocks=bucket, num_groups=len(cache.groups), tile_sizes=self.tile_sizes,
-                page_size=cache.page_size, device=self.device))
+                page_size=cache.page_size, device=self.device, pad_slot=cache.pad_slot))
         dg.ctx.fill(token_ids=[e.tokens[0] for e in entries], ctx_lens=ctx_lens,
                     slots=[cache.slot(r) for r in req_ids],
                     block_tables=[cache.block_table(g, req_ids, bucket) for g in range(len(cache.groups))])

@@ -64,10 +64,9 @@ class Scheduler:
         if need > self.max_positions:
             raise ValueError(f"request {req.req_id} requires {need} cache positions, "
                              f"but max_position_embeddings is {self.max_positions}")
-        capacity = self.cache.num_pages - 1
-        pages = max(self.cache.pages_for(need) or [0])
-        if pages > capacity:
-            raise ValueError(f"request {req.req_id} needs {pages} cache pages for {need} tokens; the pool has {capacity}")
+        for pages, capacity in zip(self.cache.pages_for(need), self.cache.capacity()):
+            if pages > capacity:
+                raise ValueError(f"request {req.req_id} needs {pages} cache pages for {need} tokens; the pool has {capacity}")
 
     def add_request(self, req: Request) -> None:
         self.validate(req)

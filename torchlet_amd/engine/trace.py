@@ -41,6 +41,7 @@ def parse_args(argv=None):
 
 def run(args, lines, out=sys.stdout) -> int:
     from .batch import StepEntry
+    from .config import EngineConfig
     from .loading import load_model, make_runner
 
     if args.max_tokens <= 0 or args.page_size <= 0:
@@ -49,8 +50,8 @@ def run(args, lines, out=sys.stdout) -> int:
     out_dir.mkdir(parents=True, exist_ok=True)
     _, model = load_model(args.model, args.dtype)
     pages = -(-args.max_tokens // args.page_size) + 1          # + the sentinel page
-    runner = make_runner(model, page_size=args.page_size, num_pages=pages, max_requests=args.max_requests,
-                         use_graphs=args.graphs)
+    runner = make_runner(model, EngineConfig(page_size=args.page_size, num_pages=pages, max_slots=args.max_requests,
+                                             dtype=args.dtype, use_graphs=args.graphs))
     for line in lines:
         line = line.strip()
         if not line:

@@ -98,8 +98,8 @@ def _i32(t: torch.Tensor | None, what: str, n: int | None = None) -> None:
 
 # ----------------------------------------------------------------------------- ops
 
-def embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
-    """``out[t] = float(table[token_ids[t]])``; ``out`` is the 32-bit residual ``[T, H]``."""
+def embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """``out[t] = float(table[token_ids[t]]) * scale``; ``out`` is the 32-bit residual ``[T, H]``."""
     T = token_ids.numel()
     V, H = table.shape
     _i32(token_ids, "embedding ids", T)
@@ -107,12 +107,12 @@ def embedding(token_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -
         raise KernelError(f"embedding: out must be contiguous float32 [{T}, {H}], got {out.dtype} {tuple(out.shape)}")
     lib = _lib("elementwise")
     _check(lib, lib.tl_embedding(_ptr(token_ids), _ptr(table), c_int(_dt(table, "embedding table")), _ptr(out),
-                                 c_int(T), c_int(H), c_int(V), _stream()))
+                                 c_int(T), c_int(H), c_int(V), c_float(scale), _stream()))
 
 
 def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: torch.Tensor, eps: float,
-                out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
-    """``r = residual (+ pending)``; ``out = r * rsqrt(mean(r^2) + eps) * weight``.
+                out: torch.Tensor, rows: torch.Tensor | None = None, gain: float = 1.0) -> None:
+    """``r = residual (+ pending)``; ``out = r * (rsqrt(mean(r^2) + eps) * gain) * weight``.
 
     ``pending`` is ``[T, H]`` of the activation dtype, or float32 ``[P, T, H]``: slabs of partial
     sums (from :func:`linear_partials`) that are added up here.  Without ``rows`` every row is
@@ -136,7 +136,7 @@ def add_rmsnorm(residual: torch.Tensor, pending: torch.Tensor | None, weight: to
     wf = _vec(weight, H, "add_rmsnorm weight")
     lib = _lib("elementwise")
     _check(lib, lib.tl_add_rmsnorm(_ptr(residual), _ptr(pending), c_int(parts), c_int(T), _ptr(weight), c_int(wf),
-                                   c_float(eps), _ptr(out), _ptr(rows), c_int(n), c_int(H),
+                                   c_float(eps), c_float(gain), _ptr(out), _ptr(rows), c_int(n), c_int(H),
                                    c_int(_dt(out, "add_rmsnorm")), _stream()))
 
 
@@ -454,6 +454,7 @@ def _check_planes(what, k_plane, v_plane, dtype, kv_heads, page_size, head_dim) 
 
 
 ATTENTION_ROWS = 16   # rows (tokens x heads of one group) a work-group owns
+SPLIT_SCRATCH_BYTES = 256 << 20     # most memory the parts of a split attention may take before they are merged
 
 
 def attention_tile_tokens(num_heads: int, num_kv_heads: int) -> int:
@@ -497,6 +498,9 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
     if merge_tokens is not None:
         _i32(merge_tokens[0], "merge_tokens", merge_tokens[1])
     part_o = part_ml = None
+    # the parts are indexed by the step's tokens: a few decode tokens beside a long portion would make the
+    # scratch large for nothing, so the split count gives way (fewer parts: the same result up to rounding)
+    splits = max(1, min(splits, SPLIT_SCRATCH_BYTES // (T * num_heads * (head_dim + 2) * 4)))
     if splits > 1:
         part_o = torch.empty((T * num_heads * splits, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T * num_heads * splits, 2), dtype=torch.float32, device=q.device)
@@ -604,6 +608,7 @@ def paged_attention_prompt(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Te
         _i32(tokens, "merge_tokens")
         if tokens.numel() < count:
             raise KernelError("paged_attention_prompt: merge_tokens shorter than its count")
+        splits = max(1, min(splits, SPLIT_SCRATCH_BYTES // (T * num_heads * (head_dim + 2) * 4)))
         part_o = torch.empty((T * num_heads * splits, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T * num_heads * splits, 2), dtype=torch.float32, device=q.device)
     _check(lib, lib.tl_paged_attention_prompt(_ptr(q), c_int(q.stride(0)), _ptr(out), _ptr(k_plane), _ptr(v_plane),

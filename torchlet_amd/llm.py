@@ -8,8 +8,10 @@ tokens per cache page, ``max_num_blocks`` the pages of the pool including the se
 (default ``max_decode_slots * ceil(max_position_embeddings / kv_block_size) + 1``,
 engine.py:40-47 of the reference, capped by free GPU memory).  ``model_id`` is a local
 model folder (nothing is downloaded).  Additions: ``dtype``, ``max_num_batched_tokens`` (the
-step's token budget), ``seed``, ``use_graphs`` (decode-only steps replay a captured HIP graph); ``generate`` also takes ``temperature``, ``seed`` and
-``stop_token_ids``, and accepts prompts as lists of token ids, which bypass the tokenizer.
+step's token budget), ``max_model_len`` (sequences no longer than this: a smaller default pool), ``seed``,
+``use_graphs`` (decode-only steps replay a captured HIP graph); or all of them at once as an
+:class:`~torchlet_amd.engine.config.EngineConfig` (``engine_config=``).  ``generate`` also takes ``temperature``,
+``seed`` and ``stop_token_ids``, and accepts prompts as lists of token ids, which bypass the tokenizer.
 
 Strings are wrapped as a single user turn and run through the tokenizer's chat template
 with the generation prompt (llm.py:87-96); the stop ids are the tokenizer's end-of-sequence
@@ -25,41 +27,35 @@ from __future__ import annotations
 import argparse
 import asyncio
 import json
-import math
 import sys
 from pathlib import Path
 
 import torch
 
-from .engine.engine import Engine
-from .engine.loading import load_model, make_runner, require_gpu
+from .engine.config import EngineConfig
+from .engine.loading import load_model, make_engine, require_gpu
 from .engine.request import Request
 
 
 class LLM:
     def __init__(self, model_id: str, max_decode_slots: int = 4, kv_block_size: int = 16,
                  max_num_blocks: int | None = None, *, dtype: str = "bfloat16",
-                 max_num_batched_tokens: int = 2048, seed: int = 0, use_graphs: bool = True,
-                 lookahead: bool = True):
+                 max_num_batched_tokens: int = 2048, max_model_len: int | None = None, seed: int = 0,
+                 use_graphs: bool = True, lookahead: bool = True, engine_config: EngineConfig | None = None):
         self.device = require_gpu()
         if kv_block_size <= 0:
             raise ValueError("kv_block_size must be positive")
         if max_decode_slots <= 0:
             raise ValueError("max_decode_slots must be positive")
+        self.engine_config = engine_config or EngineConfig(
+            page_size=kv_block_size, num_pages=max_num_blocks, max_slots=max_decode_slots,
+            max_tokens_per_step=max_num_batched_tokens, max_model_len=max_model_len, dtype=str(dtype).replace("torch.", ""),
+            use_graphs=use_graphs, lookahead=lookahead, seed=seed)
         self.model_dir = Path(model_id)
-        self.config, self.model = load_model(self.model_dir, dtype, self.device)
-        spec = self.model.spec
-        blocks_per_request = math.ceil(spec.max_positions / kv_block_size)
-        if max_num_blocks is None:
-            max_num_blocks = max_decode_slots * blocks_per_request + 1
-            probe = make_runner(self.model, page_size=kv_block_size, num_pages=2, max_requests=1)
-            per_page = max(1, probe.cache.bytes_per_page())
-            del probe
-            free, _ = torch.cuda.mem_get_info(self.device)
-            max_num_blocks = max(2, min(max_num_blocks, int(free * 0.8) // per_page))
-        self.runner = make_runner(self.model, page_size=kv_block_size, num_pages=max_num_blocks,
-                                  max_requests=max_decode_slots, use_graphs=use_graphs)
-        self.engine = Engine(self.runner, max_tokens_per_step=max_num_batched_tokens, seed=seed, lookahead=lookahead)
+        self.config, self.model = load_model(self.model_dir, self.engine_config.dtype, self.device)
+        self.engine = make_engine(self.model, self.engine_config)
+        self.runner = self.engine.runner
+        self.engine_config = self.runner.config            # with the number of pages filled in
         self.tokenizer = _load_tokenizer(self.model_dir)
         self.stop_ids = self._stop_ids()
         self._next_seed = 0
@@ -207,6 +203,7 @@ def _parser():
         q.add_argument("--kv-block-size", type=int, default=16)
         q.add_argument("--max-num-blocks", type=int, default=None)
         q.add_argument("--max-num-batched-tokens", type=int, default=2048)
+        q.add_argument("--max-model-len", type=int, default=None, help="sequences no longer than this (default: the model's limit)")
     i = sub.add_parser("init", help="write a model folder with random weights from a configuration and a seed")
     i.add_argument("--config", required=True, help="a config.json")
     i.add_argument("--seed", type=int, default=0)
@@ -235,7 +232,7 @@ def main(argv=None) -> int:
         return 2
     llm = LLM(args.model, max_decode_slots=args.max_decode_slots, kv_block_size=args.kv_block_size,
               max_num_blocks=args.max_num_blocks, dtype=args.dtype,
-              max_num_batched_tokens=args.max_num_batched_tokens, seed=args.seed)
+              max_num_batched_tokens=args.max_num_batched_tokens, max_model_len=args.max_model_len, seed=args.seed)
     outputs = llm.generate(prompts, max_new_tokens=args.max_new_tokens, temperature=args.temperature, seed=0)
     for prompt, out in zip(prompts, outputs):
         print(json.dumps({"prompt": prompt, "output": out}))

@@ -1,7 +1,9 @@
 """A decoder built from a :class:`~torchlet_amd.config.base.ModelSpec`.
 
-embedding -> the runs of the layer order -> final norm on the wanted rows -> LM head
-(/root/reference/src/torchlet/v10_triton_paged_gqa/model/qwen2_5.py:55-87).  The class
+embedding (times ``embed_scale``) -> the runs of the layer order -> final norm on the wanted rows
+(times ``logit_scale``) -> LM head (plus its bias, if the specification says it has one)
+(/root/reference/src/torchlet/v10_triton_paged_gqa/model/qwen2_5.py:55-87, where the factors are 1 and
+there is no bias).  The class
 knows nothing of any architecture: which parts a layer has, their sizes, the names of
 their tensors and the order of the runs all come from the specification.
 """
@@ -25,6 +27,7 @@ class DecoderModel:
         self.final_norm = NORMS.build(spec.final_norm, dtype, self.device)
         self.embed: torch.Tensor | None = None
         self.head: torch.Tensor | None = None
+        self.head_bias: torch.Tensor | None = None
 
     # ------------------------------------------------------------------ weights
     def weight_specs(self) -> dict[str, WeightSpec]:
@@ -37,6 +40,8 @@ class DecoderModel:
             specs[f"{s.final_norm_name}.{k}"] = v
         # a tied head is the embedding matrix; a checkpoint may still carry a copy of it
         specs[f"{s.head_name}.weight"] = WeightSpec((s.vocab_size, s.hidden), optional=s.tie_head)
+        if s.head_bias:
+            specs[f"{s.head_name}.bias"] = WeightSpec((s.vocab_size,), role="vector")
         return specs
 
     def load_weights(self, tensors: dict[str, torch.Tensor]) -> None:
@@ -52,6 +57,11 @@ class DecoderModel:
             self.head = self.embed
         else:
             self.head = tensors[f"{s.head_name}.weight"].to(device=self.device, dtype=self.dtype).contiguous()
+        if s.head_bias:
+            b = tensors[f"{s.head_name}.bias"]
+            if self.dtype == torch.float32 or b.dtype not in (torch.bfloat16, torch.float32):
+                b = b.to(torch.float32)
+            self.head_bias = b.to(self.device).contiguous()
 
     # ------------------------------------------------------------------ cache needs
     def cache_plan(self):
@@ -83,13 +93,13 @@ class DecoderModel:
         when no row is wanted)."""
         T = ctx.num_tokens
         residual = torch.empty((T, self.spec.hidden), dtype=torch.float32, device=self.device)
-        ops.embedding(ctx.token_ids, self.embed, residual)
+        ops.embedding(ctx.token_ids, self.embed, residual, self.spec.embed_scale)
         stream = Stream(residual)
         for i, e in enumerate(self.spec.order):
             stream = self.blocks[e.layer].forward(stream, ctx, caches[i])
         if ctx.want_rows is None or ctx.num_wanted == 0:
             return None
-        h = self.final_norm.forward(stream, rows=ctx.want_rows)
+        h = self.final_norm.forward(stream, rows=ctx.want_rows, gain=self.spec.logit_scale)
         logits = torch.empty((ctx.num_wanted, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-        ops.linear(h, self.head, None, logits)
+        ops.linear(h, self.head, self.head_bias, logits)
         return logits

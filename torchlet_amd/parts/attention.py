@@ -4,7 +4,7 @@ Formulas (/root/reference/src/torchlet/v10_triton_paged_gqa/layer/gqa.py:112-146
 kernel/gqa.py:58-111): ``q = h Wq^T + bq`` and likewise k, v; heads are split head-major
 (feature ``= head * head_dim + d``); q and k are position-encoded; the encoded k and the
 raw v of every new token are stored in the cache; query head ``i`` reads KV head
-``i // (heads / kv_heads)``; scores are scaled by ``head_dim ** -0.5``, masked causally
+``i // (heads / kv_heads)``; scores are scaled by ``head_dim ** -0.5`` (or the specification's ``scale``), masked causally
 (and to the last ``window`` keys if the layer has a window), soft-maxed in 32-bit, and
 the weighted values go through ``o_proj`` (no bias).
 
@@ -50,7 +50,7 @@ class GQAttention(Mixer):
         self.kv_heads = spec.num_kv_heads
         self.head_dim = spec.head_dim
         self.window = spec.window
-        self.scale = float(spec.head_dim) ** -0.5
+        self.scale = float(spec.head_dim) ** -0.5 if spec.scale is None else float(spec.scale)
         self.q_width = self.heads * self.head_dim
         self.kv_width = self.kv_heads * self.head_dim
         self.qkv_bias = spec.qkv_bias
@@ -89,7 +89,7 @@ class GQAttention(Mixer):
         # then rotates in its own epilogue.  Keys lie in the cache in that order too; scores are
         # sums over a head's dimensions and do not notice.
         self.pair_layout = (self.dtype == torch.bfloat16 and self.position is not None
-                            and hasattr(self.position, "fused_inv_freq"))
+                            and self.position.fused_inv_freq() is not None)
         rows = {"q": ops.pair_layout_rows(self.heads, self.head_dim), "k": ops.pair_layout_rows(self.kv_heads, self.head_dim)}
         order = lambda n, t: t[rows[n]] if self.pair_layout and n in rows else t
         self.w_qkv = self._place(torch.cat([order(n, tensors[f"{n}_proj.weight"]) for n in "qkv"], dim=0), "matrix")
@@ -129,7 +129,7 @@ class GQAttention(Mixer):
         v_plane = v_plane.view(v_plane.shape[0], self.kv_heads, self.head_dim, cache.page_size)
         table = ctx.block_tables[cache.group]
         kv_heads = self.kv_heads if writes else 0
-        inv_freq = self.position.fused_inv_freq() if hasattr(self.position, "fused_inv_freq") else None
+        inv_freq = self.position.fused_inv_freq() if self.position is not None else None
         cache_args = (ctx.token_req, table, k_plane, v_plane, cache.page_size) if writes else (None, None, None, None, 0)
         fused = False
         if lazy is not None:

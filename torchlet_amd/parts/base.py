@@ -75,13 +75,23 @@ class Part:
 
 @dataclass(frozen=True)
 class PagedNeed:
-    """Per-token cache: ``planes`` tensors of ``[num_heads, head_dim]`` per token
-    (keys and values are two planes), kept for all tokens (``window=None``) or for the
-    last ``window`` tokens.  Layers with equal needs share a group of pages."""
+    """Per-token cache: some planes of ``[heads, width]`` per token, kept for all tokens
+    (``window=None``) or for the last ``window`` tokens.  ``planes`` is a count of planes of
+    ``[num_heads, head_dim]`` each (keys and values are two), or a tuple of ``(heads, width)``, one per
+    plane, for planes that differ (a compressed latent beside a small rotated part).  ``dtype``: the
+    planes' element type; ``None`` is the model's.  Layers with equal needs share a group of pages."""
     num_heads: int
     head_dim: int
     window: int | None = None
-    planes: int = 2
+    planes: int | tuple[tuple[int, int], ...] = 2
+    dtype: torch.dtype | None = None
+
+    @property
+    def plane_shapes(self) -> tuple[tuple[int, int], ...]:
+        """``(heads, width)`` of every plane."""
+        if isinstance(self.planes, int):
+            return ((self.num_heads, self.head_dim),) * self.planes
+        return tuple((int(h), int(w)) for h, w in self.planes)
 
 
 @dataclass(frozen=True)
@@ -141,10 +151,11 @@ class LazyNorm:
 # ----------------------------------------------------------------------- part kinds
 
 class Norm(Part):
-    def forward(self, stream: Stream, rows: torch.Tensor | None = None) -> torch.Tensor:
+    def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0) -> torch.Tensor:
         """Add ``stream.pending`` into ``stream.residual`` (both kept up to date) and
-        return ``norm(residual)`` in the activation dtype.  With ``rows`` (int32 indices)
-        only those rows are read and returned, and the stream is left untouched."""
+        return ``norm(residual) * gain`` in the activation dtype (the factor applied in 32-bit, before
+        the one rounding of the result).  With ``rows`` (int32 indices) only those rows are read
+        and returned, and the stream is left untouched."""
         raise NotImplementedError
 
     def lazy(self, stream: Stream) -> "LazyNorm | None":
@@ -158,6 +169,14 @@ class PositionEncoding(Part):
         """Encode ``positions [T]`` into ``q [T, heads, head_dim]`` and ``k`` in place
         (views with unit stride on the last axis)."""
         raise NotImplementedError
+
+    def fused_inv_freq(self) -> torch.Tensor | None:
+        """A declared capability: an encoding that is the split-half rotary form over the whole head,
+        ``angle[j] = float32(position) * inv_freq[j]`` turning the pair ``(j, j + head_dim/2)``, returns its
+        float32 ``inv_freq [head_dim/2]`` here, and a mixer may then fold the rotation into its own kernels
+        (the projection's epilogue, the cache write) instead of calling :meth:`apply`.  ``None`` (the
+        default): the encoding is applied through :meth:`apply` only."""
+        return None
 
 
 class Mixer(Part):

@@ -27,10 +27,10 @@ class RMSNorm(Norm):
     def load_weights(self, tensors):
         self.weight = self._place(tensors["weight"], "vector")
 
-    def forward(self, stream: Stream, rows: torch.Tensor | None = None) -> torch.Tensor:
+    def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0) -> torch.Tensor:
         n = stream.residual.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.dim), dtype=self.dtype, device=stream.residual.device)
-        ops.add_rmsnorm(stream.residual, stream.pending, self.weight, self.eps, out, rows)
+        ops.add_rmsnorm(stream.residual, stream.pending, self.weight, self.eps, out, rows, gain)
         if rows is None:
             stream.pending = None
         return out

@@ -1,29 +1,32 @@
 #!/usr/bin/python3
-"""Benchmark of the serving step on one MI355X: decode throughput, prefill throughput, rooflines.
+"""Benchmark of serving on one MI355X: decode throughput, prefill throughput, rooflines.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16]
-                    [--shape 7b|14b|32b] [--context N] [--prefill-tokens T] [--workload decode|serve]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16]
+                    [--shape 7b|14b|32b] [--context N] [--new-tokens G] [--prefill-tokens T]
+                    [--workload decode|serve] [--only decode|step|prefill] [--all]
 
-The default run has the layer sizes of Qwen2.5-7B (28 layers, hidden 3584, 28 heads, 4 KV
-heads, head size 128, intermediate 18944, vocabulary 152064) with random weights, a batch
-of 8 requests that each hold a 2048-token context, and times K decode steps (one new token
-per request and step, sampled greedily) through the engine's own step function and sampler.
-It prints ONE JSON line; ``value`` is decoded tokens per second.  The same line carries
+The default run has the layer sizes of Qwen2.5-7B (28 layers, hidden 3584, 28 heads, 4 KV heads, head
+size 128, intermediate 18944, vocabulary 152064) with random weights and goes through the whole engine
+(scheduler, step function with decode steps replayed as HIP graphs and enqueued one ahead, sampler):
+8 requests with 2048-token random prompts are prefilled by the engine and generate up to 256 tokens
+each, greedily, with no stop token; after W untimed decode steps exactly K decode steps are timed.  It
+prints ONE JSON line; ``value`` is decoded tokens per second.  Every figure of the line can be
+recomputed from its own fields.  The same line carries
 
-* ``prefill``: one 2048-token prompt in one step (tokens/s, ms, fraction of the dense
-  matrix-core peak of the dtype: flops / time / peak),
-* ``roofline``: bytes a decode step has to read (every weight it uses once, plus the cache
-  of the live requests) / its time, against the 8 TB/s of HBM3E,
-* ``points``: decode tokens/s at batch 1 and batch 64.
+* ``roofline``: the bytes a decode step has to read (``bytes_per_step``: every weight it uses once,
+  the embedding rows of the batch, and the cache of the live requests at their mean length over the timed
+  steps) / its time, against the 8 TB/s of HBM3E (``frac``) and against the rate at which this GPU
+  delivers memory to a kernel that only reads (``frac_measured``; ``measured`` holds that yardstick);
+* ``step_function``: the same decode step driven directly (no scheduler): what the scheduler costs;
+* ``prefill``: one 2048-token prompt in one step (tokens/s, ms, flops, ``frac`` of the dense matrix-core
+  peak of the dtype, ``frac_measured`` of the rate this repository's own large matrix product reaches);
+* ``points``: decode tokens/s at batch 1 and batch 64 through the engine; ``points_detail`` gives each
+  point's ms per step, bytes per step and fractions.
 
-Caches of the decode runs are filled with random keys and values of 2048-token contexts
-through the cache manager (the time of a decode step does not depend on their values).
-
-Other layer sizes (``--shape 14b``, ``32b``), context lengths and prompt lengths measure the same
-step at further sizes.  ``--workload serve`` runs requests through the whole engine instead
-(scheduler, prompt portions under a token budget beside decode tokens, sampler): ``--requests``
-prompts of random lengths in ``[--prompt-min, --prompt-max]``, ``--new-tokens`` each, at most
-``--portion`` tokens per step, and prints a line of its own.
+``--all`` adds the secondary workloads as ``extra``: Qwen2.5-14B sizes served through the scheduler
+(32 requests, prompts 128-4096, 128 new tokens, 512 tokens a step), and Qwen2.5-32B sizes (prefill of
+16384 tokens, decode at batch 1 on that context and at batch 16 on 4096-token contexts).
+``--workload serve`` prints the serving run alone as a line of its own.
 """
 from __future__ import annotations
 
@@ -50,29 +53,33 @@ SHAPES = {
                                  max_position_embeddings=32768)),
 }
 CONTEXT = 2048
+NEW_TOKENS = 256
 PAGE = 16
+PREFILL_BUDGET = 8192        # tokens a step of the engine may hold: four 2048-token prompts are prefilled at a time
 
 
 def parse_args(argv=None):
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=64)
-    p.add_argument("--warmup", type=int, default=8)
+    p.add_argument("--steps", type=int, default=224, help="timed decode steps")
+    p.add_argument("--warmup", type=int, default=8, help="untimed decode steps before them")
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--shape", choices=list(SHAPES), default="7b", help="layer sizes")
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
-    p.add_argument("--context", type=int, default=CONTEXT, help="cached tokens of each request in the decode runs")
+    p.add_argument("--context", type=int, default=CONTEXT, help="prompt tokens of each request in the decode runs")
+    p.add_argument("--new-tokens", type=int, default=None, help="tokens each request may generate (decode: 256, serve: 128)")
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--workload", choices=["decode", "serve"], default="decode")
     p.add_argument("--requests", type=int, default=32)
     p.add_argument("--prompt-min", type=int, default=128)
     p.add_argument("--prompt-max", type=int, default=4096)
-    p.add_argument("--new-tokens", type=int, default=128)
     p.add_argument("--portion", type=int, default=512, help="serve: token budget of a step")
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    p.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
-    p.add_argument("--only", choices=["decode", "prefill"], default=None,
-                   help="run one part only (for profiling): the decode steps at --batch, or the 2048-token prefill")
+    p.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points, the prefill and the yardsticks")
+    p.add_argument("--only", choices=["decode", "step", "prefill"], default=None,
+                   help="run one part only (for profiling): the engine's decode steps at --batch, the bare step function's, "
+                        "or the prefill")
+    p.add_argument("--all", action="store_true", help="add the secondary workloads (14B served, 32B prefill and decode)")
     return p.parse_args(argv)
 
 
@@ -93,9 +100,9 @@ def build(shape: str, layers: int, dtype: str):
 
 
 def decode_bytes(cfg, model, batch: int, context: float) -> float:
-    """Bytes one decode step must read: every weight once (the embedding only ``batch`` rows
-    of it) and the keys and values of the live requests."""
-    esize = 2 if model.dtype.__str__().endswith("bfloat16") else 4
+    """Bytes one decode step must read: every weight once (of the embedding only ``batch`` rows)
+    and the keys and values of the live requests, ``context`` tokens each."""
+    esize = 2 if str(model.dtype).endswith("bfloat16") else 4
     h, i, v = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
     per_layer = qkv * h + qkv + cfg.num_attention_heads * cfg.head_dim * h + 3 * h * i + 2 * h
@@ -112,9 +119,62 @@ def prefill_flops(cfg, tokens: int) -> float:
     return 2.0 * tokens * linear + attn + 2.0 * v * h
 
 
+def random_prompts(vocab: int, count: int, length: int, seed: int = 0):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, vocab, (length,), generator=g).tolist() for _ in range(count)]
+
+
+def engine_decode(cfg, model, batch: int, steps: int, warmup: int, context: int, new_tokens: int) -> dict:
+    """``batch`` requests with ``context``-token random prompts through the whole engine: the prompts are
+    prefilled by the scheduler (portions under its token budget), then every step decodes one token for each
+    request.  ``warmup`` decode steps are left untimed (they capture the graphs), ``steps`` are timed.
+    No stop token; nobody may finish before the timed steps are over."""
+    import torch
+    from torchlet_amd.engine.config import EngineConfig
+    from torchlet_amd.engine.loading import make_engine
+    from torchlet_amd.engine.request import Request
+
+    pages = batch * (-(-(context + new_tokens) // PAGE)) + 1
+    engine = make_engine(model, EngineConfig(page_size=PAGE, num_pages=pages, max_slots=batch, max_tokens_per_step=max(PREFILL_BUDGET, batch),
+                                             dtype="float32" if model.dtype == torch.float32 else "bfloat16", use_graphs=True,
+                                             lookahead=True, seed=0))
+    reqs = [Request(prompt_tokens=p, max_new_tokens=new_tokens, temperature=0.0, stop_token_ids=frozenset())
+            for p in random_prompts(cfg.vocab_size, batch, context)]
+    engine.add_requests(reqs)
+    finished = []
+    while any(not r.output_tokens for r in reqs):          # the prefill phase (with decode tokens of those already through)
+        finished += engine.step()
+    ahead = max(len(r.output_tokens) for r in reqs)
+    if ahead + warmup + steps >= new_tokens:
+        raise SystemExit(f"bench.py: {warmup} + {steps} decode steps after a prefill phase in which a request already generated "
+                         f"{ahead} tokens do not fit {new_tokens} new tokens; lower --steps or raise --new-tokens")
+    for _ in range(warmup):
+        finished += engine.step()
+    torch.cuda.synchronize()
+    before = [len(r.output_tokens) for r in reqs]
+    ctx0 = sum(r.computed_tokens for r in reqs) / batch
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        finished += engine.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ctx1 = sum(r.computed_tokens for r in reqs) / batch
+    generated = sum(len(r.output_tokens) - b for r, b in zip(reqs, before))
+    assert not finished and generated == batch * steps, (len(finished), generated)
+    replays, ahead_steps = engine.runner.graph_replays, engine.steps_ahead
+    engine.shutdown()
+    del engine
+    torch.cuda.empty_cache()
+    ms = dt * 1e3 / steps
+    mean_ctx = (ctx0 + ctx1) / 2.0 + 0.5      # keys a request's token attends to (its own included), averaged over the timed steps
+    nbytes = decode_bytes(cfg, model, batch, mean_ctx)
+    return {"batch": batch, "steps": steps, "ms_per_step": round(ms, 4), "tokens_per_s": round(batch * 1e3 / ms, 2),
+            "mean_context": round(mean_ctx, 1), "bytes_per_step": int(nbytes), "graph_replays": replays, "steps_ahead": ahead_steps}
+
+
 def fill_context(runner, req_ids, context: int):
     """Give every request ``context`` cached tokens with random keys and values."""
-    import torch
     cache = runner.cache
     for r in req_ids:
         cache.add_request(r)
@@ -126,8 +186,10 @@ def fill_context(runner, req_ids, context: int):
             plane.normal_(0.0, 0.5)
 
 
-def time_decode(model, batch: int, steps: int, warmup: int, context: int = CONTEXT):
-    """ms per decode step at ``batch`` requests of ``context`` cached tokens each."""
+def step_function_decode(cfg, model, batch: int, steps: int, warmup: int, context: int) -> dict:
+    """The decode step without the scheduler: the step function and the sampler driven directly, each step
+    taking its tokens on the GPU from the sampling of the one before, on caches filled with random keys and
+    values of ``context`` tokens (the time of a decode step does not depend on their values)."""
     import torch
     from torchlet_amd.engine.batch import StepEntry
     from torchlet_amd.engine.loading import make_runner
@@ -139,8 +201,6 @@ def time_decode(model, batch: int, steps: int, warmup: int, context: int = CONTE
     fill_context(runner, ids, context)
     sampler = Sampler(0)
     zeros = [0.0] * batch
-    # As the engine runs decode steps: a step takes its tokens on the GPU from the sampling of the step
-    # before it and is enqueued while the host still waits for those tokens; every token is read.
     logits = runner.step([StepEntry(r, [1 + i], [0]) for i, r in enumerate(ids)])
     drawn = sampler.launch(logits, zeros, zeros, zeros)
     entries = [StepEntry(r, [0], [0]) for r in ids]
@@ -164,22 +224,26 @@ def time_decode(model, batch: int, steps: int, warmup: int, context: int = CONTE
     assert len(generated) == warmup + steps and all(len(t) == batch for t in generated)
     del runner
     torch.cuda.empty_cache()
-    return ms
+    mean_ctx = context + 1 + warmup + steps / 2.0
+    return {"batch": batch, "steps": steps, "ms_per_step": round(ms, 4), "tokens_per_s": round(batch * 1e3 / ms, 2),
+            "mean_context": round(mean_ctx, 1), "bytes_per_step": int(decode_bytes(cfg, model, batch, mean_ctx))}
 
 
-def time_prefill(model, tokens: int, repeats: int = 3):
+def time_prefill(model, tokens: int, repeats: int = 3, context: int = 0):
+    """ms of one step that brings ``tokens`` prompt tokens (after ``context`` tokens fed in 2048-token steps)."""
     import torch
     from torchlet_amd.engine.batch import StepEntry
     from torchlet_amd.engine.loading import make_runner
 
-    runner = make_runner(model, page_size=PAGE, num_pages=-(-tokens // PAGE) + 2, max_requests=1)
-    g = torch.Generator().manual_seed(0)
-    prompt = torch.randint(0, model.spec.vocab_size, (tokens,), generator=g).tolist()
+    runner = make_runner(model, page_size=PAGE, num_pages=-(-(context + tokens) // PAGE) + 2, max_requests=1)
+    prompt = random_prompts(model.spec.vocab_size, 1, context + tokens)[0]
     best = float("inf")
     for i in range(repeats + 1):
+        for a in range(0, context, 2048):
+            runner.step([StepEntry("p", prompt[a:min(a + 2048, context)], [])])
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        runner.step([StepEntry("p", prompt, [tokens - 1])])
+        runner.step([StepEntry("p", prompt[context:], [tokens - 1])])
         torch.cuda.synchronize()
         dt = (time.perf_counter() - t0) * 1e3
         runner.release("p")
@@ -190,40 +254,85 @@ def time_prefill(model, tokens: int, repeats: int = 3):
     return best
 
 
+def _best_ms(launch, rounds: int = 5, calls: int = 10) -> float:
+    """ms of one call of ``launch``: ``calls`` of them back to back between two events (so that the host's
+    part in a launch does not count), best of ``rounds`` after a warm-up round."""
+    import torch
+    best = float("inf")
+    for i in range(rounds + 1):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(calls):
+            launch()
+        end.record()
+        torch.cuda.synchronize()
+        if i:
+            best = min(best, start.elapsed_time(end) / calls)
+    return best
+
+
+def measure_stream_read_gbs() -> float:
+    """GB/s at which a kernel that only reads gets 2 GiB from memory (far more than the caches hold)."""
+    import torch
+    from torchlet_amd.kernels import ops
+    data = torch.empty(2 << 30, dtype=torch.uint8, device="cuda")
+    data.random_(0, 255)
+    ms = _best_ms(lambda: ops.stream_read(data))
+    del data
+    torch.cuda.empty_cache()
+    return (2 << 30) / (ms * 1e-3) / 1e9
+
+
+def measure_gemm_tflops(dtype) -> float:
+    """TFLOP/s of this repository's own matrix product at 8192 x 8192 x 8192 (float32: 4096 cubed)."""
+    import torch
+    from torchlet_amd.kernels import ops
+    n = 8192 if dtype == torch.bfloat16 else 4096
+    x = torch.randn((n, n), device="cuda").to(dtype)
+    w = torch.randn((n, n), device="cuda").to(dtype)
+    out = torch.empty((n, n), dtype=dtype, device="cuda")
+    ms = _best_ms(lambda: ops.linear(x, w, None, out), rounds=3, calls=4)
+    del x, w, out
+    torch.cuda.empty_cache()
+    return 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+
+
 def serve(cfg, model, args) -> dict:
     """Requests through the whole engine: prompts of seeded random lengths, all arriving at
     once, cut into portions under the step's token budget beside the decode tokens of the
     requests that are further on; every request generates ``--new-tokens`` (no stop ids)."""
     import torch
-    from torchlet_amd.engine.engine import Engine
-    from torchlet_amd.engine.loading import make_runner
+    from torchlet_amd.engine.config import EngineConfig
+    from torchlet_amd.engine.loading import make_engine
     from torchlet_amd.engine.request import Request
 
     g = torch.Generator().manual_seed(1)
     lengths = torch.randint(args.prompt_min, args.prompt_max + 1, (args.requests,), generator=g).tolist()
     prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in lengths]
-    pages = sum(-(-(n + args.new_tokens) // PAGE) for n in lengths) + 1
-    runner = make_runner(model, page_size=PAGE, num_pages=pages, max_requests=args.requests, use_graphs=True)
-    engine = Engine(runner, max_tokens_per_step=args.portion, seed=0)
+    new_tokens = args.serve_new_tokens
+    pages = sum(-(-(n + new_tokens) // PAGE) for n in lengths) + 1
+    engine = make_engine(model, EngineConfig(page_size=PAGE, num_pages=pages, max_slots=args.requests, max_tokens_per_step=args.portion,
+                                             dtype=args.dtype, use_graphs=True, seed=0))
 
     def run():
-        for p in prompts:
-            engine.add_request(Request(prompt_tokens=list(p), max_new_tokens=args.new_tokens))
+        engine.add_requests([Request(prompt_tokens=list(p), max_new_tokens=new_tokens) for p in prompts])
         steps0 = engine.steps
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         done = engine.run_until_done()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        assert len(done) == len(prompts) and all(len(r.output_tokens) == args.new_tokens for r in done)
+        assert len(done) == len(prompts) and all(len(r.output_tokens) == new_tokens for r in done)
         return dt, engine.steps - steps0
 
     run()                                   # warms up kernels and captures the decode graphs
     dt, steps = run()
-    generated = args.requests * args.new_tokens
+    generated = args.requests * new_tokens
+    del engine
+    torch.cuda.empty_cache()
     return {
         "metric": f"served tokens/s, {SHAPES[args.shape][0]} shape, {args.requests} requests, prompts {args.prompt_min}-{args.prompt_max}, "
-                  f"{args.new_tokens} new tokens each, at most {args.portion} tokens a step, one MI355X",
+                  f"{new_tokens} new tokens each, at most {args.portion} tokens a step, one MI355X",
         "value": round((sum(lengths) + generated) / dt, 1), "unit": "tokens/s (prompt + generated)",
         "generated_tokens_per_s": round(generated / dt, 1), "prompt_tokens": sum(lengths), "generated_tokens": generated,
         "seconds": round(dt, 3), "engine_steps": steps, "ms_per_step": round(dt * 1e3 / steps, 3),
@@ -232,8 +341,65 @@ def serve(cfg, model, args) -> dict:
     }
 
 
+def secondary(args) -> dict:
+    """The secondary workloads, each at its full layer count: 14B sizes served, 32B sizes prefilled and decoded."""
+    import torch
+    out = {}
+    cfg, model = build("14b", SHAPES["14b"][1]["num_hidden_layers"], args.dtype)
+    a = argparse.Namespace(**vars(args))
+    a.shape, a.requests, a.prompt_min, a.prompt_max, a.serve_new_tokens, a.portion = "14b", 32, 128, 4096, 128, 512
+    s = serve(cfg, model, a)
+    out["serve_14b"] = {k: s[k] for k in ("value", "unit", "generated_tokens_per_s", "prompt_tokens", "generated_tokens", "seconds",
+                                           "engine_steps", "ms_per_step", "layers")}
+    del model
+    torch.cuda.empty_cache()
+    cfg, model = build("32b", SHAPES["32b"][1]["num_hidden_layers"], args.dtype)
+    tokens = 16384
+    # the long prompt in 2048-token steps, as the engine's budget would cut it: the sum of the steps' times
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import make_runner
+    runner = make_runner(model, page_size=PAGE, num_pages=-(-tokens // PAGE) + 2, max_requests=1)
+    prompt = random_prompts(cfg.vocab_size, 1, tokens)[0]
+    best = float("inf")
+    for rep in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for a0 in range(0, tokens, 2048):
+            runner.step([StepEntry("p", prompt[a0:a0 + 2048], [2047] if a0 + 2048 == tokens else [])])
+        torch.cuda.synchronize()
+        total = time.perf_counter() - t0
+        runner.release("p")
+        if rep:
+            best = min(best, total)
+    del runner
+    torch.cuda.empty_cache()
+    flops = sum(prefill_flops_step(cfg, 2048, a0) for a0 in range(0, tokens, 2048))
+    out["prefill_32b_16384"] = {"tokens": tokens, "steps_of": 2048, "ms": round(best * 1e3, 2), "value": round(tokens / best, 1),
+                                "flops": flops, "frac": round(flops / best / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12), 4),
+                                "layers": cfg.num_hidden_layers}
+    for name, batch, context, steps in (("decode_32b_b1_ctx16384", 1, 16384, 32), ("decode_32b_b16_ctx4096", 16, 4096, 32)):
+        r = step_function_decode(cfg, model, batch, steps, 4, context)
+        gbs = r["bytes_per_step"] / (r["ms_per_step"] * 1e-3) / 1e9
+        out[name] = dict(r, achieved_gbs=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 4), layers=cfg.num_hidden_layers)
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
+def prefill_flops_step(cfg, tokens: int, context: int) -> float:
+    """Flops of a step of ``tokens`` prompt tokens on top of ``context`` cached ones (no logits)."""
+    h, i = cfg.hidden_size, cfg.intermediate_size
+    qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
+    linear = cfg.num_hidden_layers * (qkv * h + cfg.num_attention_heads * cfg.head_dim * h + 3 * h * i)
+    keys = tokens * context + tokens * tokens / 2.0
+    attn = cfg.num_hidden_layers * 4 * cfg.num_attention_heads * cfg.head_dim * keys
+    return 2.0 * tokens * linear + attn
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
+    args.serve_new_tokens = args.new_tokens or 128
+    args.new_tokens = args.new_tokens or NEW_TOKENS
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not built (this engine runs on a single MI355X)")
         return 2
@@ -246,12 +412,16 @@ def main(argv=None) -> int:
     layers = args.layers if args.layers is not None else full_layers
     cfg, model = build(args.shape, layers, args.dtype)
     ptokens = args.prefill_tokens
+    peak_tflops = MFMA_PEAK_TFLOPS[args.dtype]
 
-    def prefill_point():
+    def prefill_point(gemm_tflops=None):
         pms = time_prefill(model, ptokens)
         flops = prefill_flops(cfg, ptokens)
-        return {"value": round(ptokens * 1e3 / pms, 1), "tokens": ptokens, "ms": round(pms, 3),
-                "frac": round(flops / (pms * 1e-3) / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12), 4)}
+        point = {"value": round(ptokens * 1e3 / pms, 1), "tokens": ptokens, "ms": round(pms, 3), "flops": flops,
+                 "frac": round(flops / (pms * 1e-3) / (peak_tflops * 1e12), 4)}
+        if gemm_tflops:
+            point["frac_measured"] = round(flops / (pms * 1e-3) / (gemm_tflops * 1e12), 4)
+        return point
 
     if args.workload == "serve":
         print(json.dumps(serve(cfg, model, args)))
@@ -259,43 +429,67 @@ def main(argv=None) -> int:
     if args.only == "prefill":
         print(json.dumps({"prefill": prefill_point(), "layers": layers}))
         return 0
+    if args.only == "step":
+        print(json.dumps({"step_function": step_function_decode(cfg, model, args.batch, min(args.steps, 64), args.warmup, args.context),
+                          "layers": layers}))
+        return 0
     if args.only == "decode":
         args.no_points = True
-    ms = time_decode(model, args.batch, args.steps, args.warmup, args.context)
-    mean_ctx = args.context + args.warmup + args.steps / 2.0
-    nbytes = decode_bytes(cfg, model, args.batch, mean_ctx)
-    achieved = nbytes / (ms * 1e-3) / 1e9
+    head = engine_decode(cfg, model, args.batch, args.steps, args.warmup, args.context, args.new_tokens)
+    ms = head["ms_per_step"]
+    achieved = head["bytes_per_step"] / (ms * 1e-3) / 1e9
     result = {
-        "metric": f"decode tokens/s, {name} shape, batch {args.batch}, {args.context}-token contexts, one MI355X",
-        "value": round(args.batch * 1e3 / ms, 2),
+        "metric": f"decode tokens/s, {name} shape, batch {args.batch}, {args.context}-token prompts, {args.new_tokens} new tokens, "
+                  f"through the engine, one MI355X",
+        "value": head["tokens_per_s"],
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms, 4),
+        "ms_per_step": ms,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": f"synthetic: seeded random weights and token ids; decode caches hold random keys/values of {args.context}-token contexts",
+        "data": f"synthetic: seeded random weights and token ids; {args.context}-token random prompts prefilled by the engine, "
+                f"greedy decoding with no stop token",
         "config": {
             "model": f"{name} shape (Qwen2ForCausalLM)", "layers": layers, "layers_full_model": full_layers,
             "hidden_size": cfg.hidden_size, "num_attention_heads": cfg.num_attention_heads,
             "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
-            "global_batch": args.batch, "seq_len": args.context, "context_limit": cfg.max_position_embeddings,
-            "page_size": PAGE, "prefill_tokens": ptokens, "parallelism": "single GPU",
+            "global_batch": args.batch, "seq_len": args.context, "new_tokens": args.new_tokens,
+            "context_limit": cfg.max_position_embeddings, "page_size": PAGE, "prefill_tokens": ptokens,
+            "parallelism": "single GPU",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "bytes_per_step": head["bytes_per_step"],
+                     "mean_context": head["mean_context"]},
+        "engine": {"graph_replays": head["graph_replays"], "steps_ahead": head["steps_ahead"]},
     }
     if not args.no_points:
-        result["prefill"] = prefill_point()
-        points = {}
+        stream_gbs = measure_stream_read_gbs()
+        gemm_tflops = measure_gemm_tflops(model.dtype)
+        result["measured"] = {"stream_read_gbs": round(stream_gbs, 1), "gemm_tflops": round(gemm_tflops, 1),
+                              "how": "a kernel of this repository that only reads 2 GiB; its own 8192-cubed matrix product"}
+        result["roofline"]["frac_measured"] = round(achieved / stream_gbs, 4)
+        bare = step_function_decode(cfg, model, args.batch, 64, args.warmup, args.context)
+        result["step_function"] = bare
+        result["prefill"] = prefill_point(gemm_tflops)
+        points, detail = {}, {}
         for b in (1, 64):
-            pm = time_decode(model, b, max(8, args.steps // 2), max(2, args.warmup // 2), args.context)
-            points[f"decode_b{b}"] = round(b * 1e3 / pm, 2)
+            r = engine_decode(cfg, model, b, max(8, args.steps // 2), max(2, args.warmup // 2), args.context, args.new_tokens)
+            gbs = r["bytes_per_step"] / (r["ms_per_step"] * 1e-3) / 1e9
+            points[f"decode_b{b}"] = r["tokens_per_s"]
+            detail[f"decode_b{b}"] = {"ms_per_step": r["ms_per_step"], "steps": r["steps"], "bytes_per_step": r["bytes_per_step"],
+                                      "mean_context": r["mean_context"], "achieved_gbs": round(gbs, 1),
+                                      "frac": round(gbs / HBM_PEAK_GBS, 4), "frac_measured": round(gbs / stream_gbs, 4)}
         result["points"] = points
+        result["points_detail"] = detail
+    if args.all:
+        del model
+        torch.cuda.empty_cache()
+        result["extra"] = secondary(args)
     print(json.dumps(result))
     return 0
 

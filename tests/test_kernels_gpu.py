@@ -884,3 +884,17 @@ def test_sample_temperature_matches_formula_and_distribution(ops):
     p = torch.softmax(logits[0].double() / temp, -1)
     # 20000 draws: standard error of a frequency is at most 0.0035; allow 4 of them
     assert float((freq - p).abs().max()) < 0.015
+
+
+def test_stream_read_reads_every_word(ops):
+    """The benchmark's yardstick kernel folds every 32-bit word it reads into its result: flipping one bit
+    anywhere flips the result, for sizes that are no multiple of anything."""
+    import numpy as np
+    g = torch.Generator().manual_seed(12)
+    fold = lambda t: int(np.bitwise_xor.reduce(t.cpu().numpy().view("uint32")))
+    for words in (4, 1000, 256 * 8 * 4 * 64 + 4, 5_000_004):
+        data = torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), generator=g, dtype=torch.int64).to(torch.int32).cuda()
+        used = words // 4 * 4                     # whole 16-byte pieces
+        assert fold(ops.stream_read(data)) == fold(data[:used])
+        data[used // 2] ^= 1 << 7
+        assert fold(ops.stream_read(data)) == fold(data[:used])

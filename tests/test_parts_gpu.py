@@ -171,10 +171,14 @@ def test_block_part_alone(dtype):
 
 # ---------------------------------------------------------------- a toy mixer from outside
 
-def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path):
+@pytest.mark.parametrize("graphs", [False, True])
+def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path, graphs):
     """A mixer defined here -- a per-channel running average whose only memory is a
     fixed-size state per request -- is registered, put into a model through a configuration
-    of its own, and stepped in portions, without touching the framework's files."""
+    of its own, and stepped in portions and token by token, without touching the framework's files.
+    It says it is ``graph_safe`` (a step of one token per request works from the step's device-side
+    numbers only), so with ``graphs`` its decode steps are captured and replayed: the state tensor is a
+    static buffer, and the padding rows of a replayed step use the state row that belongs to no request."""
     from torchlet_amd.config import BlockSpec, ModelConfig, ModelSpec, PartSpec, RMSNormSpec, RunEntry, SwiGLUSpec
     from torchlet_amd.engine.batch import StepEntry
     from torchlet_amd.engine.loading import build_model, make_runner
@@ -190,6 +194,7 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path):
     @MIXERS.register("toy_decay")
     class DecayMixer(Mixer):
         """y_t = s_t with s_t = a * s_{t-1} + x_t per channel, a = sigmoid(decay)."""
+        graph_safe = True
 
         def weight_specs(self):
             return {"decay": WeightSpec((self.spec.hidden,), role="vector")}
@@ -202,6 +207,11 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path):
 
         def forward(self, h, ctx, cache):
             a = torch.sigmoid(self.decay.float())
+            if ctx.decode_only:          # one token per request: nothing of the step is read on the host
+                slots = ctx.slots.long()
+                s = a * cache.state[slots] + h.float()
+                cache.state.index_copy_(0, slots, s)
+                return s.to(h.dtype)
             out = torch.empty_like(h)
             indptr, slots = ctx.req_indptr.tolist(), ctx.slots.tolist()
             for r, slot in enumerate(slots):
@@ -234,12 +244,27 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path):
         tensors = random_tensors(cfg, seed=9, dtype=torch.float32)
         assert "model.layers.1.mix.decay" in tensors
         model = build_model(cfg, "float32", tensors=tensors)
-        runner = make_runner(model, page_size=16, num_pages=2, max_requests=2)
-        assert runner.cache.groups == [] and runner.caches[0].state.shape == (3, 24)
-        seqs = {"a": torch.randint(0, 40, (23,)).tolist(), "b": torch.randint(0, 40, (9,)).tolist()}
+        runner = make_runner(model, page_size=16, num_pages=2, max_requests=3, use_graphs=graphs)
+        assert runner.cache.groups == [] and runner.caches[0].state.shape == (4, 24) and runner.use_graphs == graphs
+        seqs = {"a": torch.randint(0, 40, (23,)).tolist(), "b": torch.randint(0, 40, (9,)).tolist(), "c": torch.randint(0, 40, (31,)).tolist()}
         whole = {k: runner.step([StepEntry(k, v, list(range(len(v))))]).cpu() for k, v in seqs.items()}
         for k in seqs:
             runner.release(k)
+        # three requests token by token from their first token on: steps of one token per request, replayed as
+        # graphs of width four (one padding row) when graphs are on; "b" ends first and the width drops to two
+        singles = {k: [] for k in seqs}
+        for i in range(31):
+            live = [k for k in seqs if i < len(seqs[k])]
+            out = runner.step([StepEntry(k, [seqs[k][i]], [0]) for k in live]).cpu()
+            for j, k in enumerate(live):
+                singles[k].append(out[j: j + 1])
+            for k in live:
+                if i == len(seqs[k]) - 1:
+                    runner.release(k)
+        for k in seqs:
+            torch.testing.assert_close(torch.cat(singles[k]), whole[k], atol=1e-5, rtol=1e-5)
+        assert (runner.graph_replays > 20) == graphs
+        del seqs["c"]
         # the same two requests interleaved, in portions: the state carries over by slot
         got = {"a": [], "b": []}
         got["a"].append(runner.step([StepEntry("a", seqs["a"][:7], list(range(7)))]).cpu())

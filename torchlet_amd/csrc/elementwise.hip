@@ -443,3 +443,54 @@ extern "C" int tl_swiglu(const void* gu, void* out, int tokens, int inter, int a
     TL_CHECK_LAUNCH("swiglu");
     return TL_OK;
 }
+
+// ------------------------------------------------------------------ streaming read (a yardstick)
+// Reads `bytes` of memory once, as fast as the machine lets a kernel read: every work-group walks a
+// contiguous share in 16-byte pieces, eight requests per thread on their way, and folds what it read into one
+// word per work-group (written to `sink`, so that no read can be dropped).  What it measures is the rate at
+// which this GPU delivers memory to any kernel that only reads; the benchmark quotes the decode step against it.
+#define STREAM_THREADS 256
+#define STREAM_DEPTH 8
+__global__ __launch_bounds__(STREAM_THREADS) void stream_read_kernel(const uint4* __restrict__ p, size_t pieces,
+                                                                     size_t per_group, uint32_t* __restrict__ sink) {
+    const size_t begin = (size_t)blockIdx.x * per_group;
+    const size_t end = begin + per_group < pieces ? begin + per_group : pieces;
+    uint32_t acc = 0;
+    size_t i = begin + threadIdx.x;
+    for (; i + (STREAM_DEPTH - 1) * STREAM_THREADS < end; i += STREAM_DEPTH * STREAM_THREADS) {
+        uint4 v[STREAM_DEPTH];
+#pragma unroll
+        for (int u = 0; u < STREAM_DEPTH; ++u) v[u] = p[i + (size_t)u * STREAM_THREADS];
+#pragma unroll
+        for (int u = 0; u < STREAM_DEPTH; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < end; i += STREAM_THREADS) {
+        const uint4 v = p[i];
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+#pragma unroll
+    for (int o = TL_WAVE / 2; o > 0; o >>= 1) acc ^= __shfl_xor(acc, o, TL_WAVE);
+    __shared__ uint32_t part[STREAM_THREADS / TL_WAVE];
+    if (threadIdx.x % TL_WAVE == 0) part[threadIdx.x / TL_WAVE] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t all = 0;
+        for (int w = 0; w < STREAM_THREADS / TL_WAVE; ++w) all ^= part[w];
+        sink[blockIdx.x] = all;
+    }
+}
+
+// Work-groups the read is dealt to by default (`sink` needs one 32-bit word per work-group).
+extern "C" int tl_stream_read_groups() { return 8192; }     // measured: 256 give 5.6 TB/s, 2048 6.2, 8192 6.3, 16384 6.2
+
+extern "C" int tl_stream_read(const void* data, size_t bytes, void* sink, int groups, hipStream_t stream) {
+    TL_REQUIRE(data != nullptr && sink != nullptr && bytes >= 16 && ((uintptr_t)data % 16) == 0,
+               "stream_read: needs 16-byte aligned memory of at least 16 bytes and a sink");
+    TL_REQUIRE(groups >= 0 && groups <= 65536, "stream_read: %d work-groups", groups);
+    const size_t pieces = bytes / 16;
+    if (groups == 0) groups = tl_stream_read_groups();
+    const size_t per_group = (pieces + groups - 1) / groups;
+    stream_read_kernel<<<dim3(groups), dim3(STREAM_THREADS), 0, stream>>>((const uint4*)data, pieces, per_group, (uint32_t*)sink);
+    TL_CHECK_LAUNCH("stream_read");
+    return TL_OK;
+}

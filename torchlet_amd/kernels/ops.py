@@ -643,3 +643,16 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor | None, keys: torch.T
     scratch = torch.empty((2, N, lib.tl_sample_chunks(c_int(V))), dtype=torch.int32, device=logits.device)
     _check(lib, lib.tl_sample(_ptr(logits), c_int(N), c_int(V), c_int(logits.stride(0)), _ptr(temperature), _ptr(keys),
                               _ptr(out), _ptr(scratch), _stream()))
+
+
+def stream_read(data: torch.Tensor, groups: int = 0) -> torch.Tensor:
+    """Read every byte of ``data`` (contiguous, on the GPU) once with a kernel that does nothing else, and
+    return the exclusive-or of its 32-bit words per work-group (int32; ``groups`` work-groups, 0: the default).  A yardstick: the time it takes is
+    what this GPU needs to deliver that much memory to a kernel, whatever the kernel does with it."""
+    if not data.is_contiguous() or data.data_ptr() % 16 or data.numel() * data.element_size() < 16:
+        raise KernelError("stream_read: contiguous, 16-byte aligned memory of at least 16 bytes")
+    lib = _lib("elementwise")
+    lib.tl_stream_read.argtypes = [c_void_p, ctypes.c_size_t, c_void_p, c_int, c_void_p]
+    sink = torch.empty(groups or lib.tl_stream_read_groups(), dtype=torch.int32, device=data.device)
+    _check(lib, lib.tl_stream_read(_ptr(data), ctypes.c_size_t(data.numel() * data.element_size()), _ptr(sink), c_int(groups), _stream()))
+    return sink

@@ -13,9 +13,8 @@ from torchlet_amd.weights.loader import SafetensorsFolder, WeightError, check_ag
 from torchlet_amd.weights.random_init import random_tensors, write_model_folder
 
 # the tiny dictionary configuration of the reference's loader test
-# (/root/reference/tests/test_weight_loading.py:75-84), with hidden 64 instead of 16: its
-# head size of 4 is one the attention kernels refuse (see test_small_head_size_is_refused)
-REF_TINY = dict(vocab_size=16, hidden_size=64, num_hidden_layers=1, num_attention_heads=4, num_key_value_heads=2,
+# (/root/reference/tests/test_weight_loading.py:75-84): heads of 4
+REF_TINY = dict(vocab_size=16, hidden_size=16, num_hidden_layers=1, num_attention_heads=4, num_key_value_heads=2,
                 intermediate_size=32, max_position_embeddings=8, tie_word_embeddings=True)
 
 
@@ -43,7 +42,7 @@ def test_every_size_comes_from_the_keys():
         assert (m.num_heads, m.num_kv_heads) == (d["num_attention_heads"], d["num_key_value_heads"])
         assert m.head_dim == d.get("head_dim", d["hidden_size"] // d["num_attention_heads"])
         assert spec.layers[0].ffn.intermediate == d["intermediate_size"]
-        assert spec.layers[0].mixer_norm.eps == d["rms_norm_eps"]
+        assert spec.layers[0].mixer_norm.eps == d.get("rms_norm_eps", 1e-6)          # F leaves it to the default
     c = Qwen2Config.from_dict(tiny_models.CONFIGS["C"])
     assert [l.mixer.window for l in c.to_spec().layers] == [None, 20, 20, 20]
     assert c.rope_theta == 500000.0 and not c.attention_bias
@@ -91,9 +90,13 @@ def _model(d, dtype=torch.bfloat16):
     return DecoderModel(Qwen2Config.from_dict(d).to_spec(), dtype, "cpu")
 
 
-def test_small_head_size_is_refused():
-    with pytest.raises(ConfigError, match="multiples of 16"):
-        _model(dict(REF_TINY, hidden_size=16))
+def test_head_sizes_that_no_kernel_takes_are_refused():
+    assert _model(REF_TINY).blocks[0].mixer.kernel_libraries() == ["attention_hd16"]        # heads of 4: served by the library of 16
+    assert _model(dict(REF_TINY, head_dim=40)).blocks[0].mixer.kernel_libraries() == ["attention_hd48"]
+    with pytest.raises(ConfigError, match="even"):
+        _model(dict(REF_TINY, head_dim=7))
+    with pytest.raises(ConfigError, match="even head sizes from 2 to 256"):
+        _model(dict(REF_TINY, head_dim=258))
 
 
 def test_reference_tiny_config_loads_strictly_in_bf16(tmp_path):
@@ -111,7 +114,7 @@ def test_reference_tiny_config_loads_strictly_in_bf16(tmp_path):
     assert blk.mixer.w_qkv.dtype == torch.bfloat16 and blk.mixer.b_qkv.dtype == torch.bfloat16
     assert blk.mixer_norm.weight.dtype == torch.bfloat16
     assert blk.mixer.position.inv_freq.dtype == torch.float32
-    assert blk.mixer.w_qkv.shape == (64 + 2 * 32, 64) and blk.ffn.gate_up.shape == (64, 64)
+    assert blk.mixer.w_qkv.shape == (16 + 2 * 8, 16) and blk.ffn.gate_up.shape == (64, 16)
 
 
 def test_tensors_stored_in_32_bit_stay_so_and_fp32_engine_widens(tmp_path):
@@ -144,7 +147,7 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     msg = str(e.value)
     assert "missing (2)" in msg and "model.layers.0.mlp.up_proj.weight" in msg and "model.norm.weight" in msg
     assert "unexpected (1)" in msg and "rotary_emb.inv_freq" in msg
-    assert "k_proj.weight: stored [4, 64], model wants [32, 64]" in msg
+    assert "k_proj.weight: stored [4, 64], model wants [8, 16]" in msg
     assert "lm_head.weight" not in msg                       # a tied head may be absent
 
 

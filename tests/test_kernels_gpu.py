@@ -278,7 +278,8 @@ def _rope_ref(x, pos, theta):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nh,nkv,hd,page,theta", [(4, 2, 16, 16, 1e4), (3, 1, 32, 8, 1e6), (28, 4, 128, 16, 1e6), (5, 5, 48, 4, 5e5)])
+@pytest.mark.parametrize("nh,nkv,hd,page,theta", [(4, 2, 16, 16, 1e4), (3, 1, 32, 8, 1e6), (28, 4, 128, 16, 1e6), (5, 5, 48, 4, 5e5),
+                                                  (4, 2, 6, 8, 1e4), (3, 1, 250, 4, 1e6)])
 def test_rope_cache_write(ops, dtype, nh, nkv, hd, page, theta):
     g = torch.Generator().manual_seed(3)
     lens, ctxs = [5, 1, 11], [0, 37, 6]           # three requests: new tokens, cached before
@@ -536,10 +537,12 @@ def _attention_ref(q, k, v, window):
     (4, 2, 16, 16, 0, 1), (3, 1, 32, 8, 0, 1), (28, 4, 128, 16, 0, 3), (6, 6, 48, 4, 0, 1),
     (20, 1, 64, 16, 0, 2), (4, 2, 16, 16, 13, 1), (8, 2, 80, 32, 29, 4), (2, 1, 256, 16, 0, 1),
     (5, 5, 32, 2, 0, 2), (14, 2, 128, 64, 40, 5),
+    (4, 2, 4, 4, 0, 1), (10, 2, 24, 16, 0, 3), (3, 3, 250, 8, 17, 2), (5, 1, 40, 16, 0, 2), (2, 1, 2, 16, 0, 1),
 ])
 def test_paged_attention(ops, dtype, general, nh, nkv, hd, page, window, splits):
     """float32 and bfloat16 through the general kernel, bfloat16 through the matrix-core kernel
-    (pages of 2 tokens fall back to the general one by themselves)."""
+    (pages of 2 tokens fall back to the general one by themselves, and so do head sizes that are
+    no multiple of 16: the library of the next multiple serves them)."""
     g = torch.Generator().manual_seed(4)
     lens, ctxs = [37, 1, 9, 1], [0, 150, 70, 0]      # a whole prompt, a decode, a portion, a first token
     R, T = len(lens), sum(lens)

@@ -17,7 +17,8 @@ pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
 
 LENGTHS = {"A": [70, 33, 97, 5, 120, 64], "B": [40, 129, 9, 64, 200, 1 + 32], "C": [150, 61, 33, 90, 47, 128],
-           "D": [260, 77, 140, 33, 200, 64], "E": [90, 35, 120, 7, 64, 50]}
+           "D": [260, 77, 140, 33, 200, 64], "E": [90, 35, 120, 7, 64, 50],
+           "F": [8, 3, 7, 8, 5, 2], "G": [150, 40, 97, 300, 18, 64]}
 TOL = {"float32": scenarios.FP32_TOL, "bfloat16": scenarios.BF16_TOL}
 
 
@@ -60,7 +61,7 @@ def expected(model_folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G"])
 @pytest.mark.parametrize("mode", ["whole", "tail_singles", "portions", "mixed"])
 def test_split(model_folders, expected, name, dtype, mode):
     reqs, exp = expected(name)
@@ -119,7 +120,7 @@ def test_decode_steps_replayed_as_graphs(model_folders, expected, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G"])
 def test_pages_that_hold_nan_where_nothing_is_written_yet(model_folders, expected, name, dtype):
     """The pool starts out full of NaN instead of zeros, as if earlier requests had left the worst
     behind: no kernel may let a place that its request has not written reach a result."""

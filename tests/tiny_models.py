@@ -6,7 +6,10 @@ out (no QKV bias, one KV head per query head, a window on the later layers); D h
 64 (the size from which the 128-row prompt attention kernel is built), groups of three, a
 window wider than a step of keys and pages of 8; E has a width, a feed-forward width and a
 vocabulary that are no multiples of 8 (the matrix-core kernels refuse them: the bfloat16 engine
-runs its general kernels), seven heads of 16 and pages of 4.
+runs its general kernels), seven heads of 16 and pages of 4; F is the tiny configuration of the
+reference's own loader test (/root/reference/tests/test_weight_loading.py:75-84: hidden 16, four heads
+of 4 in two groups, eight positions, tied) with pages of 4; G has heads of 24, a size that is no
+multiple of 16 (the attention library of 32 serves it), in groups of five, and pages of 16.
 """
 import json
 from pathlib import Path
@@ -42,9 +45,19 @@ CONFIGS = {
         num_attention_heads=7, num_key_value_heads=7, head_dim=16, intermediate_size=75,
         max_position_embeddings=300, rope_theta=20000.0, rms_norm_eps=5e-6, tie_word_embeddings=False,
     ),
+    "F": dict(
+        architectures=["Qwen2ForCausalLM"], vocab_size=16, hidden_size=16, num_hidden_layers=1,
+        num_attention_heads=4, num_key_value_heads=2, intermediate_size=32, max_position_embeddings=8,
+        tie_word_embeddings=True,
+    ),
+    "G": dict(
+        architectures=["Qwen2ForCausalLM"], vocab_size=150, hidden_size=88, num_hidden_layers=2,
+        num_attention_heads=10, num_key_value_heads=2, head_dim=24, intermediate_size=120,
+        max_position_embeddings=320, rope_theta=100000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+    ),
 }
-SEEDS = {"A": 0, "B": 1, "C": 5, "D": 8, "E": 9}
-PAGE_SIZES = {"A": 16, "B": 8, "C": 16, "D": 8, "E": 4}
+SEEDS = {"A": 0, "B": 1, "C": 5, "D": 8, "E": 9, "F": 12, "G": 13}
+PAGE_SIZES = {"A": 16, "B": 8, "C": 16, "D": 8, "E": 4, "F": 4, "G": 16}
 
 
 def write(name: str, root: Path, dtype=torch.bfloat16) -> Path:

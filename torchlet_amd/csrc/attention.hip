@@ -13,7 +13,10 @@
 // Keys lie in their pages as [kv_head][position][d]; values lie transposed,
 // [kv_head][d][position], which is the layout the matrix-core kernel below reads directly.
 //
-// Compiled per head size: -DTL_HEAD_DIM=<multiple of 16>.
+// Compiled per head size: -DTL_HEAD_DIM=<multiple of 16>.  A library serves the head sizes
+// TL_HEAD_DIM - 14 .. TL_HEAD_DIM (even ones): the general kernel takes the true size `hd` at run time and
+// treats the dimensions from hd up to TL_HEAD_DIM as zeros that are neither read nor written; the
+// matrix-core kernels are for hd == TL_HEAD_DIM.
 #include "common.h"
 
 #ifndef TL_HEAD_DIM
@@ -39,6 +42,7 @@ struct AttnArgs {
     float* part_o;            // [tokens * heads, splits, HD] (splits > 1)
     float* part_ml;           // [tokens * heads, splits, 2]
     int q_stride, bt_stride, heads, kv_heads, page, window, tq, gcap, splits;
+    int hd;                   // the true head size, <= HD: width of a head in q, out and the planes
     int page_shift;           // log2(page) when page is a power of two, else -1
     float scale;
 };
@@ -106,8 +110,8 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
         const int rr = i / AT_HD, d = i % AT_HD;
         const int tt = rr / a.gcap, gg = rr % a.gcap;
         float v = 0.f;
-        if (tt < ntok && gg < gcount)
-            v = to_float(q[(size_t)(first + tok0 + tt) * a.q_stride + (size_t)(kvh * group + g0 + gg) * AT_HD + d]);
+        if (tt < ntok && gg < gcount && d < a.hd)
+            v = to_float(q[(size_t)(first + tok0 + tt) * a.q_stride + (size_t)(kvh * group + g0 + gg) * a.hd + d]);
         qs[rr][d] = v;
     }
 
@@ -136,10 +140,10 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
             const int j = i / AT_HD, d = i % AT_HD;
             const int pos = kbase + j;
             float kv = 0.f, vv = 0.f;
-            if (pos < key_hi) {
+            if (pos < key_hi && d < a.hd) {
                 const int pg = bt[pos / a.page];
-                const size_t head = ((size_t)pg * a.kv_heads + kvh) * a.page * AT_HD;
-                kv = to_float(kp[head + (size_t)(pos % a.page) * AT_HD + d]);
+                const size_t head = ((size_t)pg * a.kv_heads + kvh) * a.page * a.hd;
+                kv = to_float(kp[head + (size_t)(pos % a.page) * a.hd + d]);
                 vv = to_float(vp[head + (size_t)d * a.page + (pos % a.page)]);
             }
             ks[j][d] = kv;
@@ -197,10 +201,11 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
 
     if (!row_ok) return;
     if (a.splits == 1) {
-        T* o = (T*)a.out + (size_t)r_token * a.heads * AT_HD + (size_t)r_head * AT_HD;
+        T* o = (T*)a.out + (size_t)r_token * a.heads * a.hd + (size_t)r_head * a.hd;
         const float inv = 1.f / l;
 #pragma unroll
-        for (int i = 0; i < AT_DPT; ++i) o[sub + 16 * i] = from_float<T>(acc[i] * inv);
+        for (int i = 0; i < AT_DPT; ++i)
+            if (sub + 16 * i < a.hd) o[sub + 16 * i] = from_float<T>(acc[i] * inv);
     } else {
         const size_t pr = ((size_t)r_token * a.heads + r_head) * a.splits + split;
         float* o = a.part_o + pr * AT_HD;
@@ -737,7 +742,7 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(AttnArgs a
 template <typename T>
 __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                               T* __restrict__ out, int splits, const int* __restrict__ tokens,
-                                                              int heads, int rows) {
+                                                              int heads, int rows, int hd) {
     const int local = threadIdx.x / ATG_TPR;
     const long listed = (long)blockIdx.x * ATG_RPW + local;
     if (local >= ATG_RPW || listed >= rows) return;
@@ -772,18 +777,23 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
             }
         mx = m8;
     }
-    T* dst = out + r * AT_HD + d;
-    dst[0] = from_float<T>(num.x / denom);
-    dst[1] = from_float<T>(num.y / denom);
-    dst[2] = from_float<T>(num.z / denom);
-    dst[3] = from_float<T>(num.w / denom);
+    T* dst = out + r * hd + d;             // the parts are HD wide, a row of out holds the true head size
+    if (d + 3 < hd) {
+        dst[0] = from_float<T>(num.x / denom);
+        dst[1] = from_float<T>(num.y / denom);
+        dst[2] = from_float<T>(num.z / denom);
+        dst[3] = from_float<T>(num.w / denom);
+    } else if (d + 1 < hd) {               // head sizes are even
+        dst[0] = from_float<T>(num.x / denom);
+        dst[1] = from_float<T>(num.y / denom);
+    }
 }
 
 static void launch_merge(const void* part_o, const void* part_ml, void* out, int splits, const void* tokens, int heads,
-                         long rows, bool f32, hipStream_t stream) {
+                         long rows, bool f32, hipStream_t stream, int hd = AT_HD) {
     dim3 grid((unsigned)((rows + ATG_RPW - 1) / ATG_RPW)), block(256);
-    if (f32) attention_merge_kernel<float><<<grid, block, 0, stream>>>((const float*)part_o, (const float*)part_ml, (float*)out, splits, (const int*)tokens, heads, (int)rows);
-    else attention_merge_kernel<bf16_t><<<grid, block, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, splits, (const int*)tokens, heads, (int)rows);
+    if (f32) attention_merge_kernel<float><<<grid, block, 0, stream>>>((const float*)part_o, (const float*)part_ml, (float*)out, splits, (const int*)tokens, heads, (int)rows, hd);
+    else attention_merge_kernel<bf16_t><<<grid, block, 0, stream>>>((const float*)part_o, (const float*)part_ml, (bf16_t*)out, splits, (const int*)tokens, heads, (int)rows, hd);
 }
 
 // =====================================================================================
@@ -1143,7 +1153,7 @@ extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out,
                "attention_prompt: splits > 1 need scratch and the tokens to merge");
     a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
     a.q_stride = q_stride; a.bt_stride = bt_stride; a.heads = heads; a.kv_heads = kv_heads; a.page = page;
-    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = splits; a.scale = scale;
+    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = splits; a.scale = scale; a.hd = AT_HD;
     a.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz(page) : -1;
     const int chunks = (group + gcap - 1) / gcap;
     static hipError_t allowed = hipFuncSetAttribute((const void*)paged_attention_prompt_kernel,
@@ -1168,10 +1178,12 @@ extern "C" int tl_attention_head_dim() { return AT_HD; }
 extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const void* k_plane, const void* v_plane,
                                   const void* block_table, int bt_stride, const void* req_indptr, const void* ctx_lens,
                                   const void* tile_req, const void* tile_tok0, int tiles, int tokens, int tq,
-                                  int heads, int kv_heads, int page, int window, float scale, int splits,
+                                  int heads, int kv_heads, int head_dim, int page, int window, float scale, int splits,
                                   void* part_o, void* part_ml, const void* merge_tokens, int merge_count, int dtype, int general,
                                   hipStream_t stream) {
     TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
+    TL_REQUIRE(head_dim > AT_HD - 16 && head_dim <= AT_HD && head_dim % 2 == 0,
+               "attention: this library serves the even head sizes %d to %d, not %d", AT_HD - 14, AT_HD, head_dim);
     TL_REQUIRE(page > 0 && bt_stride > 0 && tq > 0 && splits > 0 && window >= 0, "attention: bad page/table/tile sizes");
     TL_REQUIRE(splits == 1 || (part_o && part_ml), "attention: splits > 1 needs scratch");
     TL_REQUIRE((tile_req && tile_tok0 && req_indptr) || (!tile_req && !tile_tok0 && tiles == tokens),
@@ -1179,7 +1191,7 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
     const int group = heads / kv_heads;
     const int gcap = group < AT_ROWS ? group : AT_ROWS;
     TL_REQUIRE(tq * gcap <= AT_ROWS, "attention: tile of %d tokens x %d heads exceeds %d rows", tq, gcap, AT_ROWS);
-    TL_REQUIRE(q_stride >= heads * AT_HD, "attention: q stride %d too small", q_stride);
+    TL_REQUIRE(q_stride >= heads * head_dim, "attention: q stride %d too small", q_stride);
     if (tiles == 0 || tokens == 0) return TL_OK;
     AttnArgs a;
     a.q = q; a.out = out; a.k_plane = k_plane; a.v_plane = v_plane;
@@ -1187,14 +1199,14 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
     a.tile_req = (const int*)tile_req; a.tile_tok0 = (const int*)tile_tok0;
     a.part_o = (float*)part_o; a.part_ml = (float*)part_ml;
     a.q_stride = q_stride; a.bt_stride = bt_stride; a.heads = heads; a.kv_heads = kv_heads; a.page = page;
-    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = splits; a.scale = scale;
+    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = splits; a.scale = scale; a.hd = head_dim;
     a.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz(page) : -1;
     const int chunks = (group + gcap - 1) / gcap;
     dim3 grid(tiles, kv_heads * chunks, splits), block(256);
     const bool aligned = ((uintptr_t)q % 16) == 0 && q_stride % 8 == 0 && ((uintptr_t)out % 8) == 0 &&
                          ((uintptr_t)k_plane % 16) == 0 && ((uintptr_t)v_plane % 8) == 0;
     if (dtype == TL_DT_F32) paged_attention_kernel<float><<<grid, block, 0, stream>>>(a);
-    else if (dtype == TL_DT_BF16 && page % 4 == 0 && aligned && !general) paged_attention_mfma_kernel<<<grid, block, 0, stream>>>(a);
+    else if (dtype == TL_DT_BF16 && page % 4 == 0 && aligned && !general && head_dim == AT_HD) paged_attention_mfma_kernel<<<grid, block, 0, stream>>>(a);
     else if (dtype == TL_DT_BF16) paged_attention_kernel<bf16_t><<<grid, block, 0, stream>>>(a);
     else TL_REQUIRE(false, "attention: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("paged_attention");
@@ -1202,7 +1214,7 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
         // merge_tokens: the tokens whose rows the tiles cover, when these are not all tokens of the step
         const size_t rows = (size_t)(merge_tokens ? merge_count : tokens) * heads;
         if (rows == 0) return TL_OK;
-        launch_merge(part_o, part_ml, out, splits, merge_tokens, heads, (long)rows, dtype == TL_DT_F32, stream);
+        launch_merge(part_o, part_ml, out, splits, merge_tokens, heads, (long)rows, dtype == TL_DT_F32, stream, head_dim);
         TL_CHECK_LAUNCH("attention_merge");
     }
     return TL_OK;
@@ -1233,7 +1245,7 @@ extern "C" int tl_paged_attention_prefill(const void* q, int q_stride, void* out
     a.tile_req = (const int*)tile_req; a.tile_tok0 = (const int*)tile_tok0;
     a.part_o = nullptr; a.part_ml = nullptr;
     a.q_stride = q_stride; a.bt_stride = bt_stride; a.heads = heads; a.kv_heads = kv_heads; a.page = page;
-    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = 1; a.scale = scale;
+    a.window = window; a.tq = tq; a.gcap = gcap; a.splits = 1; a.scale = scale; a.hd = AT_HD;
     a.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz(page) : -1;
     const int chunks = (group + gcap - 1) / gcap;
     paged_attention_prefill_kernel<<<dim3(tiles, kv_heads * chunks), dim3(256), 0, stream>>>(a);

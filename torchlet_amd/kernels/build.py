@@ -30,7 +30,8 @@ FLAGS = [
 ]
 HEADERS = sorted(p.name for p in CSRC.glob("*.h"))      # every header is part of every library's stamp
 
-# head sizes compiled by build_all(): what the tests, the smoke run and the benchmark use
+# head sizes compiled by build_all(): what the tests, the smoke run and the benchmark use (each library also
+# serves the seven even head sizes below its own)
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
 
 

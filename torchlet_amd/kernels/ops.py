@@ -338,7 +338,7 @@ def linear_rope_cache_write(x: torch.Tensor, weight: torch.Tensor, bias: torch.T
     for bfloat16 and up to 16 rows; returns ``False`` without doing anything for other shapes."""
     M, K = x.shape
     N = weight.shape[0]
-    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or M > 16 or M == 0:
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or M > 16 or M == 0 or head_dim % 4:
         return False
     if x.stride(1) != 1 or out.stride(1) != 1 or not weight.is_contiguous() or weight.shape[1] != K or out.shape[0] != M:
         raise KernelError("linear_rope_cache_write: shapes or strides do not fit")
@@ -397,7 +397,7 @@ def linear_rope_cache_write_normed(residual: torch.Tensor, pending: torch.Tensor
     tensor than ``residual``).  Returns ``False`` without doing anything for shapes it is not built for."""
     K = residual.shape[-1]
     N = weight.shape[0]
-    if weight.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or residual.shape[0] != 1:
+    if weight.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or residual.shape[0] != 1 or head_dim % 4:
         return False
     if out.stride(1) != 1 or not weight.is_contiguous() or weight.shape[1] != K or out.shape[0] != 1:
         raise KernelError("linear_rope_cache_write_normed: shapes or strides do not fit")
@@ -454,6 +454,15 @@ def _check_planes(what, k_plane, v_plane, dtype, kv_heads, page_size, head_dim) 
 
 
 ATTENTION_ROWS = 16   # rows (tokens x heads of one group) a work-group owns
+
+
+def attention_library(head_dim: int) -> str:
+    """The attention library that serves ``head_dim``: one is compiled per multiple of 16 and takes the seven even
+    sizes below it too (its general kernel pads them inside; the matrix-core kernels are for the multiple itself)."""
+    if head_dim % 2 or not 2 <= head_dim <= 256:
+        raise KernelError(f"attention kernels take even head sizes from 2 to 256, not {head_dim}")
+    return f"attention_hd{-(-head_dim // 16) * 16}"
+
 SPLIT_SCRATCH_BYTES = 256 << 20     # most memory the parts of a split attention may take before they are merged
 
 
@@ -500,15 +509,16 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
     part_o = part_ml = None
     # the parts are indexed by the step's tokens: a few decode tokens beside a long portion would make the
     # scratch large for nothing, so the split count gives way (fewer parts: the same result up to rounding)
-    splits = max(1, min(splits, SPLIT_SCRATCH_BYTES // (T * num_heads * (head_dim + 2) * 4)))
+    padded = -(-head_dim // 16) * 16            # the parts are as wide as the library's head size
+    splits = max(1, min(splits, SPLIT_SCRATCH_BYTES // (T * num_heads * (padded + 2) * 4)))
     if splits > 1:
-        part_o = torch.empty((T * num_heads * splits, head_dim), dtype=torch.float32, device=q.device)
+        part_o = torch.empty((T * num_heads * splits, padded), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T * num_heads * splits, 2), dtype=torch.float32, device=q.device)
-    lib = _lib(f"attention_hd{head_dim}")
+    lib = _lib(attention_library(head_dim))
     _check(lib, lib.tl_paged_attention(_ptr(q), c_int(q.stride(0)), _ptr(out), _ptr(k_plane), _ptr(v_plane),
                                        _ptr(block_table), c_int(block_table.stride(0)), _ptr(req_indptr), _ptr(ctx_lens),
                                        _ptr(tile_req), _ptr(tile_tok0), c_int(num_tiles), c_int(T), c_int(tile_tokens),
-                                       c_int(num_heads), c_int(num_kv_heads), c_int(page_size), c_int(window),
+                                       c_int(num_heads), c_int(num_kv_heads), c_int(head_dim), c_int(page_size), c_int(window),
                                        c_float(scale), c_int(splits), _ptr(part_o), _ptr(part_ml),
                                        _ptr(merge_tokens[0]) if merge_tokens is not None else c_void_p(None),
                                        c_int(merge_tokens[1] if merge_tokens is not None else 0),
@@ -533,8 +543,8 @@ def paged_attention_prefill(q: torch.Tensor, out: torch.Tensor, k_plane: torch.T
     to 128, pages of a multiple of 4 tokens; tiles of ``tile_tokens`` tokens (64 rows) whose keys
     and values pass through shared memory once per work-group.  Writes the rows of its tiles only."""
     T = q.shape[0]
-    if q.dtype != torch.bfloat16 or head_dim > PREFILL_ATTENTION_MAX_HEAD_DIM or page_size % 4:
-        raise KernelError("paged_attention_prefill: bfloat16, head sizes up to 128 and pages of a multiple of 4 tokens only")
+    if q.dtype != torch.bfloat16 or head_dim > PREFILL_ATTENTION_MAX_HEAD_DIM or head_dim % 16 or page_size % 4:
+        raise KernelError("paged_attention_prefill: bfloat16, head sizes that are multiples of 16 up to 128 and pages of a multiple of 4 tokens only")
     if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
         raise KernelError("paged_attention_prefill: q/out shapes or dtypes do not fit")
     _check_planes("paged_attention_prefill", k_plane, v_plane, q.dtype, num_kv_heads, page_size, head_dim)

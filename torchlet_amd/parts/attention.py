@@ -41,8 +41,8 @@ class GQAttention(Mixer):
         super().__init__(spec, dtype, device)
         if spec.num_heads % spec.num_kv_heads:
             raise ConfigError(f"attention: {spec.num_heads} heads are not a multiple of {spec.num_kv_heads} KV heads")
-        if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
-            raise ConfigError(f"attention kernels are built for head sizes that are multiples of 16 up to 256, not {spec.head_dim}")
+        if spec.head_dim % 2 or not 2 <= spec.head_dim <= 256:
+            raise ConfigError(f"attention kernels are built for even head sizes from 2 to 256, not {spec.head_dim}")
         if spec.window is not None and spec.window < 1:
             raise ConfigError(f"attention: a window must hold at least one key, got {spec.window}")
         self.hidden = spec.hidden
@@ -68,7 +68,7 @@ class GQAttention(Mixer):
         return PagedNeed(num_heads=self.kv_heads, head_dim=self.head_dim, window=self.window, planes=2)
 
     def kernel_libraries(self):
-        return [f"attention_hd{self.head_dim}"]
+        return [ops.attention_library(self.head_dim)]
 
     def weight_specs(self):
         specs = {
@@ -165,7 +165,7 @@ class GQAttention(Mixer):
         rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size, -(-ctx.max_total_len // cache.page_size))
                    and ctx.max_new_tokens >= _PORTION_MIN_TOKENS)
         portions = (self.dtype == torch.bfloat16 and self.head_dim <= ops.PREFILL_ATTENTION_MAX_HEAD_DIM
-                    and cache.page_size % 4 == 0 and ctx.max_new_tokens >= _PORTION_MIN_TOKENS
+                    and self.head_dim % 16 == 0 and cache.page_size % 4 == 0 and ctx.max_new_tokens >= _PORTION_MIN_TOKENS
                     and ctx.max_total_len >= _PORTION_MIN_CONTEXT)
         if rows128 or portions:
             # prompt portions: tiles of 128 (or 64) rows with keys and values through shared memory; the

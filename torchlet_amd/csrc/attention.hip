@@ -800,12 +800,16 @@ static void launch_merge(const void* part_o, const void* part_ml, void* out, int
 // Prompt portions, 128 rows per work-group (bfloat16, head size 64 or 128, pages of 8, 16, 32, ...
 // tokens, sequences of up to ATM_BT_MAX pages).
 //
-// Four waves of 32 rows share steps of 32 keys.  Keys and transposed values of a step go from
-// the pages straight into shared memory (global_load_lds_dwordx4, four buffers: three steps are
-// on their way while one is multiplied; with two buffers of 64 keys the kernel spent half its
-// time waiting for the next step's keys), in 16-byte pieces whose slot within a row is
-// exclusive-ored with the row number, so that the operand reads of sixteen neighbouring rows
-// fall on all banks.  Both products run transposed on v_mfma_f32_32x32x16_bf16:
+// Four waves of 32 rows share steps of 64 keys.  Keys and transposed values of a step go from
+// the pages straight into shared memory (global_load_lds_dwordx4, two buffers: the next step is
+// on its way while this one is multiplied, and two work-groups share a compute unit), in 16-byte
+// pieces whose slot within a row is exclusive-ored with the row number, so that the operand reads
+// of sixteen neighbouring rows fall on all banks.  A tile's time is its number of steps times what
+// a step takes from barrier to barrier, so steps of 64 keys beat steps of 32 with more of them in
+// flight (28 heads in 4 groups, one MI355X: a prompt of 2048 tokens 86 -> 66 us, of 8192 tokens
+// 648 -> 580 us = 0.83 PFLOP/s; steps of 64 keys with three or four buffers leave room for one
+// work-group per compute unit only: 66 us at 2048 tokens but 779 us at 8192).
+// Both products run transposed on v_mfma_f32_32x32x16_bf16:
 //   S^T[key, row] = K[key, :] . Q[row, :]      A = 32 keys x 16 d from shared memory, B = Q (registers)
 //   O^T[d, row]  += V^T[d, key] . P^T[key, row] A = 32 d x 16 keys from shared memory, B = P (registers)
 // so a lane owns ONE query row (its column, lane % 32): maximum, sum and the rescaling of the
@@ -816,10 +820,10 @@ static void launch_merge(const void* part_o, const void* part_ml, void* out, int
 #if AT_HD == 64 || AT_HD == 128
 #define ATQ_ROWS 128
 #ifndef ATQ_KEYS
-#define ATQ_KEYS 32                 // keys per step: 32 or 64
+#define ATQ_KEYS 64                 // keys per step: 32 or 64
 #endif
 #ifndef ATQ_STAGES
-#define ATQ_STAGES 4               // steps in shared memory: this one and those on their way
+#define ATQ_STAGES 2               // steps in shared memory: this one and those on their way
 #endif
 #define ATQ_KB (ATQ_KEYS / 32)      // blocks of 32 keys per step
 #define ATQ_VROW (ATQ_KEYS * 2)     // bytes of a transposed value row (one d, the step's keys)

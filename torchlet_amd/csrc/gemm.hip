@@ -1127,12 +1127,19 @@ static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6,
 // Seconds for `groups` work-groups of tile t over k columns each.  The two smallest tiles run two
 // to a compute unit: each then works at half the unit's rate, and one that has a unit to itself
 // (not more work-groups than units) at about 0.62 of it.  With few rows the products wait for the
-// weights: a work-group draws its BN rows of them at about 32 GB/s (measured at 17-64 rows: 108
-// work-groups of 64 x 256 on the 14B's gate/up matrix take 81 us, 216 of 64 x 128 take 56).
-static double dl_estimate(DlTile t, long groups, int k) {
+// operands: a compute unit fills its shared memory at about 40 GB/s, and a work-group draws its BN
+// rows of weights and its BM rows of x alike (x as often as there are tiles along N: with 64 x 64 tiles
+// as many bytes of x as of weights).  Measured at 17-64 rows: on the 14B's gate/up matrix 108 work-groups
+// of 64 x 256 take 81 us, 216 of 64 x 128 take 56-59, 432 of 64 x 64 (two to a unit) 59-68; on the 7B's
+// 148 of 64 x 256 take 55-60 and 592 of 64 x 64 take 57-66; on the LM head at 128 rows 594 of 128 x 256
+// take 239 and 1188 of 128 x 128 take 266.  `weights_only`: the estimates of plan_dl_split (whether and how to
+// split K over work-groups, a few hundred rows against a narrow matrix) count the weights alone, at 32 GB/s,
+// which is what its plans were fitted with: with x counted they came out a tenth slower at 512 rows against
+// the down projections (87 against 82 us on the 7B's).
+static double dl_estimate(DlTile t, long groups, int k, bool weights_only = false) {
     const bool pairs = t == DL_64x64 || t == DL_128x128;
     const double products = 2.0 * DL_BM[t] * DL_BN[t] * k;
-    const double stream = 2.0 * DL_BN[t] * k / 32e9;
+    const double stream = weights_only ? 2.0 * DL_BN[t] * k / 32e9 : 2.0 * (DL_BN[t] + DL_BM[t]) * k / 40e9;
     if (!pairs) return (double)((groups + 255) / 256) * fmax(products / DL_RATE[t] + DL_FIXED[t], stream);
     const double rate = groups > 256 ? DL_RATE[t] / 2 : DL_RATE[t] * 0.62;
     // (a single round of 128 x 128 tiles runs a tenth behind this estimate: measured on the fused gate/up
@@ -1142,14 +1149,14 @@ static double dl_estimate(DlTile t, long groups, int k) {
     return lag * (double)((groups + 511) / 512) * fmax(products / rate + DL_FIXED[t], groups > 256 ? 2 * stream : stream);
 }
 
-static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = nullptr) {
+static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = nullptr, bool weights_only = false) {
     DlTile best = DL_128x128;
     double best_t = 1e30;
     for (int t = 0; t < DL_TILES; ++t) {
         if (sw && (t == DL_64x64 || t == DL_256x192)) continue;      // a wave of the fused gate needs whole 64-row blocks of weights
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
         if (t == DL_128x128_S4 && (tiles > 256 || M > 128)) continue;      // one round of work-groups, every weight drawn once
-        const double est = dl_estimate((DlTile)t, tiles, K);
+        const double est = dl_estimate((DlTile)t, tiles, K, weights_only);
         if (est < best_t) { best_t = est; best = (DlTile)t; }
     }
     if (estimate) *estimate = best_t;
@@ -1163,7 +1170,7 @@ static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = null
 struct DlSplit { DlTile tile; int parts; int k_per; };
 static DlSplit plan_dl_split(int M, int N, int K) {
     double best_t;
-    DlSplit best{pick_dl_tile(M, N, K, false, &best_t), 1, 0};
+    DlSplit best{pick_dl_tile(M, N, K, false, &best_t, true), 1, 0};
     best_t += (double)M * N * 2 * 2 / 3e12;
     const int steps = K / 64;
     static const DlTile alone[] = {DL_128x128_S4, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256};
@@ -1174,7 +1181,7 @@ static DlSplit plan_dl_split(int M, int N, int K) {
             if ((K + k_per - 1) / k_per != P) continue;
             if (t == DL_128x128_S4 && tiles * P > 256) continue;       // measured in one round of work-groups only
             // (a tenth on top: float slabs leave the kernel more slowly than the estimate's bfloat16 rows)
-            const double est = 1.1 * dl_estimate(t, tiles * P, k_per) + (double)P * M * N * 4 * 2 / 3e12;
+            const double est = 1.1 * dl_estimate(t, tiles * P, k_per, true) + (double)P * M * N * 4 * 2 / 3e12;
             if (est < best_t) { best_t = est; best = DlSplit{t, P, k_per}; }
         }
     }

@@ -97,6 +97,33 @@ def test_attention_window_definition():
     torch.testing.assert_close(w, expect)
 
 
+def test_attention_window_invariants_and_the_library_routine_with_a_band_mask():
+    """The window is not in the reference; what fixes it here besides its definition: a window at least as
+    long as the sequence is causal attention (the library routine), a window of one returns every token's
+    own value, and any window equals the library routine under a band mask built from ``tril``/``triu``
+    (keys ``t - W < s <= t``: a mistake by one at either edge fails it)."""
+    heads, t, hd = 3, 23, 8
+    q, k, v = (torch.randn(heads, t, hd, dtype=torch.float64) for _ in range(3))
+    causal = F.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]
+    for window in (t, t + 5):
+        torch.testing.assert_close(plain.attention_weights(q, k, window=window) @ v, causal)
+    torch.testing.assert_close(plain.attention_weights(q, k, window=1) @ v, v)
+    for window in (2, 7, 22):
+        ones = torch.ones(t, t, dtype=torch.bool)
+        band = torch.tril(ones) & torch.triu(ones, diagonal=-(window - 1))
+        ref = F.scaled_dot_product_attention(q[None], k[None], v[None], attn_mask=band)[0]
+        torch.testing.assert_close(plain.attention_weights(q, k, window=window) @ v, ref)
+        assert int(plain.attention_weights(q, k, window=window)[0].gt(0).sum(-1).max()) == window
+
+
+def test_which_layers_have_a_window():
+    base = dict(vocab_size=8, hidden_size=8, num_hidden_layers=5, num_attention_heads=2, intermediate_size=8)
+    on = plain.PlainConfig(dict(base, use_sliding_window=True, sliding_window=9, max_window_layers=2))
+    assert [on.window_of(i) for i in range(5)] == [None, None, 9, 9, 9]        # layers from max_window_layers on
+    assert [plain.PlainConfig(dict(base, sliding_window=9, max_window_layers=2)).window_of(i) for i in range(5)] == [None] * 5
+    assert [plain.PlainConfig(dict(base, use_sliding_window=True, sliding_window=9)).window_of(i) for i in range(5)] == [None] * 5
+
+
 def _attn_weights(hidden, heads, kvh, hd, bias=True):
     w = {"q_proj.weight": torch.randn(heads * hd, hidden, dtype=torch.float64) * 0.2,
          "k_proj.weight": torch.randn(kvh * hd, hidden, dtype=torch.float64) * 0.2,

@@ -218,3 +218,24 @@ def test_attention_part_fuses_its_projections_and_keeps_32_bit_biases():
     assert torch.equal(half.w_qkv, plain_rows[order]) and torch.equal(half.b_qkv, plain_bias[order])
     # within a head: row 2j is the old row j, row 2j + 1 the old row j + hd/2
     assert order[:6].tolist() == [0, 8, 1, 9, 2, 10] and order[hd:hd + 2].tolist() == [16, 24]
+
+
+def test_start_up_reports(tmp_path):
+    """The reports the reference logs when an LLM starts (llm.py:28-36): one line per tensor with name, shape and
+    stored type, and a description of the backend; a logger that stands at WARNING unless asked."""
+    import io
+    import logging
+
+    from torchlet_amd.logger import backend_info, get_logger, weights_info
+    cfg = Qwen2Config.from_dict(REF_TINY)
+    write_model_folder(cfg, 0, tmp_path)
+    lines = weights_info(SafetensorsFolder(tmp_path)).splitlines()
+    assert len(lines) == len(random_tensors(cfg, 0)) and any(l.split() == ["model.norm.weight", "[16]", "BF16"] for l in lines)
+    assert weights_info({"a": torch.zeros(2, 3)}) == "a  [2, 3]  torch.float32"
+    assert "torch:" in backend_info() and "gfx950" in backend_info()
+    stream = io.StringIO()
+    log = get_logger("torchlet_amd.test", stream=stream)
+    log.info("hidden")
+    assert stream.getvalue() == "" and log.level == logging.WARNING
+    get_logger("torchlet_amd.test", level=logging.INFO).info("shown %d", 3)
+    assert "[INFO] torchlet_amd.test" in stream.getvalue() and "shown 3" in stream.getvalue()

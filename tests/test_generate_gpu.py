@@ -228,8 +228,9 @@ def test_command_line(model_folders, tmp_path):
                          cwd=ROOT, capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stderr
     run = subprocess.run([sys.executable, "-m", "torchlet_amd", "--model", str(tmp_path / "m"), "--prompt-ids", "5,6,7", "--prompt-ids", "9",
-                          "--max-new-tokens", "4", "--dtype", "float32"], cwd=ROOT, capture_output=True, text=True, timeout=120)
+                          "--max-new-tokens", "4", "--dtype", "float32", "--verbose"], cwd=ROOT, capture_output=True, text=True, timeout=120)
     assert run.returncode == 0, run.stderr
+    assert "backend:" in run.stderr and "model.embed_tokens.weight" in run.stderr and "EngineConfig(" in run.stderr      # --verbose
     lines = [json.loads(l) for l in run.stdout.strip().splitlines()]
     cfg, w = plain_qwen2.load_folder(tmp_path / "m")
     assert [l["output"] for l in lines] == [plain_qwen2.greedy(cfg, w, [5, 6, 7], 4), plain_qwen2.greedy(cfg, w, [9], 4)]

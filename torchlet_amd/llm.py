@@ -35,6 +35,7 @@ import torch
 from .engine.config import EngineConfig
 from .engine.loading import load_model, make_engine, require_gpu
 from .engine.request import Request
+from .logger import backend_info, logger, weights_info
 
 
 class LLM:
@@ -52,10 +53,17 @@ class LLM:
             max_tokens_per_step=max_num_batched_tokens, max_model_len=max_model_len, dtype=str(dtype).replace("torch.", ""),
             use_graphs=use_graphs, lookahead=lookahead, seed=seed)
         self.model_dir = Path(model_id)
+        if logger.isEnabledFor(20):                         # INFO: the start-up reports of the reference's LLM (llm.py:28-36)
+            from .weights.loader import SafetensorsFolder
+            logger.info("backend:\n%s", backend_info())
+            logger.info("tensors of %s:\n%s", self.model_dir, weights_info(SafetensorsFolder(self.model_dir)))
         self.config, self.model = load_model(self.model_dir, self.engine_config.dtype, self.device)
         self.engine = make_engine(self.model, self.engine_config)
         self.runner = self.engine.runner
         self.engine_config = self.runner.config            # with the number of pages filled in
+        logger.info("model: %s, %d runs of %d layers, %s; engine: %s; cache: %s pages free per group, %d bytes a page",
+                    self.config.architecture, len(self.model.spec.order), len(self.model.spec.layers), self.model.dtype,
+                    self.engine_config, self.runner.cache.free_pages(), self.runner.cache.bytes_per_page())
         self.tokenizer = _load_tokenizer(self.model_dir)
         self.stop_ids = self._stop_ids()
         self._next_seed = 0
@@ -204,6 +212,7 @@ def _parser():
         q.add_argument("--max-num-blocks", type=int, default=None)
         q.add_argument("--max-num-batched-tokens", type=int, default=2048)
         q.add_argument("--max-model-len", type=int, default=None, help="sequences no longer than this (default: the model's limit)")
+        q.add_argument("--verbose", action="store_true", help="report the backend, the folder's tensors and the engine's sizes at start-up")
     i = sub.add_parser("init", help="write a model folder with random weights from a configuration and a seed")
     i.add_argument("--config", required=True, help="a config.json")
     i.add_argument("--seed", type=int, default=0)
@@ -226,6 +235,11 @@ def main(argv=None) -> int:
     if not args.model:
         print("--model is required", file=sys.stderr)
         return 2
+    if args.verbose:
+        import logging
+
+        from .logger import get_logger
+        get_logger(level=logging.INFO)
     prompts = list(args.prompt) + [[int(t) for t in s.split(",") if t.strip()] for s in args.prompt_ids]
     if not prompts:
         print("give at least one --prompt or --prompt-ids", file=sys.stderr)

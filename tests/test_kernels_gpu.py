@@ -133,6 +133,51 @@ def test_linear(ops, dtype, M, N, K, bias):
     torch.testing.assert_close(out32.double(), ref, **tol32)
 
 
+@pytest.mark.parametrize("M,N,K,bias", [(17, 129, 200, True), (65, 64, 20, False), (130, 513, 1000, True), (64, 300, 4, True),
+                                        (300, 3584, 3584, False), (1000, 257, 1028, True), (33, 1, 8, True), (2048, 130, 3584, True)])
+def test_linear_many_rows_in_32_bit_on_matrix_cores(ops, M, N, K, bias):
+    """v_mfma_f32_32x32x2_f32: true 32-bit products and sums.  Against float64 with the bound of a 32-bit sum; the
+    general v_fma_f32 kernel agrees with it to rounding; a row's result does not depend on how many rows there are
+    beside it or where it lies (bitwise: its sum runs in one order); inputs whose products need every bit of a
+    32-bit mantissa show that nothing is rounded to a shorter format on the way."""
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).cuda()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).cuda()
+    b = torch.randn(N, generator=g).cuda() if bias else None
+    ref = x.double() @ w.double().T + (b.double() if bias else 0)
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    out = torch.full((M, N), float("nan"), device="cuda")
+    ops.linear_f32_variant(x, w, b, out, True)
+    torch.testing.assert_close(out.double(), ref, **tol32)
+    fma = torch.empty(M, N, device="cuda")
+    ops.linear_f32_variant(x, w, b, fma, False)
+    torch.testing.assert_close(fma.double(), ref, **tol32)
+    through = torch.empty(M, N, device="cuda")
+    ops.linear(x, w, b, through)                               # the dispatch takes the matrix-core kernel from 17 rows on
+    assert torch.equal(through, out)
+    # some rows alone, elsewhere in a tile, inside a wider buffer: the same bits
+    rows = [M - 1, 0, M // 2] * 7
+    wide = torch.zeros(len(rows), K + 12, device="cuda")
+    wide[:, 4:4 + K] = x[rows]
+    few = torch.empty(len(rows), N, device="cuda")
+    ops.linear_f32_variant(wide[:, 4:4 + K], w, b, few, True)
+    assert torch.equal(few, out[rows])
+    # operands 1 + d with d below 2^-12 and random signs: what tells them apart lies in the low bits of a 24-bit
+    # mantissa.  A 32-bit sum of K such products (partial sums of size ~sqrt(K), each addition off by half an ulp of
+    # that) stays within 4 * 2^-24 * K; operands cut to a shorter mantissa on the way would leave that bound far behind,
+    # as the same product of bfloat16-rounded operands does.
+    xe = (1 + torch.rand(M, K, generator=g) * 2 ** -12).cuda()
+    we = ((1 + torch.rand(N, K, generator=g) * 2 ** -12) * (torch.randint(0, 2, (N, K), generator=g) * 2 - 1)).cuda()
+    exact = xe.double() @ we.double().T
+    got = torch.empty(M, N, device="cuda")
+    ops.linear_f32_variant(xe, we, None, got, True)
+    bound = 4 * 2 ** -24 * K
+    assert float((got.double() - exact).abs().max()) < bound
+    if M * N * K >= 1 << 16:
+        cut = xe.bfloat16().double() @ we.bfloat16().double().T
+        assert float((cut - exact).abs().max()) > 3 * bound
+
+
 @pytest.mark.parametrize("M", [1, 2, 3, 7, 8, 13, 16])
 @pytest.mark.parametrize("N,K", [(37, 100), (300, 1024), (129, 1028), (4608, 3584), (1, 2052), (64, 18944)])
 def test_linear_few_rows_in_32_bit(ops, M, N, K):

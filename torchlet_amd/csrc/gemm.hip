@@ -177,6 +177,158 @@ static void launch_gemv_f32(const void* x, const void* w, const void* bias, int 
 }
 
 // =====================================================================================
+// True 32-bit on the matrix cores, more than 16 rows: the prompt steps of the 32-bit engine.
+//
+// v_mfma_f32_32x32x2_f32 multiplies 32-bit operands and adds in 32-bit: it is no reduced-precision mode
+// (nothing is rounded to a shorter format on the way), and it runs at four times the rate of the
+// v_fma_f32 tile kernel above.  A work-group of four waves owns a tile of BM x 128 outputs (BM = 64 or
+// 128), a wave 32 FMB x 64 of them; slabs of 16 columns of both operands go through registers into shared
+// memory (two buffers, one barrier per slab).  A lane reads four neighbouring k of its row at once; lanes
+// 0-31 take k = 8c .. 8c+3 and lanes 32-63 k = 8c+4 .. 8c+7 of a chunk of eight, so instruction e of a chunk
+// multiplies k = 8c + e and 8c + 4 + e: which k meet in one instruction is free as long as both operands
+// agree.  The sum of an output element runs in that one fixed order whatever M is and wherever the element
+// lies in its tile, so a row's result does not depend on the batch; it differs from the other 32-bit
+// kernels' by rounding (another order of the same sum).  Needs K % 4 == 0 and 16-byte aligned rows.
+typedef float gf_f32x16_t __attribute__((ext_vector_type(16)));
+#define GF_BN 128
+#define GF_TK 16
+#define GF_LD (GF_TK + 4)          // floats between rows in shared memory: 16-byte reads of 16 rows fall on all banks
+template <int FMB>
+__global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                            const void* __restrict__ bias, int bias_f32,
+                                                            float* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+    constexpr int BM = 64 * FMB;
+    constexpr int XL = BM * 4 / 256;                       // 16-byte pieces of x a thread moves per slab (1 or 2)
+    __shared__ __attribute__((aligned(16))) float xs[2][BM * GF_LD];
+    __shared__ __attribute__((aligned(16))) float ws[2][GF_BN * GF_LD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lr = lane & 31, lh = lane >> 5;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * GF_BN;
+
+    gf_f32x16_t acc[2][FMB];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < FMB; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    // piece p of a slab: row p / 4, columns 4 (p % 4) .. + 4; rows past the end read the last row (never stored),
+    // columns past K read the last whole piece and count as zero
+    float4 gx[XL], gw[2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const int p = tid + 256 * i, k = k0 + 4 * (p & 3);
+            gx[i] = *(const float4*)(x + (size_t)min(m0 + (p >> 2), M - 1) * ldx + min(k, K - 4));
+            if (k >= K) gx[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int p = tid + 256 * i, k = k0 + 4 * (p & 3);
+            gw[i] = *(const float4*)(w + (size_t)min(n0 + (p >> 2), N - 1) * K + min(k, K - 4));
+            if (k >= K) gw[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto park = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < XL; ++i) {
+            const int p = tid + 256 * i;
+            *(float4*)(&xs[buf][(p >> 2) * GF_LD + 4 * (p & 3)]) = gx[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int p = tid + 256 * i;
+            *(float4*)(&ws[buf][(p >> 2) * GF_LD + 4 * (p & 3)]) = gw[i];
+        }
+    };
+    fetch(0);
+    park(0);
+    __syncthreads();
+    const int slabs = (K + GF_TK - 1) / GF_TK;
+    for (int s = 0; s < slabs; ++s) {
+        if (s + 1 < slabs) fetch((s + 1) * GF_TK);          // on their way while this slab is multiplied
+        const float* xb = xs[s & 1];
+        const float* wb = ws[s & 1];
+#pragma unroll
+        for (int c = 0; c < GF_TK / 8; ++c) {
+            float4 a[2], b[FMB];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[i] = *(const float4*)(wb + (wn * 64 + i * 32 + lr) * GF_LD + 8 * c + 4 * lh);
+#pragma unroll
+            for (int j = 0; j < FMB; ++j) b[j] = *(const float4*)(xb + (wm * 32 * FMB + j * 32 + lr) * GF_LD + 8 * c + 4 * lh);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < FMB; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].x, b[j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].y, b[j].y, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].z, b[j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i].w, b[j].w, acc[i][j], 0, 0, 0);
+                }
+        }
+        if (s + 1 < slabs) park((s + 1) & 1);               // everyone left that buffer before the last barrier
+        __syncthreads();
+    }
+    // weight block times x block: a lane holds row m = lane % 32 of x and the output columns
+    // n = 8 (v / 4) + 4 (lane / 32) + v % 4 of a 32 x 32 block, four neighbours at a time
+    const bool quads = N % 4 == 0 && ldo % 4 == 0 && ((uintptr_t)out % 16) == 0;
+#pragma unroll
+    for (int j = 0; j < FMB; ++j) {
+        const int m = m0 + wm * 32 * FMB + j * 32 + lr;
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + wn * 64 + i * 32 + 8 * g + 4 * lh;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e] + ((bias && n + e < N) ? load_vec(bias, bias_f32, n + e) : 0.f);
+                if (quads) {
+                    if (n < N) *(float4*)(out + (size_t)m * ldo + n) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < N) out[(size_t)m * ldo + n + e] = v[e];
+                }
+            }
+    }
+}
+
+static bool gemm_f32_mfma_fits(const void* x, const void* w, int M, int K, int ldx) {
+    return M > 16 && K >= 4 && K % 4 == 0 && ldx % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
+}
+
+static void launch_gemm_f32_mfma(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
+                                 int ldx, int ldo, hipStream_t stream) {
+    // tiles of 64 rows where those of 128 would leave most compute units without one
+    const long tiles128 = (long)((M + 127) / 128) * ((N + GF_BN - 1) / GF_BN);
+    if (M <= 64 || tiles128 < 256) {
+        dim3 grid((N + GF_BN - 1) / GF_BN, (M + 63) / 64);
+        gemm_f32_mfma_kernel<1><<<grid, dim3(256), 0, stream>>>((const float*)x, (const float*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo);
+    } else {
+        dim3 grid((N + GF_BN - 1) / GF_BN, (M + 127) / 128);
+        gemm_f32_mfma_kernel<2><<<grid, dim3(256), 0, stream>>>((const float*)x, (const float*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo);
+    }
+}
+
+// One named kernel of the 32-bit products (for tests and tuning): 0 the general tile kernel (v_fma_f32), 1 the matrix-core kernel.
+extern "C" int tl_gemm_f32_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
+                                   int M, int N, int K, int ldx, int ldo, int matrix_cores, hipStream_t stream) {
+    TL_REQUIRE(M > 0 && N > 0 && K > 0 && ldx >= K && ldo >= N, "gemm_f32: bad sizes M=%d N=%d K=%d ldx=%d ldo=%d", M, N, K, ldx, ldo);
+    if (matrix_cores) {
+        TL_REQUIRE(gemm_f32_mfma_fits(x, w, 17, K, ldx), "gemm_f32: the matrix-core kernel needs K %% 4 == 0 and 16-byte aligned rows");
+        launch_gemm_f32_mfma(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream);
+    } else {
+        launch_gemm_tile<float, float>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream);
+    }
+    TL_CHECK_LAUNCH("gemm_f32");
+    return TL_OK;
+}
+
+// =====================================================================================
 // bfloat16 on the matrix cores, few rows (M <= 64): the decode step's products.
 //
 // Such a product is a stream of the weight matrix through the chip once; the kernel is
@@ -1292,6 +1444,7 @@ static bool skinny_fits(const void* x, const void* w, int M, int K, int ldx) {
 //                                  (matrix cores, operands straight into shared memory)
 //   bfloat16, aligned, M > 64   -> gemm_mfma_tile (matrix cores, shared-memory tiles)
 //   32-bit, aligned, M <= 16    -> gemv_f32 (true 32-bit arithmetic, weight streaming)
+//   32-bit, aligned, M > 16     -> gemm_f32_mfma (true 32-bit arithmetic on the matrix cores)
 //   everything else             -> gemm_tile (true 32-bit arithmetic)
 extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_f32, void* out,
                        int M, int N, int K, int ldx, int ldo, int dtype, int out_f32, hipStream_t stream) {
@@ -1329,6 +1482,11 @@ extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_
     if (dtype == TL_DT_F32 && gemv_f32_fits(x, w, M, K, ldx)) {
         launch_gemv_f32(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream);
         TL_CHECK_LAUNCH("gemv_f32");
+        return TL_OK;
+    }
+    if (dtype == TL_DT_F32 && gemm_f32_mfma_fits(x, w, M, K, ldx)) {
+        launch_gemm_f32_mfma(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream);
+        TL_CHECK_LAUNCH("gemm_f32_mfma");
         return TL_OK;
     }
     return tl_gemm_general(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, dtype, out_f32, stream);

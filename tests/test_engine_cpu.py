@@ -260,3 +260,14 @@ def test_chat_template_runs_in_a_sandbox():
         render_chat_template("{{ raise_exception.__globals__['__builtins__'] }}", "hi")
     with pytest.raises(jinja2.exceptions.TemplateError, match="no system turn"):
         render_chat_template("{{ raise_exception('no system turn') }}", "hi")
+
+
+def test_toy_attention_that_differs_in_one_stage_on_the_host(cpu_ops):
+    """``toy_parts.run_toy_qk_norm`` (queries and keys normalised per head through the attention mixer's hook) on the host."""
+    import toy_parts
+    toy_parts.run_toy_qk_norm(torch.float32, torch.device("cpu"), lambda dtype, ref: dict(atol=2e-5, rtol=1e-4))
+
+
+def test_toy_mixer_whose_cache_planes_differ_on_the_host(cpu_ops):
+    import toy_parts
+    toy_parts.run_toy_latent(torch.float32, torch.device("cpu"))

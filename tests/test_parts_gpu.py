@@ -298,3 +298,15 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path, gr
 def test_toy_routed_feed_forward_and_toy_position_encoding_with_a_layer_run_twice(dtype):
     import toy_parts
     toy_parts.run_toy_mix(dtype, torch.device("cuda"), _tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_attention_that_differs_in_one_stage(dtype):
+    import toy_parts
+    toy_parts.run_toy_qk_norm(dtype, torch.device("cuda"), _tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_mixer_whose_cache_planes_differ_in_width_and_element_type(dtype):
+    import toy_parts
+    toy_parts.run_toy_latent(dtype, torch.device("cuda"))

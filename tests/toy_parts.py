@@ -213,3 +213,216 @@ def run_toy_mix(dtype, device, tolerance):
         unregister_architecture("ToyMixForCausalLM")
         POSITION_ENCODINGS.unregister("toy_rope_pairs")
         FEED_FORWARDS.unregister("toy_top1")
+
+
+def run_toy_qk_norm(dtype, device, tolerance):
+    """A mixer that differs from the framework's attention in one stage only -- queries and keys are normalised per
+    head before they are rotated and stored -- is a subclass that declares two more tensors and defines the
+    ``transform_qk`` hook; projection, rotation, cache write, attention kernels and output projection are the
+    framework's.  Whole requests, portions and single tokens agree with each other and with a plain computation."""
+    from torchlet_amd.config import AttentionSpec, BlockSpec, ModelConfig, ModelSpec, RMSNormSpec, RotarySpec, RunEntry, SwiGLUSpec
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import build_model, make_runner
+    from torchlet_amd.parts import MIXERS, WeightSpec
+    from torchlet_amd.parts.attention import GQAttention
+    from torchlet_amd.registry import config_class, register_architecture, unregister_architecture
+    from torchlet_amd.weights.random_init import random_tensors
+
+    H, HEADS, KVH, HD, INTER, VOCAB, THETA, EPS = 40, 6, 2, 32, 56, 60, 5000.0, 1e-6
+
+    @dataclass(frozen=True)
+    class QKNormAttentionSpec(AttentionSpec):
+        kind: ClassVar[str] = "toy_qk_norm_attention"
+
+    @MIXERS.register("toy_qk_norm_attention")
+    class QKNormAttention(GQAttention):
+        def weight_specs(self):
+            specs = super().weight_specs()
+            specs["q_norm.weight"] = WeightSpec((self.head_dim,), role="vector", init="one_plus_normal")
+            specs["k_norm.weight"] = WeightSpec((self.head_dim,), role="vector", init="one_plus_normal")
+            return specs
+
+        def load_weights(self, tensors):
+            super().load_weights(tensors)
+            self.q_norm = self._place(tensors["q_norm.weight"], "vector").float()
+            self.k_norm = self._place(tensors["k_norm.weight"], "vector").float()
+
+        def transform_qk(self, q3, k3, ctx):
+            for x, w in ((q3, self.q_norm), (k3, self.k_norm)):
+                if x is not None:
+                    f = x.float()
+                    x.copy_((f * torch.rsqrt(f.pow(2).mean(-1, keepdim=True) + EPS) * w).to(x.dtype))
+
+    @dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyQKNormForCausalLM"
+        vocab_size: int
+
+        def to_spec(self):
+            norm = RMSNormSpec(dim=H, eps=1e-5)
+            block = BlockSpec(mixer=QKNormAttentionSpec(hidden=H, num_heads=HEADS, num_kv_heads=KVH, head_dim=HD, qkv_bias=True,
+                                                        position=RotarySpec(head_dim=HD, theta=THETA, max_positions=512)),
+                              mixer_norm=norm, ffn_norm=norm, ffn=SwiGLUSpec(hidden=H, intermediate=INTER))
+            return ModelSpec(vocab_size=self.vocab_size, hidden=H, layers=(block, block), order=(RunEntry(0), RunEntry(1)),
+                             final_norm=norm, tie_head=False, max_positions=512)
+
+    def plain_forward(w, ids, stored=lambda t: t):
+        sub = lambda p: {k[len(p):]: v for k, v in w.items() if k.startswith(p)}
+        T = len(ids)
+        pos = torch.arange(T)
+        x = w["model.embed_tokens.weight"][torch.tensor(ids)]
+        norm = lambda t, weight: stored(plain.rms_norm(t, weight, 1e-5))
+        for layer in range(2):
+            lw, a = sub(f"model.layers.{layer}."), sub(f"model.layers.{layer}.self_attn.")
+            h = norm(x, lw["input_layernorm.weight"])
+            q = stored(plain.linear(h, a["q_proj.weight"], a["q_proj.bias"])).view(T, HEADS, HD)
+            k = stored(plain.linear(h, a["k_proj.weight"], a["k_proj.bias"])).view(T, KVH, HD)
+            v = stored(plain.linear(h, a["v_proj.weight"], a["v_proj.bias"])).view(T, KVH, HD).transpose(0, 1)
+            q = stored(plain.rms_norm(q, a["q_norm.weight"], EPS)).transpose(0, 1)
+            k = stored(plain.rms_norm(k, a["k_norm.weight"], EPS)).transpose(0, 1)
+            q, k = stored(plain.rope_apply(q, pos, THETA)), stored(plain.rope_apply(k, pos, THETA))
+            k, v = (t.repeat_interleave(HEADS // KVH, dim=0) for t in (k, v))
+            ctx = stored((plain.attention_weights(q, k) @ v).transpose(0, 1).reshape(T, HEADS * HD))
+            x = x + stored(plain.linear(ctx, a["o_proj.weight"]))
+            x = x + plain.swiglu_ffn(norm(x, lw["post_attention_layernorm.weight"]), sub(f"model.layers.{layer}.mlp."), stored)
+        return plain.linear(norm(x, w["model.norm.weight"]), w["lm_head.weight"])
+
+    register_architecture(ToyConfig)
+    try:
+        cfg = config_class("ToyQKNormForCausalLM").from_dict(dict(vocab_size=VOCAB))
+        tensors = {k: (v * 4 if "proj" in k else v) for k, v in random_tensors(cfg, seed=6, dtype=torch.bfloat16).items()}
+        assert tensors["model.layers.1.self_attn.q_norm.weight"].shape == (HD,)
+        model = build_model(cfg, dtype, device=device, tensors=tensors)
+        assert not model.blocks[0].mixer.pair_layout              # the hook sees the checkpoint's order of dimensions
+        runner = make_runner(model, page_size=8, num_pages=20, max_requests=2)
+        g = torch.Generator().manual_seed(3)
+        seqs = {"a": torch.randint(0, VOCAB, (45,), generator=g).tolist(), "b": torch.randint(0, VOCAB, (21,), generator=g).tolist()}
+        w = {k: v.double() for k, v in tensors.items()}
+        refs = {k: plain_forward(w, v) for k, v in seqs.items()}
+        whole = {k: runner.step([StepEntry(k, v, list(range(len(v))))]).cpu() for k, v in seqs.items()}
+        for k in seqs:
+            runner.release(k)
+        got = {"a": [], "b": []}
+        got["a"].append(runner.step([StepEntry("a", seqs["a"][:17], list(range(17)))]).cpu())
+        out = runner.step([StepEntry("b", seqs["b"][:9], list(range(9))), StepEntry("a", seqs["a"][17:18], [0])]).cpu()
+        got["b"].append(out[:9]); got["a"].append(out[9:])
+        out = runner.step([StepEntry("a", seqs["a"][18:40], list(range(22))), StepEntry("b", seqs["b"][9:], list(range(12)))]).cpu()
+        got["a"].append(out[:22]); got["b"].append(out[22:])
+        for t in seqs["a"][40:]:
+            got["a"].append(runner.step([StepEntry("a", [t], [0])]).cpu())
+        for k in seqs:
+            tol = tolerance(dtype, refs[k])
+            if dtype == torch.bfloat16:
+                moved = plain_forward(w, seqs[k], stored=lambda t: t.to(torch.bfloat16).double()) - refs[k]
+                tol = dict(atol=2 * float(moved.abs().max()), rtol=0.0)
+            torch.testing.assert_close(whole[k].double(), refs[k], **tol)
+            torch.testing.assert_close(torch.cat(got[k]).double(), refs[k], **tol)
+    finally:
+        unregister_architecture("ToyQKNormForCausalLM")
+        MIXERS.unregister("toy_qk_norm_attention")
+
+
+def run_toy_latent(dtype, device):
+    """A mixer whose per-token cache is not keys and values: two planes of different widths and of an element type of
+    their own (a compressed latent of 12 numbers and 4 position features, both float32 whatever the model's dtype),
+    declared as one ``PagedNeed`` and read back through the block table.  Requests in portions and token by token,
+    interleaved and with pages used again, give what whole requests give."""
+    from torchlet_amd.config import BlockSpec, ModelConfig, ModelSpec, PartSpec, RMSNormSpec, RunEntry, SwiGLUSpec
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import build_model, make_runner
+    from torchlet_amd.parts import MIXERS, Mixer, PagedNeed, WeightSpec
+    from torchlet_amd.registry import config_class, register_architecture, unregister_architecture
+    from torchlet_amd.weights.random_init import random_tensors
+
+    H, LATENT, POS, VOCAB = 32, 12, 4, 30
+
+    @dataclass(frozen=True)
+    class LatentSpec(PartSpec):
+        kind: ClassVar[str] = "toy_latent"
+        hidden: int = 0
+
+    @MIXERS.register("toy_latent")
+    class LatentMixer(Mixer):
+        """c_t = h_t W_c, p_t = (sin, cos)(pos * f); y_t = (sum_s a_ts c_s) W_o with a_t = softmax_s<=t(c_t.c_s + p_t.p_s)."""
+
+        def weight_specs(self):
+            return {"down.weight": WeightSpec((LATENT, self.spec.hidden)), "up.weight": WeightSpec((self.spec.hidden, LATENT))}
+
+        def load_weights(self, tensors):
+            self.down = self._place(tensors["down.weight"], "matrix")
+            self.up = self._place(tensors["up.weight"], "matrix")
+
+        def paged_need(self):
+            return PagedNeed(num_heads=1, head_dim=0, planes=((1, LATENT), (1, POS)), dtype=torch.float32)
+
+        def forward(self, h, ctx, cache):
+            latent_plane, pos_plane = cache.planes                       # [pages, 1, page, 12] and [pages, 1, page, 4], float32
+            assert latent_plane.dtype == pos_plane.dtype == torch.float32 and latent_plane.shape[-1] == LATENT and pos_plane.shape[-1] == POS
+            page = cache.page_size
+            c = h.float() @ self.down.float().T
+            pos = ctx.positions.float()[:, None] * torch.tensor([0.3, 0.05], device=h.device)
+            feat = torch.cat((pos.sin(), pos.cos()), dim=-1)
+            table = ctx.block_tables[cache.group].long()
+            req = ctx.token_req.long()
+            where = table[req, ctx.positions.long() // page]
+            latent_plane[where, 0, ctx.positions.long() % page] = c
+            pos_plane[where, 0, ctx.positions.long() % page] = feat
+            out = torch.empty((h.shape[0], LATENT), dtype=torch.float32, device=h.device)
+            indptr, ctx_lens = ctx.req_indptr.tolist(), ctx.ctx_lens.tolist()
+            for r in range(len(ctx_lens)):
+                total = ctx_lens[r] + indptr[r + 1] - indptr[r]
+                blocks = table[r, : -(-total // page)]
+                cs = latent_plane[blocks, 0].reshape(-1, LATENT)[:total]
+                ps = pos_plane[blocks, 0].reshape(-1, POS)[:total]
+                for t in range(indptr[r], indptr[r + 1]):
+                    n = ctx_lens[r] + t - indptr[r] + 1
+                    a = torch.softmax(cs[:n] @ c[t] + ps[:n] @ feat[t], dim=0)
+                    out[t] = a @ cs[:n]
+            return (out @ self.up.float().T).to(h.dtype)
+
+    @dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyLatentForCausalLM"
+        vocab_size: int
+
+        def to_spec(self):
+            norm = RMSNormSpec(dim=H, eps=1e-6)
+            block = BlockSpec(mixer=LatentSpec(hidden=H), mixer_norm=norm, ffn_norm=norm, ffn=SwiGLUSpec(hidden=H, intermediate=48), mixer_name="mix")
+            return ModelSpec(vocab_size=self.vocab_size, hidden=H, layers=(block, block), order=(RunEntry(0), RunEntry(1)),
+                             final_norm=norm, tie_head=True, max_positions=4096)
+
+    register_architecture(ToyConfig)
+    try:
+        cfg = config_class("ToyLatentForCausalLM").from_dict(dict(vocab_size=VOCAB))
+        tensors = {k: (v * 8 if ".mix." in k else v) for k, v in random_tensors(cfg, seed=2, dtype=torch.float32).items()}
+        model = build_model(cfg, dtype, device=device, tensors=tensors)
+        runner = make_runner(model, page_size=4, num_pages=26, max_requests=3)
+        group = runner.cache.groups[0]
+        assert len(runner.cache.groups) == 1 and [tuple(t.shape) for t in group.tensors] == [(2, 26, 1, 4, LATENT), (2, 26, 1, 4, POS)]
+        assert {t.dtype for t in group.tensors} == {torch.float32}
+        g = torch.Generator().manual_seed(1)
+        seqs = {k: torch.randint(0, VOCAB, (n,), generator=g).tolist() for k, n in (("a", 37), ("b", 18), ("c", 29))}
+        whole = {}
+        for k, v in seqs.items():                                       # one at a time: the next one uses the same pages again
+            whole[k] = runner.step([StepEntry(k, v, list(range(len(v))))]).cpu()
+            runner.release(k)
+        got = {k: [] for k in seqs}
+        done = {k: 0 for k in seqs}
+        plan = [{"a": 9}, {"a": 1, "b": 7}, {"b": 1, "a": 14, "c": 2}, {"c": 5, "a": 1, "b": 10}, {"a": 12, "c": 22}]
+        for step in plan:
+            entries = [StepEntry(k, seqs[k][done[k]: done[k] + n], list(range(n))) for k, n in step.items()]
+            out = runner.step(entries).cpu()
+            at = 0
+            for k, n in step.items():
+                got[k].append(out[at: at + n]); at += n; done[k] += n
+                if done[k] == len(seqs[k]):
+                    runner.release(k)
+            runner.cache.check()
+        assert done == {k: len(v) for k, v in seqs.items()} and runner.cache.live_requests() == []
+        tol = dict(atol=2e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=3e-2, rtol=3e-2)
+        for k in seqs:
+            torch.testing.assert_close(torch.cat(got[k]), whole[k], **tol)
+        assert float(whole["a"].std()) > 0.05
+    finally:
+        unregister_architecture("ToyLatentForCausalLM")
+        MIXERS.unregister("toy_latent")

@@ -88,8 +88,9 @@ class GQAttention(Mixer):
         # which the rotary encoding turns neighbouring dimensions: the projection of a decode step
         # then rotates in its own epilogue.  Keys lie in the cache in that order too; scores are
         # sums over a head's dimensions and do not notice.
+        # (not with a `transform_qk` hook: it sees the heads' dimensions in the checkpoint's order)
         self.pair_layout = (self.dtype == torch.bfloat16 and self.position is not None
-                            and self.position.fused_inv_freq() is not None)
+                            and self.position.fused_inv_freq() is not None and self.transform_qk is None)
         rows = {"q": ops.pair_layout_rows(self.heads, self.head_dim), "k": ops.pair_layout_rows(self.kv_heads, self.head_dim)}
         order = lambda n, t: t[rows[n]] if self.pair_layout and n in rows else t
         self.w_qkv = self._place(torch.cat([order(n, tensors[f"{n}_proj.weight"]) for n in "qkv"], dim=0), "matrix")
@@ -113,7 +114,29 @@ class GQAttention(Mixer):
 
     takes_lazy_norm = True
 
+    # The step has three stages, each a method of its own, so that a mixer that differs from this one in one
+    # stage overrides that stage and keeps the others: projection of q, k, v with position encoding and cache
+    # write (`project`), attention of the queries over the cache (`attend`), output projection (`output`).
+    # A mixer that only needs to do something to the projected queries and keys before they are encoded and
+    # stored (a norm per head, say) defines `transform_qk`; the kernels that fuse projection, rotation and
+    # cache write are then left out, since they would rotate what has not been transformed yet.
+    transform_qk = None      # or: def transform_qk(self, q3, k3, ctx) -> None, in place on [T, heads, head_dim] views (k3 may be None)
+
     def forward(self, h, ctx, cache):
+        qkv = self.project(h, ctx, cache)
+        out = self.attend(qkv[:, : self.q_width], ctx, cache)
+        return self.output(out)
+
+    def _cache_views(self, ctx, cache):
+        # the cache hands out two planes of [pages, kv_heads, page, head_dim]; this mixer keeps the
+        # values of a page transposed, [kv_heads, head_dim, page], as its kernels read them
+        k_plane, v_plane = cache.planes
+        v_plane = v_plane.view(v_plane.shape[0], self.kv_heads, self.head_dim, cache.page_size)
+        return k_plane, v_plane, ctx.block_tables[cache.group]
+
+    def project(self, h, ctx, cache):
+        """``[T, q_width (+ 2 kv_width)]``: position-encoded queries in the first ``q_width`` columns; the encoded
+        keys and the values of the step's tokens are in their pages when this returns (if the run owns its cache)."""
         lazy = h if isinstance(h, LazyNorm) else None      # one row whose norm the projection's kernel can make itself
         device = lazy.residual.device if lazy is not None else h.device
         T = 1 if lazy is not None else h.shape[0]
@@ -122,18 +145,14 @@ class GQAttention(Mixer):
         w = self.w_qkv if writes else self.w_qkv[: self.q_width]
         b = self.b_qkv if (self.b_qkv is None or writes) else self.b_qkv[: self.q_width]
         qkv = torch.empty((T, width), dtype=self.dtype, device=device)
-
-        # the cache hands out two planes of [pages, kv_heads, page, head_dim]; this mixer keeps the
-        # values of a page transposed, [kv_heads, head_dim, page], as its kernels read them
-        k_plane, v_plane = cache.planes
-        v_plane = v_plane.view(v_plane.shape[0], self.kv_heads, self.head_dim, cache.page_size)
-        table = ctx.block_tables[cache.group]
+        k_plane, v_plane, table = self._cache_views(ctx, cache)
         kv_heads = self.kv_heads if writes else 0
         inv_freq = self.position.fused_inv_freq() if self.position is not None else None
         cache_args = (ctx.token_req, table, k_plane, v_plane, cache.page_size) if writes else (None, None, None, None, 0)
+        plain = self.transform_qk is not None               # nothing fused: the hook sits between projection and rotation
         fused = False
         if lazy is not None:
-            if self.pair_layout:
+            if self.pair_layout and not plain:
                 residual_out = torch.empty_like(lazy.residual)
                 fused = ops.linear_rope_cache_write_normed(lazy.residual, lazy.pending, lazy.norm.weight, lazy.norm.eps,
                                                            residual_out, w, b, qkv, self.heads, self.kv_heads, self.head_dim,
@@ -142,25 +161,33 @@ class GQAttention(Mixer):
                     lazy.done(residual_out)
             if not fused:
                 h = lazy.value()
-        fused = fused or (self.pair_layout and ops.linear_rope_cache_write(h, w, b, qkv, self.heads, self.kv_heads, self.head_dim,
-                                                                           ctx.positions, inv_freq, *cache_args))
-        if not fused and self.dtype == torch.bfloat16 and (inv_freq is not None or self.position is None) \
+        fused = fused or (self.pair_layout and not plain and
+                          ops.linear_rope_cache_write(h, w, b, qkv, self.heads, self.kv_heads, self.head_dim,
+                                                      ctx.positions, inv_freq, *cache_args))
+        if not fused and not plain and self.dtype == torch.bfloat16 and (inv_freq is not None or self.position is None) \
                 and ops.linear_partials_pay(T, width, self.hidden):
             # few rows against a narrow matrix: K split over work-groups; the rotation kernel adds the slabs up
             ops.rope_cache_write(qkv, self.heads, kv_heads, self.head_dim, self.heads + kv_heads, ctx.positions, inv_freq,
                                  *cache_args, pairs=self.pair_layout, parts=ops.linear_partials(h, w), bias=b)
         elif not fused:
             ops.linear(h, w, b, qkv)
+            q3 = qkv[:, : self.q_width].unflatten(1, (self.heads, self.head_dim))
+            k3 = qkv[:, self.q_width: self.q_width + self.kv_width].unflatten(1, (self.kv_heads, self.head_dim)) if writes else None
+            if plain:
+                self.transform_qk(q3, k3, ctx)
             if self.position is not None and inv_freq is None:
-                q3 = qkv[:, : self.q_width].unflatten(1, (self.heads, self.head_dim))
-                k3 = qkv[:, self.q_width: self.q_width + self.kv_width].unflatten(1, (self.kv_heads, self.head_dim)) if writes else None
                 self.position.apply(q3, k3, ctx.positions)
             if inv_freq is not None or writes:
                 ops.rope_cache_write(qkv, self.heads, kv_heads, self.head_dim, self.heads + kv_heads, ctx.positions, inv_freq,
                                      *cache_args, pairs=self.pair_layout)
+        return qkv
 
-        out = torch.empty((T, self.q_width), dtype=self.dtype, device=device)
-        q = qkv[:, : self.q_width]
+    def attend(self, q, ctx, cache):
+        """Causal (and windowed) attention of the step's queries ``q [T, q_width]`` (a row-strided view) over their
+        requests' cached keys and values: ``[T, q_width]``."""
+        T = q.shape[0]
+        k_plane, v_plane, table = self._cache_views(ctx, cache)
+        out = torch.empty((T, self.q_width), dtype=self.dtype, device=q.device)
         common = (self.heads, self.kv_heads, self.head_dim, cache.page_size, self.window or 0, self.scale)
         rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size, -(-ctx.max_total_len // cache.page_size))
                    and ctx.max_new_tokens >= _PORTION_MIN_TOKENS)
@@ -193,9 +220,15 @@ class GQAttention(Mixer):
                 tile_req = tile_tok0 = None
             ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
                                 tile_req, tile_tok0, tiles, self.tile_tokens, *common, self._splits(ctx, tiles))
+        return out
+
+    def output(self, out):
+        """The output projection (no bias) of the mixed heads ``[T, q_width]``: ``[T, hidden]``, or float32 slabs of
+        partial sums ``[P, T, hidden]`` that the next norm adds up."""
+        T = out.shape[0]
         if self.dtype == torch.bfloat16 and ops.linear_partials_pay(T, self.hidden, self.q_width):
             # few rows against a narrow matrix: K split over work-groups; the next norm adds the slabs up
             return ops.linear_partials(out, self.w_o)
-        y = torch.empty((T, self.hidden), dtype=self.dtype, device=device)
+        y = torch.empty((T, self.hidden), dtype=self.dtype, device=out.device)
         ops.linear(out, self.w_o, None, y)
         return y

@@ -204,6 +204,29 @@ def test_linear_few_rows_in_32_bit(ops, M, N, K):
     assert bool((out2[:, N:] == 3.0).all())
 
 
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("N,K,blocks,rows", [(3584, 512, 1, 14), (4608, 320, 2, 18), (1000, 200, 1, 4), (1003, 128, 2, 31),
+                                             (530, 264, 2, 17), (4099, 64, 1, 16), (700, 96, 1, 1)])
+def test_linear_few_rows_in_strips_of_any_number_of_rows(ops, M, N, K, blocks, rows):
+    """A matrix dealt to the compute units in equal shares: strips of a number of weight rows that is no
+    multiple of 16, a last strip that is shorter still; every output written once, nothing beside them."""
+    g = torch.Generator().manual_seed(M + N + rows)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).cuda()
+    b = torch.randn(N, generator=g).to(torch.bfloat16).cuda()
+    ref = x.double() @ w.double().T + b.double()
+    wide = torch.full((M + 1, N + 9), float("nan"), device="cuda")
+    ops.linear_few_rows_variant(x, w, b, wide[:M, :N], blocks, 8, rows)
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    torch.testing.assert_close(wide[:M, :N].double(), ref, **tol32)
+    assert bool(wide[:M, N:].isnan().all()) and bool(wide[M].isnan().all())
+    plain = torch.empty(M, N, device="cuda")
+    ops.linear_few_rows_variant(x, w, b, plain, blocks, 8, 0)
+    assert torch.equal(plain, wide[:M, :N]), "the sums of a row do not depend on the strip it lies in"
+    with pytest.raises(ops.KernelError, match="holds up to"):
+        ops.linear_few_rows_variant(x, w, b, plain, blocks, 8, 16 * blocks + 1)
+
+
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
 @pytest.mark.parametrize("N,K", [(48, 64), (129, 200), (4608, 3584), (3584, 1000), (16400, 256), (33000, 128)])

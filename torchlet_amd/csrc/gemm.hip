@@ -344,7 +344,7 @@ extern "C" int tl_gemm_f32_variant(const void* x, const void* w, const void* bia
 // the result is deterministic.  One row of x is as good as free (the lanes of a wave that read the
 // same address share the fetch); with more rows x costs M / 16 of the weight traffic again, so it is
 // copied into shared memory (XL) by no more work-groups than the compute units hold at once, each
-// of which then walks the strips blockIdx.x, blockIdx.x + gridDim.x, ... and requests the first
+// of which then walks a run of outputs of its own, strip after strip, and requests the first
 // steps of its next strip before it adds up the sums of this one (measured at M = 8, 7B sizes:
 // gate/up 57 -> 51 us, LM head 207 -> 189 us).
 // Needs K % 8 == 0 and 16-byte aligned rows; other shapes go to the general kernel.
@@ -449,10 +449,11 @@ template <int R, int MT, int KS, typename TOut, bool SW = false, bool XL = false
 __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                               const void* __restrict__ bias, int bias_f32,
                                                               TOut* __restrict__ out, int M, int N, int K, int ldx, int ldo,
-                                                              int out_cols, int k_per_split, RopeArgs ra, NormArgs na) {
+                                                              int out_cols, int k_per_split, int rows_per_strip, int rows_per_group,
+                                                              RopeArgs ra, NormArgs na) {
     static_assert(!NF || (XL && MT == 1), "the fused norm makes x in shared memory, for one row");
     static_assert(!SW || (R == 1 && KS % 2 == 0), "the fused gate deals a work-group's waves to a gate strip and its up strip");
-    static_assert(!RP || (R == 1 && MT == 1 && !SW), "the fused rotation is built for one strip and up to 16 rows");
+    static_assert(!RP || (R <= 2 && MT == 1 && !SW), "the fused rotation is built for up to 16 rows of x");
     // Split K (k_per_split > 0, a multiple of 64): blockIdx.y owns the columns
     // [y * k_per_split, ...) of x and w and writes its own [M, ldo] slab of partial sums to out
     // (float, no bias); whoever reads them adds the slabs up.
@@ -469,17 +470,31 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
     bf16_t* xs = (bf16_t*)(skinny_lds + KS * R * MT * 256);             // XL: M rows of K + 8 elements
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
-    // A work-group takes the strips of 16 R weight rows blockIdx.x, blockIdx.x + gridDim.x, ...: with
-    // fewer work-groups than strips, x is copied into shared memory (XL) once for all of them, and the
-    // first fetches of the next strip are on their way while the sums of this one are added up.
-    // With the fused gate (SW) a strip is 16 outputs: the first KS / 2 waves walk K for their 16 gate rows,
-    // the others for the 16 up rows of the same outputs (the interleaved matrix holds blocks of 32 gate
-    // rows followed by their 32 up rows), and the sums of both meet in shared memory.
+    // The outputs (weight rows; with the fused gate, SW, pairs of a gate row and an up row) are dealt to the
+    // work-groups in runs of rows_per_group, and a work-group walks its run in strips of rows_per_strip, up to
+    // 16 R (0: exactly that; rows_per_group 0: one strip).  A compute unit draws its weights at a rate of its
+    // own, about 26 GB/s whatever it shares the chip with, so a product takes as long as its busiest unit: 257
+    // strips of 16 rows take as long as 512 (11.2 against 7.9 us for 256, at 3584 columns), and equal shares for
+    // all work-groups are worth more than full blocks of 16 rows.  Lanes beyond a strip's last row fetch copies
+    // of it and store nothing.  Only with x in shared memory (XL) does a work-group walk more than one strip:
+    // x is copied (or made, NF) once for all of them, and the first fetches of the next strip are on their way
+    // while the sums of this one are added up.
+    // With the fused gate the first KS / 2 waves walk K for the gate rows of the strip's outputs, the others
+    // for the up rows of the same outputs (the interleaved matrix holds blocks of 32 gate rows followed by
+    // their 32 up rows), and the sums of both meet in shared memory.
     constexpr int KW = SW ? KS / 2 : KS;       // waves along K per strip
     const int kwave = SW ? wave % KW : wave;
-    const int strips = SW ? N / 32 : (N + 16 * R - 1) / (16 * R);
-    auto first_row = [&](int st) { return SW ? (st / 2) * 64 + (wave / KW) * 32 + (st % 2) * 16 : st * (16 * R); };
-    int strip = blockIdx.x;
+    const int total = SW ? out_cols : N;
+    const int rps = rows_per_strip > 0 ? rows_per_strip : 16 * R;
+    const int run_begin = blockIdx.x * ((XL && rows_per_group > 0) ? rows_per_group : rps);
+    const int run_end = min(total, run_begin + ((XL && rows_per_group > 0) ? rows_per_group : rps));
+    auto strip_begin = [&](int i) { return run_begin + i * rps; };
+    auto strip_end = [&](int i) { return min(run_begin + i * rps + rps, run_end); };
+    auto lane_row = [&](int i, int r) {        // the weight row this lane fetches for block r of strip i
+        const int o = min(strip_begin(i) + r * 16 + li, strip_end(i) - 1);
+        return SW ? (o >> 5) * 64 + (wave / KW) * 32 + (o & 31) : o;
+    };
+    int strip = 0;
     int rp_pos = 0, rp_page = 0;               // RP: this lane's row (li), fetched now, used in the epilogue
     if (RP) {
         const int row = min(li, M - 1);
@@ -491,7 +506,7 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
     const bf16_t* xrow[MT];
     int xoff[MT];
 #pragma unroll
-    for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)min(first_row(strip) + r * 16 + li, N - 1) * ldw;
+    for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)lane_row(strip, r) * ldw;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         xrow[t] = x + (size_t)min(t * 16 + li, M - 1) * ldx;
@@ -580,7 +595,8 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
         lds_barrier();
     }
     while (true) {
-        const int n0 = strip * (16 * R);       // (not SW) first output column of the strip
+        const int n0 = strip_begin(strip);     // first output column of the strip
+        const int n_end = strip_end(strip);    // ... and the one after its last
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -641,10 +657,10 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
                     acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[r].v, b1[t].v, acc[r][t], 0, 0, 0);
                 }
         }
-        const int next = XL ? strip + (int)gridDim.x : strips;      // without the copy of x: one strip per work-group
-        if (next < strips) {                   // the next strip's first steps, before this strip's sums
+        const bool more = XL && strip_begin(strip + 1) < run_end;   // without the copy of x: one strip per work-group
+        if (more) {                            // the next strip's first steps, before this strip's sums
 #pragma unroll
-            for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)min(first_row(next) + r * 16 + li, N - 1) * ldw;
+            for (int r = 0; r < R; ++r) wrow[r] = w + (size_t)lane_row(strip + 1, r) * ldw;
 #pragma unroll
             for (int d = 0; d < D; ++d)
                 if (d < mine) SK_ISSUE(d, d)
@@ -670,11 +686,11 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
                     us += *(const f32x4_t*)(red + ((size_t)((KW + wv) * MT + t) * 64 + lane) * 4);
                 }
                 const int m = t * 16 + li;
-                const int col = strip * 16 + 4 * lg;
+                const int col = n0 + 4 * lg;
                 if (m < M) {
 #pragma unroll
                     for (int v = 0; v < 4; ++v)
-                        if (col + v < out_cols) out[(size_t)m * ldo + col + v] = from_float<TOut>(silu_mul(gs[v], us[v]));
+                        if (col + v < n_end) out[(size_t)m * ldo + col + v] = from_float<TOut>(silu_mul(gs[v], us[v]));
                 }
             }
         } else {
@@ -696,35 +712,37 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
                 const int m = t * 16 + li;
                 const int n = n0 + r * 16 + 4 * lg;
                 if (RP) {
-                    if (m >= M || n >= N) continue;                    // N is a multiple of 16 here
-                    float val[4];
+                    // two pairs of neighbouring columns per lane (pair layout: one frequency turns a pair); a strip
+                    // of a number of rows that is no multiple of four may end between them
+                    if (m >= M) continue;
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) val[v] = sum[v] + (bias ? load_vec(bias, bias_f32, n + v) : 0.f);
-                    const int head = n / ra.head_dim, dd = n - head * ra.head_dim;
-                    if (head < ra.q_heads + ra.kv_heads) {
-#pragma unroll
-                        for (int pr = 0; pr < 2; ++pr) {
-                            const float angle = (float)rp_pos * ra.inv_freq[dd / 2 + pr];
-                            const float c = cosf(angle), sn = sinf(angle);
-                            const float y1 = val[2 * pr] * c - val[2 * pr + 1] * sn;
-                            const float y2 = val[2 * pr + 1] * c + val[2 * pr] * sn;
-                            val[2 * pr] = y1;
-                            val[2 * pr + 1] = y2;
-                        }
-                    }
-                    union { uint2 u; uint16_t e[4]; } pk;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) pk.e[v] = from_float<bf16_t>(val[v]).bits;
-                    if (head < ra.q_heads || !ra.k_plane) {
-                        *(uint2*)((bf16_t*)out + (size_t)m * ldo + n) = pk.u;
-                    } else if (rp_page != 0) {         // page 0 is the sentinel (a padding row's): never written
-                        const int kvh = (head - ra.q_heads) % ra.kv_heads, off = rp_pos % ra.page;
-                        const size_t base = ((size_t)rp_page * ra.kv_heads + kvh) * ra.page * ra.head_dim;
+                    for (int pr = 0; pr < 2; ++pr) {
+                        const int np = n + 2 * pr;
+                        if (np + 1 >= n_end) continue;                 // strips hold an even number of rows
+                        float y1 = sum[2 * pr] + (bias ? load_vec(bias, bias_f32, np) : 0.f);
+                        float y2 = sum[2 * pr + 1] + (bias ? load_vec(bias, bias_f32, np + 1) : 0.f);
+                        const int head = np / ra.head_dim, dd = np - head * ra.head_dim;
                         if (head < ra.q_heads + ra.kv_heads) {
-                            *(uint2*)(ra.k_plane + base + (size_t)off * ra.head_dim + dd) = pk.u;
-                        } else {
-#pragma unroll
-                            for (int v = 0; v < 4; ++v) ra.v_plane[base + (size_t)(dd + v) * ra.page + off].bits = pk.e[v];
+                            const float angle = (float)rp_pos * ra.inv_freq[dd / 2];
+                            const float c = cosf(angle), sn = sinf(angle);
+                            const float t1 = y1 * c - y2 * sn;
+                            const float t2 = y2 * c + y1 * sn;
+                            y1 = t1;
+                            y2 = t2;
+                        }
+                        const uint16_t e1 = from_float<bf16_t>(y1).bits, e2 = from_float<bf16_t>(y2).bits;
+                        const uint32_t both = (uint32_t)e1 | ((uint32_t)e2 << 16);
+                        if (head < ra.q_heads || !ra.k_plane) {
+                            *(uint32_t*)((bf16_t*)out + (size_t)m * ldo + np) = both;
+                        } else if (rp_page != 0) {     // page 0 is the sentinel (a padding row's): never written
+                            const int kvh = (head - ra.q_heads) % ra.kv_heads, off = rp_pos % ra.page;
+                            const size_t base = ((size_t)rp_page * ra.kv_heads + kvh) * ra.page * ra.head_dim;
+                            if (head < ra.q_heads + ra.kv_heads) {
+                                *(uint32_t*)(ra.k_plane + base + (size_t)off * ra.head_dim + dd) = both;
+                            } else {
+                                ra.v_plane[base + (size_t)dd * ra.page + off].bits = e1;
+                                ra.v_plane[base + (size_t)(dd + 1) * ra.page + off].bits = e2;
+                            }
                         }
                     }
                     continue;
@@ -732,7 +750,7 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
                 if (m < M) {
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
-                        if (n + v < N) {
+                        if (n + v < n_end) {
                             float val = sum[v];
                             if (bias) val += load_vec(bias, bias_f32, n + v);
                             out[(size_t)m * ldo + n + v] = from_float<TOut>(val);
@@ -741,8 +759,8 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
                 }
             }
         }
-        if (next >= strips) break;
-        strip = next;
+        if (!more) break;
+        ++strip;
         if (KS > 1) lds_barrier();             // the sums are read until here; the next strip's overwrite them
     }
 #undef SK_ISSUE
@@ -758,27 +776,51 @@ static hipError_t allow_lds(Kernel kernel, size_t bytes) {
 #define SKINNY_XL_MAX_BYTES (60 * 1024)      // x may take this much shared memory: with the reduction buffer two
                                              // work-groups still fit the 160 KB of a compute unit
 
+// How the outputs of a product are dealt out: work-groups, the outputs of each (its run) and of a strip.
+struct StripPlan {
+    int groups, per_group, per_strip;
+};
+
+// Equal runs for up to `most` work-groups, each walked in equal strips of at most `cap` outputs (a multiple of
+// 16); `even` keeps both numbers even (the fused rotation turns pairs of neighbouring outputs).
+static StripPlan plan_strips(int total, int most, int cap, bool even) {
+    StripPlan p;
+    p.per_group = (total + most - 1) / most;
+    if (p.per_group < 4) p.per_group = 4;                     // a strip of fewer rows wastes most of its fetches
+    if (even) p.per_group += p.per_group & 1;
+    const int count = (p.per_group + cap - 1) / cap;
+    p.per_strip = (p.per_group + count - 1) / count;
+    if (even) p.per_strip += p.per_strip & 1;
+    p.groups = (total + p.per_group - 1) / p.per_group;
+    return p;
+}
+
+// rows_per_strip > 0: one strip of that many outputs per work-group, whatever else holds.
 template <int R, int MT, int KS, typename TOut, bool SW, int D>
 static void launch_skinny_d(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
-                            int ldx, int ldo, int out_cols, hipStream_t stream) {
-    const int strips = SW ? N / 32 : (N + 16 * R - 1) / (16 * R);
-    dim3 grid(strips), block(KS * 64);
+                            int ldx, int ldo, int out_cols, hipStream_t stream, int rows_per_strip = 0) {
+    const int total = SW ? out_cols : N;
+    const int rps = rows_per_strip > 0 ? rows_per_strip : 16 * R;
+    dim3 grid((total + rps - 1) / rps), block(KS * 64);
     const size_t red_bytes = (size_t)KS * R * MT * 1024;
     const size_t x_bytes = (size_t)M * (K + 8) * 2;
     // More than one row of x: two work-groups per compute unit copy x into shared memory once and walk
-    // the strips between them (each strip's own copy took longer than it saved: 87 against 64 us on the
+    // their runs of outputs (each strip's own copy took longer than it saved: 87 against 64 us on the
     // fused gate/up product at M = 8 with four waves).
     if (M > 1 && red_bytes + x_bytes <= 156 * 1024) {
         auto kernel = gemm_skinny_kernel<R, MT, KS, TOut, SW, true, D>;
         static hipError_t allowed = allow_lds(kernel, 156 * 1024);
         if (allowed == hipSuccess) {
             const int most = x_bytes <= SKINNY_XL_MAX_BYTES ? 512 : 256;      // a larger x leaves room for one work-group only
-            dim3 few(strips < most ? strips : most);
-            kernel<<<few, block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{}, NormArgs{});
+            StripPlan p = plan_strips(total, most, 16 * R, false);
+            if (rows_per_strip > 0) p = StripPlan{(int)grid.x, rps, rps};
+            kernel<<<dim3(p.groups), block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo,
+                                                                           out_cols, 0, p.per_strip, p.per_group, RopeArgs{}, NormArgs{});
             return;
         }
     }
-    gemm_skinny_kernel<R, MT, KS, TOut, SW, false, D><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo, out_cols, 0, RopeArgs{}, NormArgs{});
+    gemm_skinny_kernel<R, MT, KS, TOut, SW, false, D><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo,
+                                                                                          out_cols, 0, rps, 0, RopeArgs{}, NormArgs{});
 }
 
 // A wave with many K steps ahead of it (a long K: the down projection) keeps as many in flight as
@@ -786,19 +828,35 @@ static void launch_skinny_d(const void* x, const void* w, const void* bias, int 
 // (measured at 3584 x 18944, one row: 33 -> 28 us with eight in flight; at 4608 x 3584: 11 -> 12.6 us).
 template <int R, int MT, int KS, typename TOut, bool SW>
 static void launch_skinny_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
-                            int ldx, int ldo, int out_cols, hipStream_t stream) {
+                            int ldx, int ldo, int out_cols, hipStream_t stream, int rows_per_strip = 0) {
     constexpr int deep = skinny_depth<R, MT, KS>();
     if (deep > 2 && K / 64 / KS >= 16)
-        launch_skinny_d<R, MT, KS, TOut, SW, deep>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+        launch_skinny_d<R, MT, KS, TOut, SW, deep>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, rows_per_strip);
     else
-        launch_skinny_d<R, MT, KS, TOut, SW, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream);
+        launch_skinny_d<R, MT, KS, TOut, SW, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, rows_per_strip);
 }
 
 template <int R, int MT, int KS>
 static void launch_skinny(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
-                          int ldx, int ldo, int out_f32, hipStream_t stream) {
-    if (out_f32) launch_skinny_t<R, MT, KS, float, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
-    else launch_skinny_t<R, MT, KS, bf16_t, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
+                          int ldx, int ldo, int out_f32, hipStream_t stream, int rows_per_strip = 0) {
+    if (out_f32) launch_skinny_t<R, MT, KS, float, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream, rows_per_strip);
+    else launch_skinny_t<R, MT, KS, bf16_t, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream, rows_per_strip);
+}
+
+// Rows a strip gets so that a matrix of N rows is dealt to the compute units in equal shares, one strip to
+// each (0: the plain strips of 16 R rows are as good; *blocks: how many blocks of 16 rows a strip then has, 1 or
+// 2).  A compute unit draws its weights at a rate of its own, about 26 GB/s whatever shares it with, so a product
+// takes as long as its busiest unit: at 3584 columns 256 strips of 16 rows take 7.9 us, 257 take 11.2, 288 (the
+// 7B's query/key/value matrix) 11.9 and 512 take 13.4.  The number is even (the fused rotation turns pairs).
+#define TL_COMPUTE_UNITS 256
+static int balanced_rows(int N, int* blocks) {
+    *blocks = 1;
+    if (N < 4 * TL_COMPUTE_UNITS || N > 32 * TL_COMPUTE_UNITS) return 0;      // a few rows a unit, or more than two blocks
+    if (N % (16 * TL_COMPUTE_UNITS) == 0) return 0;                               // whole blocks already come out even
+    int rows = (N + TL_COMPUTE_UNITS - 1) / TL_COMPUTE_UNITS;
+    rows += rows & 1;
+    *blocks = rows > 16 ? 2 : 1;
+    return rows;
 }
 
 template <int MT>
@@ -810,6 +868,12 @@ static void pick_skinny(const void* x, const void* w, const void* bias, int bias
     // ones (qkv, o, down); with 64 rows the x operand weighs more and several strips per wave
     // share each x load.
     const int strips = (N + 15) / 16;
+    if (MT == 1) {
+        int blocks = 1;
+        const int rows = balanced_rows(N, &blocks);
+        if (rows > 0 && blocks == 1) return launch_skinny<1, 1, 8>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream, rows);
+        if (rows > 0) return launch_skinny<2, 1, 8>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream, rows);
+    }
     if (MT <= 2) {
         if (strips >= 1024) launch_skinny<1, MT, 16>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
         else launch_skinny<1, MT, 8>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream);
@@ -820,15 +884,18 @@ static void pick_skinny(const void* x, const void* w, const void* bias, int bias
     }
 }
 
-// One named instance of the few-rows kernel, of those the dispatch below can pick (for tests and tuning).
+// One named instance of the few-rows kernel, of those the dispatch below can pick (for tests and tuning);
+// rows_per_strip: 0 for strips of 16 R rows, else that many (at most 16 R).
 extern "C" int tl_gemm_skinny_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
-                                      int M, int N, int K, int ldx, int ldo, int out_f32, int R, int KS, hipStream_t stream) {
+                                      int M, int N, int K, int ldx, int ldo, int out_f32, int R, int KS, int rows_per_strip,
+                                      hipStream_t stream) {
     TL_REQUIRE(M > 0 && M <= 64 && K % 8 == 0 && ldx % 8 == 0, "gemm_skinny: needs 0 < M <= 64 and K, ldx multiples of 8");
+    TL_REQUIRE(rows_per_strip >= 0 && rows_per_strip <= 16 * R, "gemm_skinny: a strip of %d blocks holds up to %d rows, not %d", R, 16 * R, rows_per_strip);
     const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
 #define TL_SKINNY_CASE(r, t, k) \
-    if (R == r && MT == t && KS == k) { launch_skinny<r, t, k>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream); TL_CHECK_LAUNCH("gemm_skinny"); return TL_OK; }
+    if (R == r && MT == t && KS == k) { launch_skinny<r, t, k>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_f32, stream, rows_per_strip); TL_CHECK_LAUNCH("gemm_skinny"); return TL_OK; }
     // the instances pick_skinny can choose
-    TL_SKINNY_CASE(1, 1, 16) TL_SKINNY_CASE(1, 2, 16) TL_SKINNY_CASE(1, 1, 8) TL_SKINNY_CASE(1, 2, 8)
+    TL_SKINNY_CASE(1, 1, 16) TL_SKINNY_CASE(1, 2, 16) TL_SKINNY_CASE(1, 1, 8) TL_SKINNY_CASE(1, 2, 8) TL_SKINNY_CASE(2, 1, 8)
     TL_SKINNY_CASE(4, 4, 4) TL_SKINNY_CASE(2, 4, 2) TL_SKINNY_CASE(1, 4, 8)
 #undef TL_SKINNY_CASE
     TL_REQUIRE(false, "gemm_skinny: no instance R=%d MT=%d KS=%d", R, MT, KS);
@@ -1497,14 +1564,15 @@ extern "C" int tl_gemm(const void* x, const void* w, const void* bias, int bias_
 // are in the pair layout).  Returns TL_NOT_FUSED (nothing launched) for shapes it is not built for;
 // the caller then runs the product and the rotation as two kernels.
 #define TL_NOT_FUSED 100
-template <int KS, bool XL>
+template <int KS, bool XL, int R = 1>
 static void launch_skinny_rope(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
-                               int ldx, int ldo, const RopeArgs& ra, hipStream_t stream) {
-    dim3 grid((N + 15) / 16), block(KS * 64);
-    const size_t lds = (size_t)KS * 1024 + (XL ? (size_t)M * (K + 8) * 2 : 0);
-    auto kernel = gemm_skinny_kernel<1, 1, KS, bf16_t, false, XL, 2, true>;
+                               int ldx, int ldo, const RopeArgs& ra, hipStream_t stream, int rows_per_strip = 0) {
+    const int rps = rows_per_strip > 0 ? rows_per_strip : 16 * R;
+    dim3 grid((N + rps - 1) / rps), block(KS * 64);
+    const size_t lds = (size_t)KS * R * 1024 + (XL ? (size_t)M * (K + 8) * 2 : 0);
+    auto kernel = gemm_skinny_kernel<R, 1, KS, bf16_t, false, XL, 2, true>;
     if (XL) { static hipError_t allowed = allow_lds(kernel, 96 * 1024); (void)allowed; }
-    kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo, 0, 0, ra, NormArgs{});
+    kernel<<<grid, block, lds, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, M, N, K, ldx, ldo, 0, 0, rps, 0, ra, NormArgs{});
 }
 
 extern "C" int tl_gemm_partials_pay(int M, int N, int K);
@@ -1529,7 +1597,10 @@ extern "C" int tl_gemm_rope(const void* x, const void* w, const void* bias, int 
     ra.block_table = (const int*)block_table; ra.k_plane = (bf16_t*)k_plane; ra.v_plane = (bf16_t*)v_plane;
     ra.bt_stride = bt_stride; ra.page = page > 0 ? page : 1; ra.q_heads = q_heads; ra.kv_heads = k_plane ? kv_heads : 0; ra.head_dim = head_dim;
     const bool xl = M > 1 && (size_t)M * (K + 8) * 2 <= SKINNY_XL_MAX_BYTES;
-    if (ks == 8) { if (xl) launch_skinny_rope<8, true>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); else launch_skinny_rope<8, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); }
+    int blocks = 1;
+    const int rows = ks == 8 ? balanced_rows(N, &blocks) : 0;
+    if (rows > 0 && blocks == 2) { if (xl) launch_skinny_rope<8, true, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream, rows); else launch_skinny_rope<8, false, 2>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream, rows); }
+    else if (ks == 8) { if (xl) launch_skinny_rope<8, true>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream, rows); else launch_skinny_rope<8, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream, rows); }
     else { if (xl) launch_skinny_rope<16, true>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); else launch_skinny_rope<16, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, ra, stream); }
     TL_CHECK_LAUNCH("gemm_rope");
     return TL_OK;
@@ -1573,14 +1644,19 @@ extern "C" int tl_gemm_rope_normed(const void* residual, void* residual_out, con
     ra.positions = (const int*)positions; ra.inv_freq = (const float*)inv_freq; ra.token_req = (const int*)token_req;
     ra.block_table = (const int*)block_table; ra.k_plane = (bf16_t*)k_plane; ra.v_plane = (bf16_t*)v_plane;
     ra.bt_stride = bt_stride; ra.page = page > 0 ? page : 1; ra.q_heads = q_heads; ra.kv_heads = k_plane ? kv_heads : 0; ra.head_dim = head_dim;
-    dim3 grid(strips);
-    const size_t lds = (size_t)ks * 1024 + (size_t)(K + 8) * 2;
-    if (ks == 8)
+    int blocks = 1;
+    const int rows = ks == 8 ? balanced_rows(N, &blocks) : 0;
+    dim3 grid(rows > 0 ? (N + rows - 1) / rows : strips);
+    const size_t lds = (size_t)ks * blocks * 1024 + (size_t)(K + 8) * 2;
+    if (rows > 0 && blocks == 2)
+        gemm_skinny_kernel<2, 1, 8, bf16_t, false, true, 2, true, true><<<grid, dim3(8 * 64), lds, stream>>>(
+            nullptr, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, 1, N, K, K, ldo, 0, 0, rows, 0, ra, na);
+    else if (ks == 8)
         gemm_skinny_kernel<1, 1, 8, bf16_t, false, true, 2, true, true><<<grid, dim3(8 * 64), lds, stream>>>(
-            nullptr, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, 1, N, K, K, ldo, 0, 0, ra, na);
+            nullptr, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, 1, N, K, K, ldo, 0, 0, rows, 0, ra, na);
     else
         gemm_skinny_kernel<1, 1, 16, bf16_t, false, true, 2, true, true><<<grid, dim3(16 * 64), lds, stream>>>(
-            nullptr, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, 1, N, K, K, ldo, 0, 0, ra, na);
+            nullptr, (const bf16_t*)w, bias, bias_f32, (bf16_t*)out, 1, N, K, K, ldo, 0, 0, 0, 0, ra, na);
     TL_CHECK_LAUNCH("gemm_rope_normed");
     return TL_OK;
 }
@@ -1595,11 +1671,10 @@ extern "C" int tl_gemm_swiglu_normed(const void* residual, void* residual_out, c
     const int N = ((I + 31) / 32) * 64;          // rows of the interleaved matrix
     if (!norm_fits(na, K, 16 * 64) || ((uintptr_t)w % 16) || K / 64 / 16 >= 16)
         return TL_NOT_FUSED;
-    const int strips = N / 32;
-    dim3 grid(strips < 512 ? strips : 512);       // every work-group makes x once and walks its strips
+    const StripPlan p = plan_strips(I, 512, 16, false);       // every work-group makes x once and walks its run of outputs
     const size_t lds = (size_t)16 * 1024 + (size_t)(K + 8) * 2;
-    gemm_skinny_kernel<1, 1, 16, bf16_t, true, true, 2, false, true><<<grid, dim3(16 * 64), lds, stream>>>(
-        nullptr, (const bf16_t*)w, nullptr, 0, (bf16_t*)out, 1, N, K, K, I, I, 0, RopeArgs{}, na);
+    gemm_skinny_kernel<1, 1, 16, bf16_t, true, true, 2, false, true><<<dim3(p.groups), dim3(16 * 64), lds, stream>>>(
+        nullptr, (const bf16_t*)w, nullptr, 0, (bf16_t*)out, 1, N, K, K, I, I, 0, p.per_strip, p.per_group, RopeArgs{}, na);
     TL_CHECK_LAUNCH("gemm_swiglu_normed");
     return TL_OK;
 }
@@ -1719,14 +1794,14 @@ extern "C" int tl_gemm_partials(const void* x, const void* w, void* out, int M, 
     dim3 grid((N + 63) / 64, P), block(8 * 64);
     const size_t red_bytes = (size_t)8 * 4 * (M <= 16 ? 1 : (M <= 32 ? 2 : 4)) * 1024;
     if (M <= 16)
-        gemm_skinny_kernel<4, 1, 8, float, false, false, skinny_depth<4, 1, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{}, NormArgs{});
+        gemm_skinny_kernel<4, 1, 8, float, false, false, skinny_depth<4, 1, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, 0, 0, RopeArgs{}, NormArgs{});
     else if (M <= 32)
-        gemm_skinny_kernel<4, 2, 8, float, false, false, skinny_depth<4, 2, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{}, NormArgs{});
+        gemm_skinny_kernel<4, 2, 8, float, false, false, skinny_depth<4, 2, 8>()><<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, 0, 0, RopeArgs{}, NormArgs{});
     else {
         auto kernel = gemm_skinny_kernel<4, 4, 8, float, false, false, skinny_depth<4, 4, 8>()>;
         static hipError_t allowed = allow_lds(kernel, 128 * 1024);
         TL_REQUIRE(allowed == hipSuccess, "gemm_partials: cannot get %zu bytes of shared memory", red_bytes);
-        kernel<<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, RopeArgs{}, NormArgs{});
+        kernel<<<grid, block, red_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, nullptr, 0, (float*)out, M, N, K, ldx, N, 0, k_per, 0, 0, RopeArgs{}, NormArgs{});
     }
     TL_CHECK_LAUNCH("gemm_partials");
     return TL_OK;

@@ -201,8 +201,9 @@ def linear_f32_variant(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
                                         c_int(x.stride(0)), c_int(out.stride(0)), c_int(1 if matrix_cores else 0), _stream()))
 
 
-def linear_few_rows_variant(x, weight, bias, out, strips_per_wave: int, waves_along_k: int) -> None:
-    """One named instance of the few-rows matrix-core kernel (for tests and tuning)."""
+def linear_few_rows_variant(x, weight, bias, out, strips_per_wave: int, waves_along_k: int, rows_per_strip: int = 0) -> None:
+    """One named instance of the few-rows matrix-core kernel (for tests and tuning); ``rows_per_strip``: the weight
+    rows a work-group takes, up to 16 ``strips_per_wave`` (0: exactly that many)."""
     M, K = x.shape
     N = weight.shape[0]
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or out.shape != (M, N) or not weight.is_contiguous():
@@ -212,7 +213,7 @@ def linear_few_rows_variant(x, weight, bias, out, strips_per_wave: int, waves_al
     _check(lib, lib.tl_gemm_skinny_variant(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N),
                                            c_int(K), c_int(x.stride(0)), c_int(out.stride(0)),
                                            c_int(1 if out.dtype == torch.float32 else 0), c_int(strips_per_wave),
-                                           c_int(waves_along_k), _stream()))
+                                           c_int(waves_along_k), c_int(rows_per_strip), _stream()))
 
 
 def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int, slab: int = 32) -> None:

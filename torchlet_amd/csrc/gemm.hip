@@ -1108,6 +1108,13 @@ __device__ __forceinline__ void load_to_lds(const void* gptr, unsigned lds_addr)
 template <int N>
 __device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
+// Rows of one slab in shared memory: the BM rows of x and the BN rows of w, rounded up to what the waves'
+// load instructions (64 lanes x 16 bytes each) fill between them.
+constexpr int dl_slab_rows(int bm, int bn, int waves, int tk) {
+    const int per = (64 / (tk / 8)) * waves;
+    return (bm + bn + per - 1) / per * per;
+}
+
 template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW = false, int TK = 64>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                                       const void* __restrict__ bias, int bias_f32,
@@ -1135,10 +1142,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
     constexpr int WM = BM / WGM, WN = BN / WGN;          // wave tile
     constexpr int FM = WM / 32, FN = WN / 32;            // 32x32 blocks per wave
     constexpr int ROWS = BM + BN;
-    constexpr int LOADS = ROWS / RPL / NW;               // load instructions per wave and slab (RPL rows each)
-    static_assert(ROWS % (RPL * NW) == 0, "slab rows must divide over the waves");
+    constexpr int LROWS = dl_slab_rows(BM, BN, NW, TK);  // a slab's rows in shared memory: ROWS, rounded up so that ...
+    constexpr int LOADS = LROWS / RPL / NW;              // ... every wave issues as many load instructions per slab (RPL rows each)
     static_assert(LOADS * (STAGES - 1) < 64, "outstanding loads must fit the counter");
-    extern __shared__ __attribute__((aligned(16))) bf16_t lds_raw[];   // [STAGES][ROWS][TK]
+    extern __shared__ __attribute__((aligned(16))) bf16_t lds_raw[];   // [STAGES][LROWS][TK]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -1165,7 +1172,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
         const int base_row = RPL * (wave + j * NW);
-        const int row = base_row + lane / PPR;
+        const int row = min(base_row + lane / PPR, ROWS - 1);      // (rows of the rounding: copies of the last row, never read)
         const int c = (lane % PPR) ^ DL_SWZ(row);
         if (row < BM) src[j] = x + (size_t)min(m0 + row, M - 1) * ldx + c * 8;
         else src[j] = w + (size_t)min(n0 + row - BM, N - 1) * ldw + c * 8;
@@ -1208,7 +1215,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
     };
     auto request_slab = [&](int slab) {
         const int k0 = min(slab, slabs - 1) * TK;
-        const unsigned nb = lds_base + (slab % STAGES) * ROWS * TK * 2;
+        const unsigned nb = lds_base + (slab % STAGES) * LROWS * TK * 2;
 #pragma unroll
         for (int j = 0; j < LOADS; ++j) load_to_lds(src[j] + k0, nb + ldst[j]);
     };
@@ -1222,7 +1229,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
 
     constexpr int PHASES = TK / 16;
     for (int sl = 0; sl < slabs; ++sl) {
-        const bf16_t* cb = lds_raw + (sl % STAGES) * ROWS * TK;
+        const bf16_t* cb = lds_raw + (sl % STAGES) * LROWS * TK;
 #pragma unroll
         for (int kk = 0; kk < PHASES; ++kk) {
             const int cur = kk & 1, nxt = cur ^ 1;
@@ -1232,7 +1239,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
                 wait_direct_loads<(STAGES - 2) * LOADS>();
                 __syncthreads();
                 request_slab(sl + STAGES);
-                read_operands(nxt, lds_raw + ((sl + 1) % STAGES) * ROWS * TK, 0);
+                read_operands(nxt, lds_raw + ((sl + 1) % STAGES) * LROWS * TK, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1337,11 +1344,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
 // (DL_128x128_S4: 128 x 128 with four slabs in shared memory, one work-group to a compute unit: for products of up
 // to 128 rows split over K, where what counts is how many bytes of weights a work-group has on their way; measured
 // at 128 rows against the best other tile: 3584 x 18944 48.8 -> 37.1 us, 3584 x 3584 18.6 -> 15.8, 5120 x 5120 29.7 -> 21.4)
-enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_64x128, DL_128x128_S4, DL_TILES };
-static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 192, 256, 256, 64, 128};
-static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256, 128, 128};
-static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12, 2.1e12, 4.2e12};   // FLOP/s of one compute unit
-static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6, 5e-6, 4.5e-6};       // seconds per tile
+enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_64x128, DL_128x128_S4, DL_64x192, DL_128x192, DL_TILES };
+static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 192, 256, 256, 64, 128, 64, 128};
+static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256, 128, 128, 192, 192};
+static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12, 2.1e12, 4.2e12, 3.0e12, 4.4e12};   // FLOP/s of one compute unit
+static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6, 5e-6, 4.5e-6, 9e-6, 9e-6};       // seconds per tile
 
 // Seconds for `groups` work-groups of tile t over k columns each.  The two smallest tiles run two
 // to a compute unit: each then works at half the unit's rate, and one that has a unit to itself
@@ -1411,7 +1418,7 @@ static DlSplit plan_dl_split(int M, int N, int K) {
 template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW, int TK = 64>
 static int launch_dl_tile_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                             int ldx, int ldo, int out_cols, hipStream_t stream, int parts = 1, int k_per = 0) {
-    constexpr size_t lds = (size_t)STAGES * (BM + BN) * TK * sizeof(bf16_t);
+    constexpr size_t lds = (size_t)STAGES * dl_slab_rows(BM, BN, WGM * WGN, TK) * TK * sizeof(bf16_t);
     auto kernel = gemm_dl_tile_kernel<BM, BN, WGM, WGN, STAGES, TOut, SW, TK>;
     static hipError_t allowed = allow_lds(kernel, lds);
     if (allowed != hipSuccess) {
@@ -1437,6 +1444,8 @@ static int launch_dl_tile(DlTile tile, const void* x, const void* w, const void*
     case DL_128x256: return launch_dl_tile_t<128, 256, 2, 4, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_256x128: return launch_dl_tile_t<256, 128, 4, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_64x128: return launch_dl_tile_t<64, 128, 1, 2, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+    case DL_64x192: return launch_dl_tile_t<64, 192, 1, 3, 4, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+    case DL_128x192: return launch_dl_tile_t<128, 192, 2, 3, 3, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_192x256: return launch_dl_tile_t<192, 256, 2, 4, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
     case DL_256x192:
         if constexpr (!SW) return launch_dl_tile_t<256, 192, 4, 2, 2, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
@@ -1476,6 +1485,22 @@ extern "C" int tl_gemm_direct_variant(const void* x, const void* w, const void* 
     TL_REQUIRE(tile >= 0, "gemm_direct: no tile of %d x %d", BM, BN);
     const int rc = out_f32 ? launch_dl_tile<float, false>((DlTile)tile, x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream)
                            : launch_dl_tile<bf16_t, false>((DlTile)tile, x, w, bias, bias_f32, out, M, N, K, ldx, ldo, 0, stream);
+    if (rc != TL_OK) return rc;
+    TL_CHECK_LAUNCH("gemm_dl_tile");
+    return TL_OK;
+}
+
+// The fused gate/up product (see tl_gemm_swiglu) on one named tile shape; for tests and tuning.
+extern "C" int tl_gemm_swiglu_direct_variant(const void* x, const void* w, void* out, int M, int I, int K, int ldx, int ldo,
+                                             int BM, int BN, hipStream_t stream) {
+    TL_REQUIRE(M > 0 && I > 0 && K % 64 == 0 && ldx % 8 == 0 && ldo >= I && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
+               "gemm_swiglu_direct: needs M > 0, K a multiple of 64 and 16-byte aligned rows");
+    int tile = -1;
+    for (int t = 0; t < DL_TILES; ++t)
+        if (DL_BM[t] == BM && DL_BN[t] == BN && t != DL_128x128_S4 && t != DL_64x64 && t != DL_256x192) tile = t;
+    TL_REQUIRE(tile >= 0, "gemm_swiglu_direct: no tile of %d x %d with the fused gate", BM, BN);
+    const int N = ((I + 31) / 32) * 64;
+    const int rc = launch_dl_tile<bf16_t, true>((DlTile)tile, x, w, nullptr, 0, out, M, N, K, ldx, ldo, I, stream);
     if (rc != TL_OK) return rc;
     TL_CHECK_LAUNCH("gemm_dl_tile");
     return TL_OK;

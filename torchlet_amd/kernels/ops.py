@@ -229,7 +229,7 @@ def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int, sla
                                          c_int(1 if out.dtype == torch.float32 else 0), c_int(tile_m), c_int(tile_n), c_int(slab), _stream()))
 
 
-DIRECT_TILES = ((64, 64), (64, 128), (64, 256), (128, 128), (128, 256), (256, 128), (192, 256), (256, 192), (256, 256))
+DIRECT_TILES = ((64, 64), (64, 128), (64, 192), (64, 256), (128, 128), (128, 192), (128, 256), (256, 128), (192, 256), (256, 192), (256, 256))
 
 
 def linear_direct_variant(x, weight, bias, out, tile_m: int, tile_n: int) -> None:
@@ -286,6 +286,19 @@ def linear_swiglu(x: torch.Tensor, gate_up: torch.Tensor, out: torch.Tensor) -> 
     lib = _lib("gemm")
     _check(lib, lib.tl_gemm_swiglu(_ptr(x), _ptr(gate_up), _ptr(out), c_int(M), c_int(I), c_int(K),
                                    c_int(x.stride(0)), c_int(out.stride(0)), _stream()))
+
+
+def linear_swiglu_direct_variant(x: torch.Tensor, gate_up: torch.Tensor, out: torch.Tensor, tile_m: int, tile_n: int) -> None:
+    """:func:`linear_swiglu` on one named tile shape of the kernel that fetches its operands straight into shared
+    memory (K a multiple of 64; for tests and tuning)."""
+    M, K = x.shape
+    I = out.shape[1]
+    if x.dtype != torch.bfloat16 or gate_up.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 \
+            or gate_up.shape != (-(-I // 32) * 64, K) or out.shape[0] != M or not gate_up.is_contiguous() or x.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("linear_swiglu_direct_variant: bfloat16 operands and fitting shapes only")
+    lib = _lib("gemm")
+    _check(lib, lib.tl_gemm_swiglu_direct_variant(_ptr(x), _ptr(gate_up), _ptr(out), c_int(M), c_int(I), c_int(K),
+                                                  c_int(x.stride(0)), c_int(out.stride(0)), c_int(tile_m), c_int(tile_n), _stream()))
 
 
 def rope_cache_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int, rot_heads: int,

@@ -1382,6 +1382,9 @@ static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = null
         if (sw && (t == DL_64x64 || t == DL_256x192)) continue;      // a wave of the fused gate needs whole 64-row blocks of weights
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
         if (t == DL_128x128_S4 && (tiles > 256 || M > 128)) continue;      // one round of work-groups, every weight drawn once
+        // (the split planner's unsplit baseline is fitted without the 192-wide tiles: with them it kept 512 rows against the
+        // 14B's query/key/value matrix whole, 74.8 us, where it used to split K, 53.9 us)
+        if (weights_only && (t == DL_64x192 || t == DL_128x192)) continue;
         const double est = dl_estimate((DlTile)t, tiles, K, weights_only);
         if (est < best_t) { best_t = est; best = (DlTile)t; }
     }

@@ -271,3 +271,18 @@ def test_toy_attention_that_differs_in_one_stage_on_the_host(cpu_ops):
 def test_toy_mixer_whose_cache_planes_differ_on_the_host(cpu_ops):
     import toy_parts
     toy_parts.run_toy_latent(torch.float32, torch.device("cpu"))
+
+
+def test_parts_of_the_keys_for_prompt_portions():
+    """How the attention mixer deals the keys of 128-row tiles to work-groups: few tiles are split to fill the
+    compute units; many tiles of equal length are split when that evens out the rounds of 512 work-groups."""
+    from torchlet_amd.parts.attention import _prompt_splits
+    assert _prompt_splits(160, 16384, uniform=True) == 4 and _prompt_splits(160, 16384, uniform=False) == 4
+    assert _prompt_splits(160, 1100, uniform=True) == 2               # parts of at least 512 keys
+    assert _prompt_splits(448, 2048, uniform=False) == 1              # a whole prompt: one round
+    assert _prompt_splits(640, 16384, uniform=False) == 1             # tiles of a causal prompt differ in length: no rounds to even out
+    assert _prompt_splits(640, 16384, uniform=True) == 4              # two rounds whole, five quarter rounds in four parts
+    assert _prompt_splits(640, 1200, uniform=True) == 2
+    assert _prompt_splits(1024, 16384, uniform=True) == 1             # two full rounds already
+    assert _prompt_splits(1280, 16384, uniform=True) == 2             # 2.5 rounds: three whole, five half rounds in two parts
+    assert _prompt_splits(512, 16384, uniform=True) == 1

@@ -154,14 +154,17 @@ def test_decode_attention_split_many_ways(ops, dtype, general, nh, nkv, hd, page
             _check_rows(got, ref, cache.v[r], f"request {r} of {totals[r]} keys, {splits} splits")
 
 
-@pytest.mark.parametrize("nh,nkv,hd,page,window,new,ctx", [
-    (28, 4, 128, 16, 0, 2048, 0),           # the benchmark's prefill
-    (40, 8, 128, 16, 0, 4096, 0),
-    (28, 4, 128, 16, 0, 512, 15872),        # a portion deep into a prompt: few tiles, each split over its keys
-    (40, 8, 128, 8, 0, 512, 15872),         # 2048 pages: the most the kernel keeps in shared memory
-    (12, 4, 64, 16, 3000, 700, 4000),       # heads of 64, a window
+@pytest.mark.parametrize("nh,nkv,hd,page,window,new,ctx,parts", [
+    (28, 4, 128, 16, 0, 2048, 0, 1),           # the benchmark's prefill
+    (40, 8, 128, 16, 0, 4096, 0, 1),
+    (28, 4, 128, 16, 0, 512, 15872, 4),        # a portion deep into a prompt: few tiles, each split over its keys
+    (40, 8, 128, 8, 0, 512, 15872, 4),         # 2048 pages: the most the kernel keeps in shared memory
+    (12, 4, 64, 16, 3000, 700, 4000, 4),       # heads of 64, a window
+    (40, 8, 128, 16, 0, 2048, 6144, 3),        # 656 tiles of about equal length: two rounds of work-groups whole, four thirds in three parts
+    (28, 4, 128, 16, 0, 2048, 6144, 1),        # 456 tiles: one round
 ])
-def test_prompt_attention_at_benchmark_lengths(ops, nh, nkv, hd, page, window, new, ctx):
+def test_prompt_attention_at_benchmark_lengths(ops, nh, nkv, hd, page, window, new, ctx, parts):
+    from torchlet_amd.parts.attention import _prompt_splits
     total = ctx + new
     cache = _Paged([total], nkv, hd, page, seed=new + ctx)
     g = torch.Generator(device="cuda").manual_seed(9)
@@ -170,9 +173,9 @@ def test_prompt_attention_at_benchmark_lengths(ops, nh, nkv, hd, page, window, n
     tok0 = list(range(0, new, tq))
     tiles = len(tok0)
     groups = tiles * nkv
-    splits = 1 if groups > 256 else max(1, min(4, 1024 // groups, total // 512))     # as the attention mixer decides
+    splits = _prompt_splits(groups, total if not window else min(total, window + tq), uniform=total >= 2 * new)   # as the attention mixer decides
     print(f"{new} new tokens on {ctx}: {tiles} tiles, {splits} splits", flush=True)
-    assert (splits > 1) == (ctx > 0)
+    assert splits == parts
     out = torch.full((new, nh * hd), float("nan"), dtype=torch.bfloat16, device="cuda")
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
     extra = dict(max_total_len=total, splits=splits)

@@ -30,7 +30,24 @@ _PROMPT_TARGET_WORKGROUPS = 1024  # the 128-row kernel: two work-groups fit a co
 _PROMPT_SPLIT_BELOW = 256        # ... but only steps whose tiles alone cannot give every compute unit one (a whole prompt of
                                  # 2048 tokens has 456: split in two it took 85 + 19 us of merge against 90 us)
 _PROMPT_MIN_KEYS_PER_SPLIT = 512
+_PROMPT_ROUND = 512                 # work-groups of the 128-row kernel that run at once
 _PROMPT_MAX_SPLITS = 4
+
+
+def _prompt_splits(groups: int, keys: int, uniform: bool) -> int:
+    """Into how many parts the 128-row kernel deals the keys of every tile: ``groups`` work-groups without a split,
+    ``keys`` the longest sequence; ``uniform``: every tile sees about as many keys (portions deep into their
+    prompts), so the work-groups come in rounds of equal length."""
+    most = max(1, min(_PROMPT_MAX_SPLITS, keys // _PROMPT_MIN_KEYS_PER_SPLIT))
+    if groups <= _PROMPT_SPLIT_BELOW:
+        return max(1, min(most, _PROMPT_TARGET_WORKGROUPS // max(groups, 1)))
+    if not uniform or groups <= _PROMPT_ROUND:
+        return 1
+    # rounds of 512 work-groups (two to a compute unit), the last one as long as the others however few are in it:
+    # 640 tiles of a 2048-token step of 40 heads take two rounds whole and five quarter rounds in four parts
+    # (measured at 32B sizes, 2048 tokens after 0 to 14336 cached ones: 545 -> 442 us a layer, and 24 us of merge)
+    cost = lambda n: -(-groups * n // _PROMPT_ROUND) / n * (1.0 if n == 1 else 1.08)
+    return min(range(1, most + 1), key=cost)
 
 
 @MIXERS.register("gqa_attention")
@@ -206,8 +223,7 @@ class GQAttention(Mixer):
                 # each tile's keys are dealt to several work-groups, so that the compute units have work
                 groups = long[2] * self.kv_heads * -(-(self.heads // self.kv_heads) // ops.PROMPT_ATTENTION_ROWS)
                 keys = ctx.max_total_len if self.window is None else min(ctx.max_total_len, self.window + tq)
-                splits = 1 if groups > _PROMPT_SPLIT_BELOW else \
-                    max(1, min(_PROMPT_MAX_SPLITS, _PROMPT_TARGET_WORKGROUPS // max(groups, 1), keys // _PROMPT_MIN_KEYS_PER_SPLIT))
+                splits = _prompt_splits(groups, keys, uniform=long[5] >= 2 * ctx.max_new_tokens)
                 extra = dict(max_total_len=ctx.max_total_len, splits=splits, merge_tokens=(long[3], long[4]))
             kernel(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens, long[0], long[1], long[2], tq, *common, **extra)
             if short[2]:     # split over their keys; the merge of the parts is kept to the rows of these requests

@@ -378,7 +378,7 @@ constexpr int skinny_depth() {
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + expf(-g)) * u; }
 
 // SW (gate/up product with the SwiGLU gate applied to the accumulators): w holds blocks of 64
-// rows, 32 gate rows followed by the 32 up rows of the same columns; a work-group's strip is 16
+// rows, 32 gate rows followed by the 32 up rows of the same columns; a work-group's strip is up to 16
 // outputs, whose gate rows half of its waves walk and whose up rows the other half (R == 1: each
 // wave streams one strip of 16 rows, which is what reaches the memory's rate; four strips per
 // wave, as an earlier version had, stayed at 56-58 us on the 7B's matrix where this takes 50-53);
@@ -845,8 +845,8 @@ static void launch_skinny(const void* x, const void* w, const void* bias, int bi
 
 // Rows a strip gets so that a matrix of N rows is dealt to the compute units in equal shares, one strip to
 // each (0: the plain strips of 16 R rows are as good; *blocks: how many blocks of 16 rows a strip then has, 1 or
-// 2).  A compute unit draws its weights at a rate of its own, about 26 GB/s whatever shares it with, so a product
-// takes as long as its busiest unit: at 3584 columns 256 strips of 16 rows take 7.9 us, 257 take 11.2, 288 (the
+// 2).  A compute unit draws its weights at a rate of its own, about 26 GB/s whatever shares it with, and the strips
+// beyond one per unit run when the others are done, nearly alone, at the latency of every fetch: at 3584 columns 256 strips of 16 rows take 7.9 us, 257 take 11.2, 288 (the
 // 7B's query/key/value matrix) 11.9 and 512 take 13.4.  The number is even (the fused rotation turns pairs).
 #define TL_COMPUTE_UNITS 256
 static int balanced_rows(int N, int* blocks) {

@@ -1402,13 +1402,16 @@ static DlSplit plan_dl_split(int M, int N, int K) {
     DlSplit best{pick_dl_tile(M, N, K, false, &best_t, true), 1, 0};
     best_t += (double)M * N * 2 * 2 / 3e12;
     const int steps = K / 64;
-    static const DlTile alone[] = {DL_128x128_S4, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256};
+    static const DlTile alone[] = {DL_128x128_S4, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_64x64};
     for (DlTile t : alone) {
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
         for (int P = 2; P <= 8 && K / P >= 512; ++P) {
             const int k_per = ((steps + P - 1) / P) * 64;
             if ((K + k_per - 1) / k_per != P) continue;
             if (t == DL_128x128_S4 && tiles * P > 256) continue;       // measured in one round of work-groups only
+            // (the small tile as for up to 64 rows, one work-group to a compute unit: 128 rows against the 7B's output
+            // projection 13.0 us in two parts where four parts of 128 x 128 take 17.0)
+            if (t == DL_64x64 && (M > 128 || tiles * P > 256)) continue;
             // (a tenth on top: float slabs leave the kernel more slowly than the estimate's bfloat16 rows)
             const double est = 1.1 * dl_estimate(t, tiles * P, k_per, true) + (double)P * M * N * 4 * 2 / 3e12;
             if (est < best_t) { best_t = est; best = DlSplit{t, P, k_per}; }

@@ -225,8 +225,8 @@ def load_folder(folder: str | Path, dtype: torch.dtype = torch.float64):
 
 
 def forward(cfg: PlainConfig, weights: dict[str, torch.Tensor], token_ids: list[int], first_position: int = 0,
-            stored=lambda t: t) -> torch.Tensor:
-    """Logits ``[T, vocab]`` of one whole request.
+            stored=lambda t: t, last: int | None = None) -> torch.Tensor:
+    """Logits ``[T, vocab]`` of one whole request (``last``: of its last that many positions only).
 
     embedding, ``layers`` blocks, final norm, LM head without bias (the embedding
     matrix itself when tied).  Reference: v00_full_recompute/model/qwen2_5.py:55-82.
@@ -238,6 +238,8 @@ def forward(cfg: PlainConfig, weights: dict[str, torch.Tensor], token_ids: list[
     x = weights["model.embed_tokens.weight"][ids]
     for i in range(cfg.layers):
         x = block(x, _sub(weights, f"model.layers.{i}."), cfg, i, positions, stored)
+    if last is not None:
+        x = x[-last:]
     x = stored(rms_norm(x, weights["model.norm.weight"], cfg.eps))
     head = weights["model.embed_tokens.weight"] if cfg.tied else weights["lm_head.weight"]
     return linear(x, head)

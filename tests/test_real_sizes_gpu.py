@@ -106,3 +106,63 @@ def test_every_split_at_checkpoint_widths(sized, dtype):
             assert err <= 1.25 * rms16, f"{name} {mode}: rms error {err:.3e}, bfloat16 roundings alone give {rms16:.3e}"
     del model
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", ["7B", "14B"])
+def test_the_benchmarks_own_steps_at_checkpoint_widths(shape, dtype):
+    """What the benchmark times, with its logits looked at: the widths of the 7B checkpoint (two layers, the whole
+    vocabulary; and of the 14B one, 40 heads in 8 groups, one layer), 8 requests with 2048-token prompts, each prefilled whole in one step (the 128-row prompt kernel
+    over 456 tiles, the large tiles of the products), then four decode steps of all 8 as replayed graphs (keys in
+    16 parts and their merge, the few-rows products with rotation and cache write in their epilogue, products
+    split over K whose slabs the norms add up).  Every logit row against the plain implementation in 64-bit,
+    with the bounds derived from the plain implementation as above."""
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import build_model, make_runner
+    from torchlet_amd.registry import ARCHITECTURES
+    from torchlet_amd.weights.random_init import random_tensors
+    prompt, new, batch = 2048, 4, 8
+    d = dict(COMMON, **SHAPES[shape])
+    config = ARCHITECTURES["Qwen2ForCausalLM"].from_dict(d)
+    tensors = random_tensors(config, seed=21, dtype=torch.bfloat16, device="cuda")
+    requests = scenarios.make_requests(d["vocab_size"], [prompt + new] * batch, seed=9)
+    cfg = plain.PlainConfig(d)
+    rows = new + 1                       # the prompt's last position and the four decoded ones
+    w64 = {k: v.double() for k, v in tensors.items()}
+    expected = {r: plain.forward(cfg, w64, t, last=rows).cpu() for r, t in requests.items()}
+    rounded = lambda t: t.to(torch.bfloat16).double()
+    moved = torch.stack([plain.forward(cfg, w64, t, stored=rounded, last=rows).cpu() - expected[r] for r, t in requests.items()])
+    del w64
+    w32 = {k: v.float() for k, v in tensors.items()}
+    noise = max(float((plain.forward(cfg, w32, t, last=rows).cpu().double() - expected[r]).abs().max()) for r, t in requests.items())
+    del w32
+    torch.cuda.empty_cache()
+    noise16, rms16 = float(moved.abs().max()), float(moved.pow(2).mean().sqrt())
+    rms = float(torch.stack(list(expected.values())).pow(2).mean().sqrt())
+    print(f"32-bit noise {noise:.3e}, bfloat16 roundings move the logits by {noise16:.3e} at most, {rms16:.3e} rms, logits {rms:.3e} rms", flush=True)
+    assert 0 < noise < 1e-3 * rms and noise16 < 0.1 * rms
+    tol = dict(atol=NOISE_FACTOR * noise, rtol=2e-5) if dtype == "float32" else dict(atol=2 * noise16, rtol=0.0)
+
+    model = build_model(config, dtype, tensors=tensors)
+    del tensors
+    runner = make_runner(model, page_size=PAGE, num_pages=batch * (-(-(prompt + new) // PAGE)) + 1, max_requests=batch, use_graphs=True)
+    errors = []
+
+    def compare(logits, place, row_of):
+        got = logits.double().cpu()
+        for i, r in enumerate(requests):
+            ref = expected[r][row_of]
+            if not torch.allclose(got[i], ref, **tol):
+                raise AssertionError(f"{shape} {dtype}: request {r} {place}: max abs error {float((got[i] - ref).abs().max()):.3e}, allowed {tol['atol']:.3e}")
+            errors.append(got[i] - ref)
+
+    first = [runner.step([StepEntry(r, t[:prompt], [prompt - 1])]) for r, t in requests.items()]
+    compare(torch.cat(first), "after its prompt", 0)
+    for n in range(new):
+        logits = runner.step([StepEntry(r, [t[prompt + n]], [0]) for r, t in requests.items()])
+        compare(logits, f"decode step {n}", 1 + n)
+    assert runner.graph_replays >= new - 1        # (the first of them may be the run that captures the graph)
+    if dtype == "bfloat16":
+        err = float(torch.stack(errors).pow(2).mean().sqrt())
+        print(f"    rms error {err:.3e}", flush=True)
+        assert err <= 1.25 * rms16, f"rms error {err:.3e}, bfloat16 roundings alone give {rms16:.3e}"

@@ -109,32 +109,35 @@ def test_every_split_at_checkpoint_widths(sized, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", ["7B", "14B"])
-def test_the_benchmarks_own_steps_at_checkpoint_widths(shape, dtype):
+@pytest.mark.parametrize("shape,batch", [("7B", 8), ("14B", 8), ("7B", 1), ("7B", 64)])
+def test_the_benchmarks_own_steps_at_checkpoint_widths(shape, batch, dtype):
     """What the benchmark times, with its logits looked at: the widths of the 7B checkpoint (two layers, the whole
     vocabulary; and of the 14B one, 40 heads in 8 groups, one layer), 8 requests with 2048-token prompts, each prefilled whole in one step (the 128-row prompt kernel
     over 456 tiles, the large tiles of the products), then four decode steps of all 8 as replayed graphs (keys in
     16 parts and their merge, the few-rows products with rotation and cache write in their epilogue, products
-    split over K whose slabs the norms add up).  Every logit row against the plain implementation in 64-bit,
-    with the bounds derived from the plain implementation as above."""
+    split over K whose slabs the norms add up); and the benchmark's other two points, one request (norms made
+    inside the kernels that read them) and 64 (the tile kernels of 17 rows up, the rotation kernel that adds up
+    the projection's slabs).  Every logit row of up to 8 of the requests against the plain implementation in
+    64-bit, with the bounds derived from the plain implementation as above."""
     from torchlet_amd.engine.batch import StepEntry
     from torchlet_amd.engine.loading import build_model, make_runner
     from torchlet_amd.registry import ARCHITECTURES
     from torchlet_amd.weights.random_init import random_tensors
-    prompt, new, batch = 2048, 4, 8
+    prompt, new = 2048, 4
     d = dict(COMMON, **SHAPES[shape])
     config = ARCHITECTURES["Qwen2ForCausalLM"].from_dict(d)
     tensors = random_tensors(config, seed=21, dtype=torch.bfloat16, device="cuda")
     requests = scenarios.make_requests(d["vocab_size"], [prompt + new] * batch, seed=9)
     cfg = plain.PlainConfig(d)
     rows = new + 1                       # the prompt's last position and the four decoded ones
+    checked = {r: requests[r] for r in list(requests)[:: max(1, batch // 8)]}
     w64 = {k: v.double() for k, v in tensors.items()}
-    expected = {r: plain.forward(cfg, w64, t, last=rows).cpu() for r, t in requests.items()}
+    expected = {r: plain.forward(cfg, w64, t, last=rows).cpu() for r, t in checked.items()}
     rounded = lambda t: t.to(torch.bfloat16).double()
-    moved = torch.stack([plain.forward(cfg, w64, t, stored=rounded, last=rows).cpu() - expected[r] for r, t in requests.items()])
+    moved = torch.stack([plain.forward(cfg, w64, t, stored=rounded, last=rows).cpu() - expected[r] for r, t in checked.items()])
     del w64
     w32 = {k: v.float() for k, v in tensors.items()}
-    noise = max(float((plain.forward(cfg, w32, t, last=rows).cpu().double() - expected[r]).abs().max()) for r, t in requests.items())
+    noise = max(float((plain.forward(cfg, w32, t, last=rows).cpu().double() - expected[r]).abs().max()) for r, t in checked.items())
     del w32
     torch.cuda.empty_cache()
     noise16, rms16 = float(moved.abs().max()), float(moved.pow(2).mean().sqrt())
@@ -151,6 +154,8 @@ def test_the_benchmarks_own_steps_at_checkpoint_widths(shape, dtype):
     def compare(logits, place, row_of):
         got = logits.double().cpu()
         for i, r in enumerate(requests):
+            if r not in expected:
+                continue
             ref = expected[r][row_of]
             if not torch.allclose(got[i], ref, **tol):
                 raise AssertionError(f"{shape} {dtype}: request {r} {place}: max abs error {float((got[i] - ref).abs().max()):.3e}, allowed {tol['atol']:.3e}")

@@ -81,7 +81,7 @@ def rope_cache_write(qkv, q_heads, kv_heads, head_dim, rot_heads, positions, inv
 
 
 def paged_attention(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles,
-                    tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale, splits=1, general=False, merge_tokens=None):
+                    tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale, splits=1, general=False, merge_tokens=None, waves=4):
     _attend(q, out, k_plane, v_plane, block_table, req_indptr, ctx_lens, tile_req, tile_tok0, num_tiles,
             tile_tokens, num_heads, num_kv_heads, head_dim, page_size, window, scale)
 

@@ -616,14 +616,14 @@ def _attention_ref(q, k, v, window):
     return torch.einsum("hnt,thd->nhd", torch.softmax(s, -1), vv)
 
 
-@pytest.mark.parametrize("dtype,general", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+@pytest.mark.parametrize("dtype,general,waves", [(torch.float32, False, 4), (torch.bfloat16, False, 4), (torch.bfloat16, False, 8), (torch.bfloat16, True, 4)])
 @pytest.mark.parametrize("nh,nkv,hd,page,window,splits", [
     (4, 2, 16, 16, 0, 1), (3, 1, 32, 8, 0, 1), (28, 4, 128, 16, 0, 3), (6, 6, 48, 4, 0, 1),
     (20, 1, 64, 16, 0, 2), (4, 2, 16, 16, 13, 1), (8, 2, 80, 32, 29, 4), (2, 1, 256, 16, 0, 1),
     (5, 5, 32, 2, 0, 2), (14, 2, 128, 64, 40, 5),
     (4, 2, 4, 4, 0, 1), (10, 2, 24, 16, 0, 3), (3, 3, 250, 8, 17, 2), (5, 1, 40, 16, 0, 2), (2, 1, 2, 16, 0, 1),
 ])
-def test_paged_attention(ops, dtype, general, nh, nkv, hd, page, window, splits):
+def test_paged_attention(ops, dtype, general, waves, nh, nkv, hd, page, window, splits):
     """float32 and bfloat16 through the general kernel, bfloat16 through the matrix-core kernel
     (pages of 2 tokens fall back to the general one by themselves, and so do head sizes that are
     no multiple of 16: the library of the next multiple serves them)."""
@@ -662,7 +662,7 @@ def test_paged_attention(ops, dtype, general, nh, nkv, hd, page, window, splits)
     ops.paged_attention(wide[:, : nh * hd], out, kp.cuda(), vp.cuda(), bt.cuda(), indptr.cuda(),
                         torch.tensor(ctxs, dtype=torch.int32).cuda(), torch.tensor(tile_req, dtype=torch.int32).cuda(),
                         torch.tensor(tile_tok0, dtype=torch.int32).cuda(), len(tile_req), tq, nh, nkv, hd, page, window,
-                        1.0 / math.sqrt(hd), splits, general=general)
+                        1.0 / math.sqrt(hd), splits, general=general, waves=waves)
     got = out.cpu().double().view(T, nh, hd)
     for r in range(R):
         a, b = int(indptr[r]), int(indptr[r + 1])

@@ -112,19 +112,21 @@ def test_decode_attention_at_benchmark_contexts_with_the_mixers_own_split_count(
     g = torch.Generator(device="cuda").manual_seed(3)
     q = torch.randn((batch, nh * hd), generator=g, device="cuda").to(torch.bfloat16)
     ctx_lens = torch.tensor([t - 1 for t in totals], dtype=torch.int32, device="cuda")
-    splits = _mixer_splits(nh, nkv, hd, 0, max(totals), batch)
-    print(f"heads {nh}/{nkv}, batch {batch}: {splits} splits, longest {max(totals)}", flush=True)
-    assert splits == {1: 64, 8: 16 if nkv == 4 else 8, 64: 2 if nkv == 4 else 1}[batch]
+    splits, waves = _mixer_splits(nh, nkv, hd, 0, max(totals), batch)
+    print(f"heads {nh}/{nkv}, batch {batch}: {splits} splits, {waves} waves, longest {max(totals)}", flush=True)
+    # work-groups of eight waves, one to a compute unit, while one per request and head group would leave units idle;
+    # 64 requests with 8 groups of heads fill them twice with work-groups of four
+    assert (splits, waves) == {1: (64, 8) if nkv == 4 else (32, 8), 8: (8, 8) if nkv == 4 else (4, 8), 64: (1, 8) if nkv == 4 else (1, 4)}[batch]
     out = torch.full((batch, nh * hd), float("nan"), dtype=torch.bfloat16, device="cuda")
     tq = ops.attention_tile_tokens(nh, nkv)
     ops.paged_attention(q, out, cache.kp, cache.vp, cache.table, None, ctx_lens, None, None, batch, tq,
-                        nh, nkv, hd, page, 0, 1.0 / math.sqrt(hd), splits)
+                        nh, nkv, hd, page, 0, 1.0 / math.sqrt(hd), splits, waves=waves)
     for r in range(batch):
         ref = _reference(q[r: r + 1].view(1, nh, hd), cache.k[r], cache.v[r], 0)
         _check_rows(out[r].double().view(1, nh, hd), ref, cache.v[r], f"request {r} of {totals[r]} keys")
 
 
-@pytest.mark.parametrize("dtype,general", [(torch.bfloat16, False), (torch.float32, False)])
+@pytest.mark.parametrize("dtype,general,waves", [(torch.bfloat16, False, 4), (torch.bfloat16, False, 8), (torch.float32, False, 4)])
 @pytest.mark.parametrize("nh,nkv,hd,page,window,splits,totals,width", [
     (28, 4, 128, 16, 0, 8, [2500, 4999, 3000], 0),
     (28, 4, 128, 16, 0, 9, [2500, 4999, 3000], 0),          # the merge's second pass over the parts
@@ -133,7 +135,7 @@ def test_decode_attention_at_benchmark_contexts_with_the_mixers_own_split_count(
     (6, 2, 128, 16, 3000, 12, [4999, 3001, 2999], 0),       # a window that cuts into the long ones
     (28, 4, 128, 16, 0, 33, [40000, 33000], 0),             # 2500 pages in use
 ])
-def test_decode_attention_split_many_ways(ops, dtype, general, nh, nkv, hd, page, window, splits, totals, width):
+def test_decode_attention_split_many_ways(ops, dtype, general, waves, nh, nkv, hd, page, window, splits, totals, width):
     if dtype == torch.float32 and max(totals) > 5000:
         totals = [t // 8 + 2048 for t in totals]             # the 32-bit kernel is slow; its tables stay narrow
     cache = _Paged(totals, nkv, hd, page, seed=splits, table_width=width, dtype=dtype)
@@ -144,7 +146,7 @@ def test_decode_attention_split_many_ways(ops, dtype, general, nh, nkv, hd, page
     out = torch.full((R, nh * hd), float("nan"), dtype=dtype, device="cuda")
     tq = ops.attention_tile_tokens(nh, nkv)
     ops.paged_attention(q, out, cache.kp, cache.vp, cache.table, None, ctx_lens, None, None, R, tq,
-                        nh, nkv, hd, page, window, 1.0 / math.sqrt(hd), splits, general=general)
+                        nh, nkv, hd, page, window, 1.0 / math.sqrt(hd), splits, general=general, waves=waves)
     for r in range(R):
         ref = _reference(q[r: r + 1].view(1, nh, hd), cache.k[r], cache.v[r], window)
         got = out[r].double().view(1, nh, hd)

@@ -235,8 +235,12 @@ __global__ __launch_bounds__(256) void paged_attention_kernel(AttnArgs a) {
 // 4g..4g+3 of the second}, for A and B alike, which is why no shuffle or shared memory is
 // needed.  The online softmax works in base 2 on scores pre-multiplied by scale * log2(e);
 // running maximum and sum are float, probabilities are rounded to bfloat16 for the product
-// with V.  The four waves of a work-group take the chunks of the tile's key range (or of its
-// split) in turn and merge their states pairwise through shared memory at the end.
+// with V.  The waves of a work-group (NW: four or eight) take the chunks of the tile's key range (or of its
+// split) in turn and merge their states pairwise through shared memory at the end.  Eight waves with half as
+// many parts per request are as many waves on as many keys, with half the partial results to write, read and
+// merge, or none (7B sizes, contexts of 2048: the decode step at batch 1 / 8 / 64 3.33 / 3.72 / 5.34 ->
+// 3.28 / 3.66 / 5.24 ms); where every request has a work-group of four to itself and the compute units are
+// full with those, four stay ahead (batch 128: 7.61 against 7.75 ms).
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
@@ -254,8 +258,9 @@ union FragK {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
-    __shared__ float park[2 * ATM_SLOT];
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void paged_attention_mfma_kernel(AttnArgs a) {
+    __shared__ float park[(NW / 2) * ATM_SLOT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, g = lane >> 4;
 
@@ -276,7 +281,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
     const int* bt_g = a.block_table + (size_t)req * a.bt_stride;
     const bool bt_whole = a.bt_stride <= ATM_BT_MAX;        // the whole row, before the length says which part is needed
     if (bt_whole)
-        for (int i = threadIdx.x; i < a.bt_stride; i += 256) bt_s[i] = bt_g[i];
+        for (int i = threadIdx.x; i < a.bt_stride; i += 64 * NW) bt_s[i] = bt_g[i];
     const int tok0 = one_each ? 0 : a.tile_tok0[tile];
     const int first = one_each ? req : a.req_indptr[req];
     const int n_new = one_each ? 1 : a.req_indptr[req + 1] - first;
@@ -320,7 +325,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
     const bool bt_local = bt_whole || blk_n <= ATM_BT_MAX;
     if (bt_local) {
         if (!bt_whole)
-            for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
+            for (int i = threadIdx.x; i < blk_n; i += 64 * NW) bt_s[i] = bt_g[blk0 + i];
         __syncthreads();
     }
 #define ATM_PAGE_OF(blk) (bt_local ? bt_s[(blk) - blk0] : bt_g[(blk)])
@@ -375,7 +380,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
 
     int ch = ch_begin + wave;
     if (ch < ch_end) ATM_FETCH(kf, vfa, vfb, ch)
-    for (; ch < ch_end; ch += 4) {
+    for (; ch < ch_end; ch += NW) {
         const int kbase = ch * 32;
         // ---- scores: two halves of 16 keys
         f32x4_t sc[2];
@@ -437,26 +442,24 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(AttnArgs a) {
             if (moved) acc[t] *= alpha;
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[t], 0, 0, 0);
         }
-        if (ch + 4 < ch_end) ATM_FETCH(kf, vfa, vfb, ch + 4)
+        if (ch + NW < ch_end) ATM_FETCH(kf, vfa, vfb, ch + NW)
     }
 #undef ATM_FETCH
 #undef ATM_PAGE_OF
 
-    // ---- merge the four waves: 2,3 -> 0,1, then 1 -> 0
+    // ---- merge the waves: the upper half of those left hands its state to the lower half, until one is left
 #pragma unroll
-    for (int round = 0; round < 2; ++round) {
-        const int senders_from = round == 0 ? 2 : 1;
-        const int senders_to = round == 0 ? 4 : 2;
+    for (int half = NW / 2; half >= 1; half >>= 1) {
         __syncthreads();
-        if (wave >= senders_from && wave < senders_to) {
-            float* dst = park + (size_t)(wave - senders_from) * ATM_SLOT;
+        if (wave >= half && wave < 2 * half) {
+            float* dst = park + (size_t)(wave - half) * ATM_SLOT;
 #pragma unroll
             for (int t = 0; t < ATM_DT; ++t) *(f32x4_t*)(dst + (t * 64 + lane) * 4) = acc[t];
             dst[ATM_DT * 256 + lane] = m;
             dst[ATM_DT * 256 + 64 + lane] = l;
         }
         __syncthreads();
-        if (wave < senders_from && wave + senders_from < senders_to) {
+        if (wave < half) {
             const float* src = park + (size_t)wave * ATM_SLOT;
             const float mo = src[ATM_DT * 256 + lane], lo = src[ATM_DT * 256 + 64 + lane];
             const float mm = fmaxf(m, mo);
@@ -1184,8 +1187,9 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
                                   const void* tile_req, const void* tile_tok0, int tiles, int tokens, int tq,
                                   int heads, int kv_heads, int head_dim, int page, int window, float scale, int splits,
                                   void* part_o, void* part_ml, const void* merge_tokens, int merge_count, int dtype, int general,
-                                  hipStream_t stream) {
+                                  int waves, hipStream_t stream) {
     TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
+    TL_REQUIRE(waves == 4 || waves == 8, "attention: work-groups of 4 or 8 waves, not %d", waves);
     TL_REQUIRE(head_dim > AT_HD - 16 && head_dim <= AT_HD && head_dim % 2 == 0,
                "attention: this library serves the even head sizes %d to %d, not %d", AT_HD - 14, AT_HD, head_dim);
     TL_REQUIRE(page > 0 && bt_stride > 0 && tq > 0 && splits > 0 && window >= 0, "attention: bad page/table/tile sizes");
@@ -1210,7 +1214,10 @@ extern "C" int tl_paged_attention(const void* q, int q_stride, void* out, const 
     const bool aligned = ((uintptr_t)q % 16) == 0 && q_stride % 8 == 0 && ((uintptr_t)out % 8) == 0 &&
                          ((uintptr_t)k_plane % 16) == 0 && ((uintptr_t)v_plane % 8) == 0;
     if (dtype == TL_DT_F32) paged_attention_kernel<float><<<grid, block, 0, stream>>>(a);
-    else if (dtype == TL_DT_BF16 && page % 4 == 0 && aligned && !general && head_dim == AT_HD) paged_attention_mfma_kernel<<<grid, block, 0, stream>>>(a);
+    else if (dtype == TL_DT_BF16 && page % 4 == 0 && aligned && !general && head_dim == AT_HD) {
+        if (waves == 8) paged_attention_mfma_kernel<8><<<grid, dim3(512), 0, stream>>>(a);
+        else paged_attention_mfma_kernel<4><<<grid, block, 0, stream>>>(a);
+    }
     else if (dtype == TL_DT_BF16) paged_attention_kernel<bf16_t><<<grid, block, 0, stream>>>(a);
     else TL_REQUIRE(false, "attention: unknown dtype %d", dtype);
     TL_CHECK_LAUNCH("paged_attention");

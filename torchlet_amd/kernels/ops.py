@@ -504,7 +504,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
                     block_table: torch.Tensor, req_indptr: torch.Tensor, ctx_lens: torch.Tensor,
                     tile_req: torch.Tensor, tile_tok0: torch.Tensor, num_tiles: int, tile_tokens: int,
                     num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
-                    scale: float, splits: int = 1, general: bool = False, merge_tokens=None) -> None:
+                    scale: float, splits: int = 1, general: bool = False, merge_tokens=None, waves: int = 4) -> None:
     """Causal attention of the step's tokens over their requests' cached keys.
 
     ``q [T, >= heads*hd]`` (row-strided view), ``out [T, heads*hd]``, ``k_plane [pages,
@@ -516,8 +516,11 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
     indices of those tokens, their number)`` keeps the merge of the parts to their rows.
     ``tile_req = tile_tok0 = None``: every request brings exactly one token, token ``i`` that of
     request ``i`` (a decode step); the kernel then looks nothing up before it asks for the
-    request's length, block table and query."""
+    request's length, block table and query.  ``waves``: 4 or 8 to a work-group of the matrix-core kernel
+    (they deal a part's keys among themselves; the other kernels take no notice)."""
     T = q.shape[0]
+    if waves not in (4, 8):
+        raise KernelError("paged_attention: work-groups of 4 or 8 waves")
     if q.stride(1) != 1 or out.shape != (T, num_heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
         raise KernelError("paged_attention: q/out shapes or dtypes do not fit")
     _check_planes("paged_attention", k_plane, v_plane, q.dtype, num_kv_heads, page_size, head_dim)
@@ -550,7 +553,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, k_plane: torch.Tensor, v
                                        c_float(scale), c_int(splits), _ptr(part_o), _ptr(part_ml),
                                        _ptr(merge_tokens[0]) if merge_tokens is not None else c_void_p(None),
                                        c_int(merge_tokens[1] if merge_tokens is not None else 0),
-                                       c_int(_dt(q, "paged_attention")), c_int(1 if general else 0), _stream()))
+                                       c_int(_dt(q, "paged_attention")), c_int(1 if general else 0), c_int(waves), _stream()))
 
 
 PREFILL_ATTENTION_ROWS = 64      # rows a work-group of the prompt-portion kernel owns

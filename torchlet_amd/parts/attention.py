@@ -19,7 +19,8 @@ from ..config.base import ConfigError
 from ..kernels import ops
 from .base import MIXERS, POSITION_ENCODINGS, LazyNorm, Mixer, PagedNeed, WeightSpec
 
-_TARGET_WORKGROUPS = 512     # enough work-groups to fill 256 compute units twice
+_COMPUTE_UNITS = 256
+_TARGET_WORKGROUPS = 512     # enough work-groups of four waves to fill 256 compute units twice
 _MIN_KEYS_PER_SPLIT = 256
 _PORTION_MIN_TOKENS = 16     # requests that bring at least this many tokens go to a prompt-portion kernel: the
                              # 128-row one where it is built (head size 64 or 128, pages of 8, 16, 32, ...
@@ -119,15 +120,19 @@ class GQAttention(Mixer):
         self.w_o = self._place(tensors["o_proj.weight"], "matrix")
 
     # -- the step -----------------------------------------------------------------
-    def _splits(self, ctx, tiles: int, longest: int | None = None) -> int:
+    def _splits(self, ctx, tiles: int, longest: int | None = None) -> tuple[int, int]:
+        """(parts of every request's keys, waves of a work-group) for the 16-row kernel: work-groups of eight waves
+        while one per tile and head group leaves compute units idle, with as many parts as give each unit one
+        work-group; from there on work-groups of four waves, two to a unit, and no parts beyond that."""
         group = self.heads // self.kv_heads
         chunks = -(-group // ops.ATTENTION_ROWS)
         base = max(1, tiles * self.kv_heads * chunks)
-        by_fill = -(-_TARGET_WORKGROUPS // base)
+        waves = 8 if base <= _COMPUTE_UNITS else 4
+        by_fill = -(-(_COMPUTE_UNITS if waves == 8 else _TARGET_WORKGROUPS) // base)
         longest = ctx.max_total_len if longest is None else longest
         longest = longest if self.window is None else min(longest, self.window + ctx.max_new_tokens)
         by_keys = max(1, longest // _MIN_KEYS_PER_SPLIT)
-        return max(1, min(by_fill, by_keys, 64))
+        return max(1, min(by_fill, by_keys, 64)), waves
 
     takes_lazy_norm = True
 
@@ -227,15 +232,17 @@ class GQAttention(Mixer):
                 extra = dict(max_total_len=ctx.max_total_len, splits=splits, merge_tokens=(long[3], long[4]))
             kernel(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens, long[0], long[1], long[2], tq, *common, **extra)
             if short[2]:     # split over their keys; the merge of the parts is kept to the rows of these requests
+                splits, waves = self._splits(ctx, short[2], short[5])
                 ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
                                     short[0], short[1], short[2], self.tile_tokens, *common,
-                                    self._splits(ctx, short[2], short[5]), merge_tokens=(short[3], short[4]))
+                                    splits, merge_tokens=(short[3], short[4]), waves=waves)
         else:
             tile_req, tile_tok0, tiles = ctx.tiles(self.tile_tokens)
             if ctx.decode_only and tiles == T:      # one token per request: no tile list to look up
                 tile_req = tile_tok0 = None
+            splits, waves = self._splits(ctx, tiles)
             ops.paged_attention(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens,
-                                tile_req, tile_tok0, tiles, self.tile_tokens, *common, self._splits(ctx, tiles))
+                                tile_req, tile_tok0, tiles, self.tile_tokens, *common, splits, waves=waves)
         return out
 
     def output(self, out):

@@ -239,3 +239,87 @@ def test_start_up_reports(tmp_path):
     assert stream.getvalue() == "" and log.level == logging.WARNING
     get_logger("torchlet_amd.test", level=logging.INFO).info("shown %d", 3)
     assert "[INFO] torchlet_amd.test" in stream.getvalue() and "shown 3" in stream.getvalue()
+
+
+def test_compute_dtype_follows_the_folder(tmp_path):
+    """The reference types its parameters and its cache after the checkpoint's tensors
+    (/root/reference/src/torchlet/utils.py:18-38, v10_triton_paged_gqa/engine.py:58): a folder stored in
+    32-bit runs in 32-bit.  Here the folder's ``torch_dtype`` decides, else what it stores; a named
+    dtype converts at load; anything but bfloat16 and float32 is refused by name."""
+    from torchlet_amd.engine.loading import load_model, resolve_dtype
+    cfg = Qwen2Config.from_dict(REF_TINY)
+    assert cfg.torch_dtype == "" and cfg.to_dict()["torch_dtype"] is None
+    f32 = write_model_folder(cfg, 0, tmp_path / "f32", torch.float32)
+    bf16 = write_model_folder(cfg, 0, tmp_path / "bf16", torch.bfloat16)
+    assert json.loads((f32 / "config.json").read_text())["torch_dtype"] == "float32"
+    assert resolve_dtype(f32, load_config(f32)) == "float32" and resolve_dtype(bf16, load_config(bf16)) == "bfloat16"
+    for folder in (f32, bf16):                       # without the key: the stored element type decides
+        d = json.loads((folder / "config.json").read_text())
+        del d["torch_dtype"]
+        (folder / "config.json").write_text(json.dumps(d))
+    assert resolve_dtype(f32, load_config(f32)) == "float32" and resolve_dtype(bf16, load_config(bf16)) == "bfloat16"
+    assert resolve_dtype(f32, load_config(f32), "bfloat16") == "bfloat16"       # named: converts at load
+    assert resolve_dtype(bf16, load_config(bf16), torch.float32) == "float32"
+    _, model = load_model(f32, device="cpu")
+    assert model.dtype == torch.float32 and model.embed.dtype == torch.float32 and model.blocks[0].mixer.w_qkv.dtype == torch.float32
+    _, model = load_model(bf16, device="cpu")
+    assert model.dtype == torch.bfloat16 and model.embed.dtype == torch.bfloat16
+    _, model = load_model(f32, "bfloat16", device="cpu")
+    assert model.dtype == torch.bfloat16 and model.blocks[0].ffn.down.dtype == torch.bfloat16
+    # a dtype for which no engine is built: refused by its name, from the key and from the stored tensors
+    d = json.loads((bf16 / "config.json").read_text())
+    (bf16 / "config.json").write_text(json.dumps(dict(d, torch_dtype="float16")))
+    with pytest.raises(ValueError, match="float16"):
+        load_model(bf16, device="cpu")
+    f16 = write_model_folder(cfg, 0, tmp_path / "f16", torch.float16)
+    d = json.loads((f16 / "config.json").read_text())
+    del d["torch_dtype"]
+    (f16 / "config.json").write_text(json.dumps(d))
+    with pytest.raises(ValueError, match="float16"):
+        load_model(f16, device="cpu")
+    assert load_model(f16, "float32", device="cpu")[1].dtype == torch.float32
+
+
+def test_dtype_policy_of_a_tensor_is_apart_from_its_shape_and_laws_are_named():
+    from torchlet_amd.parts.base import INIT_LAWS, WeightSpec, place, register_init_law
+    m = torch.randn(3, 5).to(torch.bfloat16)
+    assert place(m, "compute", torch.bfloat16, "cpu").dtype == torch.bfloat16
+    assert place(m, "float32", torch.bfloat16, "cpu").dtype == torch.float32            # a matrix that stays 32-bit
+    assert place(m.float(), "stored", torch.bfloat16, "cpu").dtype == torch.float32     # stored in 32-bit: stays
+    assert place(m, "stored", torch.float32, "cpu").dtype == torch.float32              # a 32-bit engine widens
+    assert place(m.half(), "stored", torch.bfloat16, "cpu").dtype == torch.float32      # neither of the two: widened
+    assert place(torch.arange(4), "int32", torch.bfloat16, "cpu").dtype == torch.int32
+    for bad in (dict(keep="vector"), dict(init="no_such_law")):
+        with pytest.raises(ConfigError):
+            WeightSpec((2, 2), **bad)
+    with pytest.raises(ConfigError):
+        place(m, "matrix", torch.bfloat16, "cpu")
+    register_init_law("test_all_sevens")(lambda shape, gen, device, std: torch.full(shape, 7.0, device=device))
+    try:
+        assert WeightSpec((2,), init="test_all_sevens").init == "test_all_sevens"
+        assert float(INIT_LAWS["test_all_sevens"]((2,), None, "cpu", 0.02).sum()) == 14.0
+    finally:
+        INIT_LAWS.pop("test_all_sevens")
+
+
+def test_every_part_is_asked_whether_a_step_may_be_recorded():
+    """Not the mixers alone: a feed-forward, a norm or a position encoding that reads values of the step on the host
+    keeps the whole model off graphs.  ``False`` is the default of a part; the built-in parts say ``True``."""
+    from torchlet_amd.parts import FEED_FORWARDS, FeedForward, Part
+    from torchlet_amd.parts.base import LazyNorm, Stream
+    assert Part.graph_safe is False
+    model = _model(REF_TINY)
+    kinds = {type(p).__name__ for p in model.parts()}
+    assert kinds == {"PreNormBlock", "RMSNorm", "GQAttention", "RotaryEncoding", "SwiGLU"} and model.graph_safe()
+
+    class HostReadingFFN(FeedForward):
+        def forward(self, h, ctx):
+            return h
+    model.blocks[0].ffn = model.blocks[0]._children["mlp"] = HostReadingFFN(None, torch.bfloat16, "cpu")
+    assert not model.graph_safe()
+    # a norm that has not run yet names its kind, and only a root-mean-square norm hands out (weight, eps)
+    norm = model.final_norm
+    norm.weight = torch.ones(16)
+    lazy = LazyNorm(norm, Stream(torch.zeros(1, 16)), "rmsnorm", weight=norm.weight, eps=norm.eps)
+    assert lazy.rmsnorm() == (norm.weight, norm.eps)
+    assert LazyNorm(norm, Stream(torch.zeros(1, 16)), "layernorm", weight=norm.weight, bias=None, eps=1e-5).rmsnorm() is None

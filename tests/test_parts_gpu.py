@@ -183,6 +183,7 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path, gr
     from torchlet_amd.engine.batch import StepEntry
     from torchlet_amd.engine.loading import build_model, make_runner
     from torchlet_amd.parts import MIXERS, Mixer, StateNeed, WeightSpec
+    from torchlet_amd.parts.base import INIT_LAWS, register_init_law
     from torchlet_amd.registry import config_class, register_architecture, unregister_architecture
     from torchlet_amd.weights.random_init import random_tensors
 
@@ -197,10 +198,10 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path, gr
         graph_safe = True
 
         def weight_specs(self):
-            return {"decay": WeightSpec((self.spec.hidden,), role="vector")}
+            return {"decay": WeightSpec((self.spec.hidden,), keep="float32", init="toy_decay_logit")}
 
         def load_weights(self, tensors):
-            self.decay = self._place(tensors["decay"], "vector")
+            self.decay = self._place(tensors["decay"], "float32")
 
         def state_need(self):
             return StateNeed((self.spec.hidden,), torch.float32)
@@ -238,11 +239,13 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path, gr
                              order=tuple(RunEntry(i) for i in range(self.num_hidden_layers)), final_norm=norm,
                              tie_head=True, max_positions=1 << 20)
 
+    # a law of the random-weights mode that the framework does not have, added by name from here
+    register_init_law("toy_decay_logit")(lambda shape, gen, device, std: torch.rand(shape, generator=gen, device=device) * 4 - 2)
     register_architecture(ToyConfig)
     try:
         cfg = config_class("ToyDecayForCausalLM").from_dict(dict(vocab_size=40, hidden_size=24, num_hidden_layers=2, intermediate_size=56))
         tensors = random_tensors(cfg, seed=9, dtype=torch.float32)
-        assert "model.layers.1.mix.decay" in tensors
+        assert "model.layers.1.mix.decay" in tensors and float(tensors["model.layers.1.mix.decay"].abs().max()) > 1.0   # U(-2, 2), not N(0, 0.02)
         model = build_model(cfg, "float32", tensors=tensors)
         runner = make_runner(model, page_size=16, num_pages=2, max_requests=3, use_graphs=graphs)
         assert runner.cache.groups == [] and runner.caches[0].state.shape == (4, 24) and runner.use_graphs == graphs
@@ -292,6 +295,7 @@ def test_toy_mixer_with_state_of_its_own_registers_builds_and_steps(tmp_path, gr
     finally:
         unregister_architecture("ToyDecayForCausalLM")
         MIXERS.unregister("toy_decay")
+        INIT_LAWS.pop("toy_decay_logit", None)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -36,14 +36,40 @@ def _both(lib, logits, temperature, keys):
     rc = lib.tl_sample(_ptr(logits), c_int(rows), c_int(vocab), c_int(logits.stride(0)), _ptr(temperature), _ptr(keys),
                        _ptr(want), _ptr(scratch), stream)
     assert rc == 0, lib.tl_last_error().decode()
-    torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
-    rc = lib.tl_sample_static(_ptr(logits), c_int(rows), c_int(vocab), c_int(logits.stride(0)), _ptr(temperature), _ptr(keys),
-                              _ptr(got), stream)
+    static = lambda: lib.tl_sample_static(_ptr(logits), c_int(rows), c_int(vocab), c_int(logits.stride(0)), _ptr(temperature),
+                                          _ptr(keys), _ptr(got), stream)
+    rc = static()           # (the first call on a device asks for the array's address and loads the kernels)
     assert rc == 0, lib.tl_last_error().decode()
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    # Free memory of the device itself, not the count of torch's allocator (which a hipMalloc inside the
+    # library would not move): with torch's allocator idle, a call must leave it where it was.
+    free_before, _ = torch.cuda.mem_get_info()
+    held_before = torch.cuda.memory_reserved()
+    got.fill_(-2)
+    torch.cuda.synchronize()
+    rc = static()
+    assert rc == 0, lib.tl_last_error().decode()
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_reserved() == held_before, "torch's own allocator moved: the measurement below would not be the library's"
+    assert torch.cuda.mem_get_info()[0] == free_before, "tl_sample_static changed the device's free memory"
     return want.tolist(), got.tolist()
+
+
+def test_the_measurement_of_free_device_memory_sees_an_allocation_that_torch_does_not_count():
+    """What the check above relies on: memory taken from the device behind torch's back (here through the HIP runtime
+    directly, as a ``hipMalloc`` inside the library would be) lowers ``mem_get_info`` and leaves torch's count alone."""
+    torch.cuda.synchronize()
+    # the HIP runtime this process already runs on (the copy torch loaded), not a second one
+    loaded = {line.split()[-1] for line in open("/proc/self/maps") if "libamdhip64" in line}
+    assert len(loaded) == 1, loaded
+    hip = ctypes.CDLL(loaded.pop())
+    free_before, counted = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
+    ptr = c_void_p()
+    assert hip.hipMalloc(ctypes.byref(ptr), ctypes.c_size_t(64 << 20)) == 0
+    try:
+        assert torch.cuda.mem_get_info()[0] <= free_before - (64 << 20) and torch.cuda.memory_allocated() == counted
+    finally:
+        assert hip.hipFree(ptr) == 0
 
 
 def test_sampling_without_allocation_matches_the_entry_point_with_scratch():

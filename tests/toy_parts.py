@@ -65,7 +65,7 @@ def run_toy_mix(dtype, device, tolerance):
 
         def weight_specs(self):
             s = self.spec
-            specs = {"router.weight": WeightSpec((s.experts, s.hidden), role="vector")}
+            specs = {"router.weight": WeightSpec((s.experts, s.hidden), keep="float32")}     # a matrix that stays 32-bit
             for e in range(s.experts):
                 specs[f"experts.{e}.gate.weight"] = WeightSpec((s.intermediate, s.hidden))
                 specs[f"experts.{e}.up.weight"] = WeightSpec((s.intermediate, s.hidden))
@@ -73,8 +73,8 @@ def run_toy_mix(dtype, device, tolerance):
             return specs
 
         def load_weights(self, tensors):
-            self.router = self._place(tensors["router.weight"], "vector").float()
-            self.w = {k: self._place(v, "matrix") for k, v in tensors.items() if k.startswith("experts.")}
+            self.router = self._place(tensors["router.weight"], "float32")
+            self.w = {k: self._place(v, "compute") for k, v in tensors.items() if k.startswith("experts.")}
 
         def forward(self, h, ctx):
             s = self.spec
@@ -177,6 +177,7 @@ def run_toy_mix(dtype, device, tolerance):
         assert "model.layers.1.moe.experts.2.down.weight" in tensors and "model.layers.1.moe.router.weight" in tensors
         assert tensors["lm_head.bias"].shape == (VOCAB,) and "lm_head.weight" not in tensors
         model = build_model(cfg, dtype, device=device, tensors=tensors)
+        assert model.blocks[1].ffn.router.dtype == torch.float32 and model.blocks[1].ffn.router.shape == (EXPERTS, H)   # a matrix kept in 32-bit
         runner = make_runner(model, page_size=8, num_pages=24, max_requests=2)
         assert len(runner.caches) == 3 and runner.caches[2].planes[0].data_ptr() == runner.caches[0].planes[0].data_ptr() and not runner.caches[2].writable
         # token sequences for which no token's choice of expert hangs on the last bits of a
@@ -200,6 +201,22 @@ def run_toy_mix(dtype, device, tolerance):
         got["b"].append(out[:6]); got["a"].append(out[6:])
         out = runner.step([StepEntry("a", seqs["a"][14:], list(range(27))), StepEntry("b", seqs["b"][6:], list(range(13)))]).cpu()
         got["a"].append(out[:27]); got["b"].append(out[27:])
+        # The router reads which tokens chose which expert on the host (`.nonzero()`): it does not say it is safe to
+        # record, neither does the toy position encoding, so the model is not, and a step function asked for graphs
+        # runs every step of this model eagerly (a recorded step would replay the shapes of the step it recorded).
+        assert not model.blocks[1].ffn.graph_safe and not model.blocks[0].mixer.position.graph_safe
+        assert model.blocks[0].ffn.graph_safe and model.blocks[1].mixer.position.graph_safe and not model.graph_safe()
+        for k in seqs:
+            runner.release(k)
+        eager = make_runner(model, page_size=8, num_pages=24, max_requests=2, use_graphs=True)
+        assert not eager.use_graphs and eager.warm_up() == 0
+        singles = {k: [] for k in seqs}
+        for i in range(len(seqs["a"])):               # both requests token by token: decode-only steps, the router's shapes change
+            live = [k for k in seqs if i < len(seqs[k])]
+            out = eager.step([StepEntry(k, [seqs[k][i]], [0]) for k in live]).cpu()
+            for j, k in enumerate(live):
+                singles[k].append(out[j: j + 1])
+        assert eager.graph_replays == 0 and not eager._graphs
         for k in seqs:
             tol = tolerance(dtype, refs[k])
             if dtype == torch.bfloat16:
@@ -209,6 +226,7 @@ def run_toy_mix(dtype, device, tolerance):
                 tol = dict(atol=2 * float(moved.abs().max()), rtol=0.0)
             torch.testing.assert_close(whole[k].double(), refs[k], **tol)
             torch.testing.assert_close(torch.cat(got[k]).double(), refs[k], **tol)
+            torch.testing.assert_close(torch.cat(singles[k]).double(), refs[k], **tol)
     finally:
         unregister_architecture("ToyMixForCausalLM")
         POSITION_ENCODINGS.unregister("toy_rope_pairs")
@@ -238,14 +256,14 @@ def run_toy_qk_norm(dtype, device, tolerance):
     class QKNormAttention(GQAttention):
         def weight_specs(self):
             specs = super().weight_specs()
-            specs["q_norm.weight"] = WeightSpec((self.head_dim,), role="vector", init="one_plus_normal")
-            specs["k_norm.weight"] = WeightSpec((self.head_dim,), role="vector", init="one_plus_normal")
+            specs["q_norm.weight"] = WeightSpec((self.head_dim,), keep="stored", init="one_plus_normal")
+            specs["k_norm.weight"] = WeightSpec((self.head_dim,), keep="stored", init="one_plus_normal")
             return specs
 
         def load_weights(self, tensors):
             super().load_weights(tensors)
-            self.q_norm = self._place(tensors["q_norm.weight"], "vector").float()
-            self.k_norm = self._place(tensors["k_norm.weight"], "vector").float()
+            self.q_norm = self._place(tensors["q_norm.weight"], "stored").float()
+            self.k_norm = self._place(tensors["k_norm.weight"], "stored").float()
 
         def transform_qk(self, q3, k3, ctx):
             for x, w in ((q3, self.q_norm), (k3, self.k_norm)):
@@ -349,8 +367,8 @@ def run_toy_latent(dtype, device):
             return {"down.weight": WeightSpec((LATENT, self.spec.hidden)), "up.weight": WeightSpec((self.spec.hidden, LATENT))}
 
         def load_weights(self, tensors):
-            self.down = self._place(tensors["down.weight"], "matrix")
-            self.up = self._place(tensors["up.weight"], "matrix")
+            self.down = self._place(tensors["down.weight"], "compute")
+            self.up = self._place(tensors["up.weight"], "compute")
 
         def paged_need(self):
             return PagedNeed(num_heads=1, head_dim=0, planes=((1, LATENT), (1, POS)), dtype=torch.float32)

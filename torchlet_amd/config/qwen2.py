@@ -50,7 +50,7 @@ class Qwen2Config(ModelConfig):
     use_sliding_window: bool = False
     sliding_window: int = 0               # 0: none given
     max_window_layers: int = -1           # -1: every layer attends to all keys
-    torch_dtype: str = "bfloat16"
+    torch_dtype: str = ""                 # "": the folder does not say; the engine then goes by what it stores
     bos_token_id: int = -1
     eos_token_id: int = -1
 
@@ -149,6 +149,8 @@ class Qwen2Config(ModelConfig):
         for key in ("bos_token_id", "eos_token_id"):
             if d[key] < 0:
                 d[key] = None
+        if not d["torch_dtype"]:
+            d["torch_dtype"] = None
         if not self.use_sliding_window and self.sliding_window == 0:
             d["sliding_window"] = None
         return d

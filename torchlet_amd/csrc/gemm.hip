@@ -9,6 +9,14 @@
 // output element, whatever M is, so a row's result does not depend on the batch.
 #include "common.h"
 
+// The compute units of the GPU the library runs on: the caller tells it once (tl_gemm_set_compute_units, from
+// the device's properties); 256, the MI355X on which every plan below was measured, until it does.
+static int g_compute_units = 256;
+extern "C" void tl_gemm_set_compute_units(int n) { if (n > 0) g_compute_units = n; }
+extern "C" int tl_gemm_compute_units() { return g_compute_units; }
+#define TL_COMPUTE_UNITS g_compute_units
+
+
 #define GT_K 16
 
 // BT x BT tile, 256 threads with a (BT / 16) x (BT / 16) micro-tile each: 64 x 64 for small products,
@@ -811,7 +819,7 @@ static void launch_skinny_d(const void* x, const void* w, const void* bias, int 
         auto kernel = gemm_skinny_kernel<R, MT, KS, TOut, SW, true, D>;
         static hipError_t allowed = allow_lds(kernel, 156 * 1024);
         if (allowed == hipSuccess) {
-            const int most = x_bytes <= SKINNY_XL_MAX_BYTES ? 512 : 256;      // a larger x leaves room for one work-group only
+            const int most = x_bytes <= SKINNY_XL_MAX_BYTES ? 2 * TL_COMPUTE_UNITS : TL_COMPUTE_UNITS;      // a larger x leaves room for one work-group only
             StripPlan p = plan_strips(total, most, 16 * R, false);
             if (rows_per_strip > 0) p = StripPlan{(int)grid.x, rps, rps};
             kernel<<<dim3(p.groups), block, red_bytes + x_bytes, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, bias_f32, (TOut*)out, M, N, K, ldx, ldo,
@@ -848,7 +856,6 @@ static void launch_skinny(const void* x, const void* w, const void* bias, int bi
 // 2).  A compute unit draws its weights at a rate of its own, about 26 GB/s whatever shares it with, and the strips
 // beyond one per unit run when the others are done, nearly alone, at the latency of every fetch: at 3584 columns 256 strips of 16 rows take 7.9 us, 257 take 11.2, 288 (the
 // 7B's query/key/value matrix) 11.9 and 512 take 13.4.  The number is even (the fused rotation turns pairs).
-#define TL_COMPUTE_UNITS 256
 static int balanced_rows(int N, int* blocks) {
     *blocks = 1;
     if (N < 4 * TL_COMPUTE_UNITS || N > 32 * TL_COMPUTE_UNITS) return 0;      // a few rows a unit, or more than two blocks
@@ -1366,13 +1373,14 @@ static double dl_estimate(DlTile t, long groups, int k, bool weights_only = fals
     const bool pairs = t == DL_64x64 || t == DL_128x128;
     const double products = 2.0 * DL_BM[t] * DL_BN[t] * k;
     const double stream = weights_only ? 2.0 * DL_BN[t] * k / 32e9 : 2.0 * (DL_BN[t] + DL_BM[t]) * k / 40e9;
-    if (!pairs) return (double)((groups + 255) / 256) * fmax(products / DL_RATE[t] + DL_FIXED[t], stream);
-    const double rate = groups > 256 ? DL_RATE[t] / 2 : DL_RATE[t] * 0.62;
+    const int cus = TL_COMPUTE_UNITS;
+    if (!pairs) return (double)((groups + cus - 1) / cus) * fmax(products / DL_RATE[t] + DL_FIXED[t], stream);
+    const double rate = groups > cus ? DL_RATE[t] / 2 : DL_RATE[t] * 0.62;
     // (a single round of 128 x 128 tiles runs a tenth behind this estimate: measured on the fused gate/up
     // products of the 7B, 14B and 32B at 96 to 512 rows, where it otherwise displaced 128 x 256 tiles
     // that were up to a fifth faster)
-    const double lag = (t == DL_128x128 && groups <= 512) ? 1.1 : 1.0;
-    return lag * (double)((groups + 511) / 512) * fmax(products / rate + DL_FIXED[t], groups > 256 ? 2 * stream : stream);
+    const double lag = (t == DL_128x128 && groups <= 2 * cus) ? 1.1 : 1.0;
+    return lag * (double)((groups + 2 * cus - 1) / (2 * cus)) * fmax(products / rate + DL_FIXED[t], groups > cus ? 2 * stream : stream);
 }
 
 static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = nullptr, bool weights_only = false) {
@@ -1381,7 +1389,7 @@ static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = null
     for (int t = 0; t < DL_TILES; ++t) {
         if (sw && (t == DL_64x64 || t == DL_256x192 || t == DL_64x320)) continue;      // a wave of the fused gate needs whole 64-row blocks of weights
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
-        if (t == DL_128x128_S4 && (tiles > 256 || M > 128)) continue;      // one round of work-groups, every weight drawn once
+        if (t == DL_128x128_S4 && (tiles > TL_COMPUTE_UNITS || M > 128)) continue;      // one round of work-groups, every weight drawn once
         // (the split planner's unsplit baseline is fitted without the 192-wide tiles: with them it kept 512 rows against the
         // 14B's query/key/value matrix whole, 74.8 us, where it used to split K, 53.9 us)
         if (weights_only && (t == DL_64x192 || t == DL_128x192 || t == DL_64x320)) continue;
@@ -1408,10 +1416,10 @@ static DlSplit plan_dl_split(int M, int N, int K) {
         for (int P = 2; P <= 8 && K / P >= 512; ++P) {
             const int k_per = ((steps + P - 1) / P) * 64;
             if ((K + k_per - 1) / k_per != P) continue;
-            if (t == DL_128x128_S4 && tiles * P > 256) continue;       // measured in one round of work-groups only
+            if (t == DL_128x128_S4 && tiles * P > TL_COMPUTE_UNITS) continue;       // measured in one round of work-groups only
             // (the small tile as for up to 64 rows, one work-group to a compute unit: 128 rows against the 7B's output
             // projection 13.0 us in two parts where four parts of 128 x 128 take 17.0)
-            if (t == DL_64x64 && (M > 128 || tiles * P > 256)) continue;
+            if (t == DL_64x64 && (M > 128 || tiles * P > TL_COMPUTE_UNITS)) continue;
             // (a tenth on top: float slabs leave the kernel more slowly than the estimate's bfloat16 rows)
             const double est = 1.1 * dl_estimate(t, tiles * P, k_per, true) + (double)P * M * N * 4 * 2 / 3e12;
             if (est < best_t) { best_t = est; best = DlSplit{t, P, k_per}; }
@@ -1705,7 +1713,7 @@ extern "C" int tl_gemm_swiglu_normed(const void* residual, void* residual_out, c
     const int N = ((I + 31) / 32) * 64;          // rows of the interleaved matrix
     if (!norm_fits(na, K, 16 * 64) || ((uintptr_t)w % 16) || K / 64 / 16 >= 16)
         return TL_NOT_FUSED;
-    const StripPlan p = plan_strips(I, 512, 16, false);       // every work-group makes x once and walks its run of outputs
+    const StripPlan p = plan_strips(I, 2 * TL_COMPUTE_UNITS, 16, false);       // every work-group makes x once and walks its run of outputs
     const size_t lds = (size_t)16 * 1024 + (size_t)(K + 8) * 2;
     gemm_skinny_kernel<1, 1, 16, bf16_t, true, true, 2, false, true><<<dim3(p.groups), dim3(16 * 64), lds, stream>>>(
         nullptr, (const bf16_t*)w, nullptr, 0, (bf16_t*)out, 1, N, K, K, I, I, 0, p.per_strip, p.per_group, RopeArgs{}, na);
@@ -1770,7 +1778,7 @@ extern "C" int tl_gemm_partials_max() { return 8; }
 // (320 strips, one work-group of eight waves with eight steps in flight per compute unit: two rounds,
 // the second nearly empty).
 static bool partials_on_tiles(int M, int N, int K) {
-    return K % 64 == 0 && (M >= 2 || N > 16 * 256);
+    return K % 64 == 0 && (M >= 2 || N > 16 * TL_COMPUTE_UNITS);
 }
 
 // Whether a consumer that can add slabs up should ask for them instead of the whole product.
@@ -1781,7 +1789,7 @@ extern "C" int tl_gemm_partials_parts(int M, int N, int K) {
     if (M > 64 && K % 64 == 0) return plan_dl_split(M, N, K).parts;
     if (partials_on_tiles(M, N, K)) {
         const long tiles = (long)((M + 63) / 64) * ((N + 63) / 64);
-        int P = (int)(256 / tiles);                       // about one work-group per compute unit
+        int P = (int)(TL_COMPUTE_UNITS / tiles);          // about one work-group per compute unit
         const int by_k = K / 512;                         // at least eight slabs of 64 per part
         if (P > by_k) P = by_k;
         if (P > 8) P = 8;

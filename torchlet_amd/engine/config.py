@@ -22,7 +22,7 @@ class EngineConfig:
     max_slots: int = 4                   # most requests live at a time (max_decode_slots)
     max_tokens_per_step: int = 2048      # token budget of a step: decode tokens first, prompt portions with the rest
     max_model_len: int | None = None     # most positions of a sequence; None: the model's max_position_embeddings
-    dtype: str = "bfloat16"              # compute dtype: bfloat16, or float32 for the true 32-bit path
+    dtype: str | None = None             # compute dtype: bfloat16, or float32 for the true 32-bit path; None: the model folder's
     kv_dtype: str | None = None          # element type of the cache pages; None: the compute dtype (no other is built)
     use_graphs: bool = False             # decode-only steps replay a captured HIP graph
     lookahead: bool = True               # the engine enqueues a decode step before it has read the tokens of the one before
@@ -40,7 +40,9 @@ class EngineConfig:
             raise ValueError("max_model_len must be positive")
         if not 0.0 < self.memory_fraction <= 1.0:
             raise ValueError("memory_fraction must lie in (0, 1]")
-        if self.kv_dtype is not None and _canonical(self.kv_dtype) != _canonical(self.dtype):
+        if self.dtype is not None and _canonical(self.dtype) not in ("bfloat16", "float32"):
+            raise ValueError(f"compute dtype must be bfloat16 or float32, got {self.dtype!r}")
+        if self.kv_dtype is not None and self.dtype is not None and _canonical(self.kv_dtype) != _canonical(self.dtype):
             raise ValueError(f"cache pages of {self.kv_dtype} under a {self.dtype} engine are not built: the cache has the compute dtype")
 
     def model_len(self, model_max_positions: int) -> int:

@@ -10,7 +10,7 @@ from ..config.base import ModelConfig
 from ..kernels import ops
 from ..models.decoder import DecoderModel
 from ..registry import load_config
-from ..weights.loader import load_folder, load_into
+from ..weights.loader import folder_dtype, load_folder, load_into
 from .config import EngineConfig
 from .runner import ModelRunner
 
@@ -52,9 +52,21 @@ def build_model(config: ModelConfig, dtype, device=None, tensors=None, folder: s
     return model
 
 
-def load_model(folder: str | Path, dtype="bfloat16", device=None) -> tuple[ModelConfig, DecoderModel]:
+def resolve_dtype(folder: str | Path, config: ModelConfig, dtype=None) -> str:
+    """The engine's compute dtype for a model folder: ``dtype`` if the caller names one (the weights are
+    converted at load), else what the folder says: its ``config.json``'s ``torch_dtype`` (for a configuration
+    class that reads the key), else the element type of its first floating-point tensor.  The reference types
+    its parameters and its cache after the checkpoint (/root/reference/src/torchlet/utils.py:18-38,
+    v10_triton_paged_gqa/engine.py:58), so a folder stored in 32-bit gives a 32-bit engine."""
+    if dtype is not None:
+        return "float32" if parse_dtype(dtype) == torch.float32 else "bfloat16"
+    return folder_dtype(folder, getattr(config, "torch_dtype", None) or None)
+
+
+def load_model(folder: str | Path, dtype=None, device=None) -> tuple[ModelConfig, DecoderModel]:
+    """``dtype=None``: the folder's own (see :func:`resolve_dtype`)."""
     config = load_config(folder)
-    return config, build_model(config, dtype, device, folder=folder)
+    return config, build_model(config, resolve_dtype(folder, config, dtype), device, folder=folder)
 
 
 def make_runner(model: DecoderModel, config: EngineConfig | None = None, *, page_size: int | None = None,
@@ -66,8 +78,10 @@ def make_runner(model: DecoderModel, config: EngineConfig | None = None, *, page
     the tokens of a step (a scheduler's budget), which sizes the pools of windowed groups; ``None`` for
     callers that step as they like."""
     from dataclasses import replace
-    config = config or EngineConfig(dtype="float32" if model.dtype == torch.float32 else "bfloat16")
+    config = config or EngineConfig()
     given = dict(page_size=page_size, num_pages=num_pages, max_slots=max_requests, use_graphs=use_graphs, max_model_len=max_model_len)
+    if config.dtype is None:             # not named: the dtype the model was built in
+        given["dtype"] = "float32" if model.dtype == torch.float32 else "bfloat16"
     config = replace(config, **{k: v for k, v in given.items() if v is not None})
     if parse_dtype(config.dtype) != model.dtype:
         raise ValueError(f"the engine is configured for {config.dtype}, the model was built in {model.dtype}")

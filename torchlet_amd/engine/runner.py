@@ -7,6 +7,7 @@ raises :class:`~torchlet_amd.cache.manager.OutOfPages` and leaves the cache as i
 """
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, OutOfPages
@@ -30,8 +31,9 @@ class ModelRunner:
     """``use_graphs``: decode-only steps (one new token for every request) run from static
     buffers under a captured HIP graph, one graph per (batch width, context length) bucket,
     as the reference replays its decode step as a CUDA graph
-    (/root/reference/src/torchlet/v10_triton_paged_gqa/engine.py:137-185).  A bucket's first
-    step runs eagerly from the static buffers and is then captured; capture records without
+    (/root/reference/src/torchlet/v10_triton_paged_gqa/engine.py:137-185).  :meth:`warm_up` captures
+    the graphs an engine can reach before it serves; a bucket that was not captured ahead runs its first
+    step eagerly from the static buffers and is captured then.  Capture records without
     running, so results are only ever read after an eager run or a replay (the reference
     reads its output buffer right after capture, engine.py:165-176)."""
 
@@ -47,6 +49,7 @@ class ModelRunner:
         self.use_graphs = use_graphs and torch.device(self.device).type == "cuda" and model.graph_safe()
         self.max_graph_width = max_graph_width
         self._graphs: dict[tuple[int, int], _DecodeGraph] = {}
+        self._graph_pool = None
         self.graph_replays = 0
 
     def step(self, entries: list[StepEntry], device_tokens: tuple | None = None) -> torch.Tensor | None:
@@ -139,30 +142,78 @@ class ModelRunner:
             cache.commit(e.req_id, c + n)
         return logits
 
+    def _bucket(self, blocks: int) -> int:
+        """The context bucket (block-table width) of a graph step whose longest sequence has ``blocks`` pages."""
+        most = -(-self.max_positions // self.cache.page_size)
+        return min(most, max(_next_pow2(blocks), min(most, 256 // self.cache.page_size or 1)))
+
+    def _decode_graph(self, key: tuple[int, int]) -> _DecodeGraph:
+        dg = self._graphs.get(key)
+        if dg is None:
+            cache = self.cache
+            dg = self._graphs[key] = _DecodeGraph(StaticDecodeContext(
+                width=key[0], blocks=key[1], num_groups=len(cache.groups), tile_sizes=self.tile_sizes,
+                page_size=cache.page_size, device=self.device, pad_slot=cache.pad_slot))
+        return dg
+
+    def _capture(self, dg: _DecodeGraph) -> None:
+        """Record the forward pass over ``dg.ctx`` (recording runs nothing).  All graphs share one pool of
+        memory: they replay one after the other on one stream, and what reads a graph's logits is enqueued
+        before the next replay."""
+        torch.cuda.synchronize()
+        if self._graph_pool is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, pool=self._graph_pool):
+            dg.logits = self.model.forward(dg.ctx, self.caches)
+        dg.graph = graph
+
+    def warm_up(self, widths=None, max_len: int | None = None) -> int:
+        """Capture, ahead of need, the graph of every (batch width, context bucket) that decode steps of up to
+        ``max(widths)`` requests (default: as many as the cache has slots) and sequences of up to ``max_len``
+        tokens (default: the engine's limit) can ask for, so that no serving step stops to capture one
+        (the reference captures its one shape inside its first decode step,
+        /root/reference/src/torchlet/v10_triton_paged_gqa/engine.py:137-176).  Each shape runs once eagerly
+        on padding rows alone, which write to no page and to no request's state, and is then recorded.
+        Returns the number of graphs captured; nothing happens without ``use_graphs``."""
+        if not self.use_graphs:
+            return 0
+        cache = self.cache
+        if widths is None:
+            widths = [cache.max_requests]
+        top = min(_next_pow2(max(widths)), _next_pow2(self.max_graph_width))
+        max_len = self.max_positions if max_len is None else min(max_len, self.max_positions)
+        most_blocks = _next_pow2(-(-max_len // cache.page_size))
+        buckets = sorted({self._bucket(1 << i) for i in range(most_blocks.bit_length())})   # of 1, 2, 4, ... pages
+        captured = 0
+        width = 1
+        while width <= top:
+            for bucket in buckets:
+                dg = self._decode_graph((width, bucket))
+                if dg.graph is None:
+                    dg.ctx.fill(token_ids=[], ctx_lens=[], slots=[],
+                                block_tables=[np.zeros((0, bucket), dtype=np.int32) for _ in cache.groups])
+                    self.model.forward(dg.ctx, self.caches)       # eager once: kernels loaded, buffers of this shape known
+                    self._capture(dg)
+                    captured += 1
+            width *= 2
+        torch.cuda.synchronize()
+        return captured
+
     def _graph_step(self, entries, req_ids, ctx_lens, blocks, taken=None) -> torch.Tensor:
         cache = self.cache
         width = _next_pow2(len(entries))
-        most = -(-self.max_positions // cache.page_size)
-        bucket = min(most, max(_next_pow2(blocks), min(most, 256 // cache.page_size or 1)))
-        key = (width, bucket)
-        dg = self._graphs.get(key)
-        if dg is None:
-            dg = self._graphs[key] = _DecodeGraph(StaticDecodeContext(
-                width=width, blocks=bucket, num_groups=len(cache.groups), tile_sizes=self.tile_sizes,
-                page_size=cache.page_size, device=self.device, pad_slot=cache.pad_slot))
+        bucket = self._bucket(blocks)
+        dg = self._decode_graph((width, bucket))
         dg.ctx.fill(token_ids=[e.tokens[0] for e in entries], ctx_lens=ctx_lens,
                     slots=[cache.slot(r) for r in req_ids],
                     block_tables=[cache.block_table(g, req_ids, bucket) for g in range(len(cache.groups))])
         if taken is not None:
             dg.ctx.token_ids[: len(entries)].copy_(taken)             # after the copy of the step's other numbers
-        if dg.graph is None:
+        if dg.graph is None:                                          # a shape that was not captured ahead
             logits = self.model.forward(dg.ctx, self.caches)          # eager: this step's result
             result = logits[: len(entries)].clone()
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):                             # records, does not run
-                dg.logits = self.model.forward(dg.ctx, self.caches)
-            dg.graph = graph
+            self._capture(dg)
             return result
         dg.graph.replay()
         self.graph_replays += 1

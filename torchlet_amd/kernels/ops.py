@@ -39,6 +39,8 @@ def _lib(name: str) -> ctypes.CDLL:
             raise KernelError(f"cannot load {path}: {exc}") from exc
         lib.tl_last_error.restype = ctypes.c_char_p
         _libs[name] = lib
+        if name == "gemm" and torch.cuda.is_available():
+            lib.tl_gemm_set_compute_units(c_int(compute_units()))
     return lib
 
 
@@ -50,6 +52,24 @@ def load(names) -> None:
         _build.build_many(stale)
     for n in missing:
         _lib(n)
+
+
+MEASURED_COMPUTE_UNITS = 256      # the MI355X on which the kernels' plans were fitted
+_compute_units: int | None = None
+
+
+def compute_units() -> int:
+    """The compute units of the current GPU, read from the device once; the matrix-product library's planners are
+    told the same number, and parts that deal work to the compute units (how many parts a request's keys are cut
+    into) get it from here.  Without a GPU: the MI355X's 256, for which the plans were measured."""
+    global _compute_units
+    if _compute_units is None:
+        if not torch.cuda.is_available():
+            return MEASURED_COMPUTE_UNITS
+        _compute_units = int(torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count)
+        if "gemm" in _libs:
+            _libs["gemm"].tl_gemm_set_compute_units(c_int(_compute_units))
+    return _compute_units
 
 
 def loaded_libraries() -> list[str]:

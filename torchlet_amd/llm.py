@@ -7,7 +7,9 @@ meanings: ``max_decode_slots`` is the most requests live at a time, ``kv_block_s
 tokens per cache page, ``max_num_blocks`` the pages of the pool including the sentinel
 (default ``max_decode_slots * ceil(max_position_embeddings / kv_block_size) + 1``,
 engine.py:40-47 of the reference, capped by free GPU memory).  ``model_id`` is a local
-model folder (nothing is downloaded).  Additions: ``dtype``, ``max_num_batched_tokens`` (the
+model folder (nothing is downloaded).  Additions: ``dtype`` (default: the folder's own, its ``torch_dtype`` or the
+element type it stores, as the reference runs a checkpoint in the dtype it is stored in, utils.py:18-38;
+``bfloat16`` or ``float32`` converts at load), ``max_num_batched_tokens`` (the
 step's token budget), ``max_model_len`` (sequences no longer than this: a smaller default pool), ``seed``,
 ``use_graphs`` (decode-only steps replay a captured HIP graph); or all of them at once as an
 :class:`~torchlet_amd.engine.config.EngineConfig` (``engine_config=``).  ``generate`` also takes ``temperature``,
@@ -40,7 +42,7 @@ from .logger import backend_info, logger, weights_info
 
 class LLM:
     def __init__(self, model_id: str, max_decode_slots: int = 4, kv_block_size: int = 16,
-                 max_num_blocks: int | None = None, *, dtype: str = "bfloat16",
+                 max_num_blocks: int | None = None, *, dtype: str | None = None,
                  max_num_batched_tokens: int = 2048, max_model_len: int | None = None, seed: int = 0,
                  use_graphs: bool = True, lookahead: bool = True, engine_config: EngineConfig | None = None):
         self.device = require_gpu()
@@ -50,7 +52,7 @@ class LLM:
             raise ValueError("max_decode_slots must be positive")
         self.engine_config = engine_config or EngineConfig(
             page_size=kv_block_size, num_pages=max_num_blocks, max_slots=max_decode_slots,
-            max_tokens_per_step=max_num_batched_tokens, max_model_len=max_model_len, dtype=str(dtype).replace("torch.", ""),
+            max_tokens_per_step=max_num_batched_tokens, max_model_len=max_model_len, dtype=None if dtype is None else str(dtype).replace("torch.", ""),
             use_graphs=use_graphs, lookahead=lookahead, seed=seed)
         self.model_dir = Path(model_id)
         if logger.isEnabledFor(20):                         # INFO: the start-up reports of the reference's LLM (llm.py:28-36)
@@ -60,7 +62,8 @@ class LLM:
         self.config, self.model = load_model(self.model_dir, self.engine_config.dtype, self.device)
         self.engine = make_engine(self.model, self.engine_config)
         self.runner = self.engine.runner
-        self.engine_config = self.runner.config            # with the number of pages filled in
+        self.engine_config = self.runner.config            # with the dtype and the number of pages filled in
+        self.graphs_captured = self.runner.warm_up()       # ahead of need: no serving step stops to capture one
         logger.info("model: %s, %d runs of %d layers, %s; engine: %s; cache: %s pages free per group, %d bytes a page",
                     self.config.architecture, len(self.model.spec.order), len(self.model.spec.layers), self.model.dtype,
                     self.engine_config, self.runner.cache.free_pages(), self.runner.cache.bytes_per_page())
@@ -206,7 +209,7 @@ def _parser():
         q.add_argument("--max-new-tokens", type=int, default=128)
         q.add_argument("--temperature", type=float, default=0.0, help="0: greedy")
         q.add_argument("--seed", type=int, default=0, help="sampler seed")
-        q.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+        q.add_argument("--dtype", default=None, choices=["bfloat16", "float32"], help="compute dtype (default: the model folder's own)")
         q.add_argument("--max-decode-slots", type=int, default=4)
         q.add_argument("--kv-block-size", type=int, default=16)
         q.add_argument("--max-num-blocks", type=int, default=None)

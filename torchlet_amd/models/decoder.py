@@ -14,6 +14,7 @@ import torch
 from ..config.base import ModelSpec
 from ..kernels import ops
 from ..parts import BLOCKS, NORMS, Stream, WeightSpec
+from ..parts.base import KEEP_COMPUTE, KEEP_STORED, place
 
 
 class DecoderModel:
@@ -41,12 +42,12 @@ class DecoderModel:
         # a tied head is the embedding matrix; a checkpoint may still carry a copy of it
         specs[f"{s.head_name}.weight"] = WeightSpec((s.vocab_size, s.hidden), optional=s.tie_head)
         if s.head_bias:
-            specs[f"{s.head_name}.bias"] = WeightSpec((s.vocab_size,), role="vector")
+            specs[f"{s.head_name}.bias"] = WeightSpec((s.vocab_size,), keep=KEEP_STORED)
         return specs
 
     def load_weights(self, tensors: dict[str, torch.Tensor]) -> None:
         s = self.spec
-        self.embed = tensors[f"{s.embed_name}.weight"].to(device=self.device, dtype=self.dtype).contiguous()
+        self.embed = place(tensors[f"{s.embed_name}.weight"], KEEP_COMPUTE, self.dtype, self.device)
         names = list(tensors)      # `tensors` may read from disk on access: touch each name once
         for i, block in enumerate(self.blocks):
             prefix = f"{s.layers_prefix}.{i}."
@@ -56,12 +57,9 @@ class DecoderModel:
         if s.tie_head:
             self.head = self.embed
         else:
-            self.head = tensors[f"{s.head_name}.weight"].to(device=self.device, dtype=self.dtype).contiguous()
+            self.head = place(tensors[f"{s.head_name}.weight"], KEEP_COMPUTE, self.dtype, self.device)
         if s.head_bias:
-            b = tensors[f"{s.head_name}.bias"]
-            if self.dtype == torch.float32 or b.dtype not in (torch.bfloat16, torch.float32):
-                b = b.to(torch.float32)
-            self.head_bias = b.to(self.device).contiguous()
+            self.head_bias = place(tensors[f"{s.head_name}.bias"], KEEP_STORED, self.dtype, self.device)
 
     # ------------------------------------------------------------------ cache needs
     def cache_plan(self):
@@ -75,9 +73,16 @@ class DecoderModel:
     def tile_token_sizes(self) -> set[int]:
         return {b.mixer.tile_tokens for b in self.blocks if hasattr(b.mixer, "tile_tokens")}
 
+    def parts(self):
+        """Every part of the model: each block with what is inside it, and the final norm."""
+        for b in self.blocks:
+            yield from b.parts()
+        yield from self.final_norm.parts()
+
     def graph_safe(self) -> bool:
-        """Every mixer runs from device-side metadata only, so a step can be captured as a graph."""
-        return all(getattr(b.mixer, "graph_safe", False) for b in self.blocks)
+        """Every part of every block (and the final norm) says that it runs from device-side values only,
+        so a decode step can be captured once as a graph and replayed."""
+        return all(getattr(p, "graph_safe", False) for p in self.parts())
 
     def kernel_libraries(self) -> list[str]:
         libs = ["elementwise", "gemm", "sampling"]

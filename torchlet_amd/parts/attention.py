@@ -17,43 +17,45 @@ import torch
 
 from ..config.base import ConfigError
 from ..kernels import ops
-from .base import MIXERS, POSITION_ENCODINGS, LazyNorm, Mixer, PagedNeed, WeightSpec
+from .base import KEEP_COMPUTE, KEEP_STORED, MIXERS, POSITION_ENCODINGS, LazyNorm, Mixer, PagedNeed, WeightSpec
 
-_COMPUTE_UNITS = 256
-_TARGET_WORKGROUPS = 512     # enough work-groups of four waves to fill 256 compute units twice
+# The plans below deal work-groups to the GPU's compute units; their number comes from the device
+# (``ops.compute_units()``), the thresholds in keys and tokens were measured on an MI355X (256 units).
 _MIN_KEYS_PER_SPLIT = 256
 _PORTION_MIN_TOKENS = 16     # requests that bring at least this many tokens go to a prompt-portion kernel: the
                              # 128-row one where it is built (head size 64 or 128, pages of 8, 16, 32, ...
                              # tokens; measured on MI355X at 28/4 heads of 128: 2048 new tokens 222 -> 110 us,
                              # 8192 new tokens 2.9 -> 0.84 ms), else the 64-row one ...
 _PORTION_MIN_CONTEXT = 4096  # ... which pays only in steps whose longest sequence has at least this many tokens
-_PROMPT_TARGET_WORKGROUPS = 1024  # the 128-row kernel: two work-groups fit a compute unit; two rounds of them (measured: 14B serving 16.2k -> 16.5k tokens/s against one round)
-_PROMPT_SPLIT_BELOW = 256        # ... but only steps whose tiles alone cannot give every compute unit one (a whole prompt of
-                                 # 2048 tokens has 456: split in two it took 85 + 19 us of merge against 90 us)
+# The 128-row kernel: two work-groups fit a compute unit; the keys of a step's tiles are dealt out to make two rounds
+# of them (measured: 14B serving 16.2k -> 16.5k tokens/s against one round), but only in steps whose tiles alone
+# cannot give every compute unit one (a whole prompt of 2048 tokens has 456: split in two it took 85 + 19 us of
+# merge against 90 us)
 _PROMPT_MIN_KEYS_PER_SPLIT = 512
-_PROMPT_ROUND = 512                 # work-groups of the 128-row kernel that run at once
 _PROMPT_MAX_SPLITS = 4
 
 
-def _prompt_splits(groups: int, keys: int, uniform: bool) -> int:
+def _prompt_splits(groups: int, keys: int, uniform: bool, units: int = ops.MEASURED_COMPUTE_UNITS) -> int:
     """Into how many parts the 128-row kernel deals the keys of every tile: ``groups`` work-groups without a split,
     ``keys`` the longest sequence; ``uniform``: every tile sees about as many keys (portions deep into their
-    prompts), so the work-groups come in rounds of equal length."""
+    prompts), so the work-groups come in rounds of equal length; ``units``: the GPU's compute units."""
     most = max(1, min(_PROMPT_MAX_SPLITS, keys // _PROMPT_MIN_KEYS_PER_SPLIT))
-    if groups <= _PROMPT_SPLIT_BELOW:
-        return max(1, min(most, _PROMPT_TARGET_WORKGROUPS // max(groups, 1)))
-    if not uniform or groups <= _PROMPT_ROUND:
+    round_ = 2 * units                  # work-groups of the 128-row kernel that run at once
+    if groups <= units:
+        return max(1, min(most, 2 * round_ // max(groups, 1)))
+    if not uniform or groups <= round_:
         return 1
-    # rounds of 512 work-groups (two to a compute unit), the last one as long as the others however few are in it:
+    # rounds of work-groups (two to a compute unit; 512 on the MI355X), the last one as long as the others however few are in it:
     # 640 tiles of a 2048-token step of 40 heads take two rounds whole and five quarter rounds in four parts
     # (measured at 32B sizes, 2048 tokens after 0 to 14336 cached ones: 545 -> 442 us a layer, and 24 us of merge)
-    cost = lambda n: -(-groups * n // _PROMPT_ROUND) / n * (1.0 if n == 1 else 1.08)
+    cost = lambda n: -(-groups * n // round_) / n * (1.0 if n == 1 else 1.08)
     return min(range(1, most + 1), key=cost)
 
 
 @MIXERS.register("gqa_attention")
 class GQAttention(Mixer):
-    graph_safe = True       # nothing in forward() depends on host-side values of the step
+    graph_safe = True       # nothing in forward() depends on host-side values of the step; a subclass whose stage or
+                            # `transform_qk` hook reads values of the step on the host must set it back to False
 
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
@@ -73,6 +75,7 @@ class GQAttention(Mixer):
         self.kv_width = self.kv_heads * self.head_dim
         self.qkv_bias = spec.qkv_bias
         self.position = POSITION_ENCODINGS.build(spec.position, dtype, device) if spec.position is not None else None
+        self.compute_units = ops.compute_units()       # of the GPU it runs on: how far the keys of a request are dealt out
         self.tile_tokens = ops.attention_tile_tokens(self.heads, self.kv_heads)
         self.portion_tile_tokens = ops.prefill_attention_tile_tokens(self.heads, self.kv_heads)
         self.prompt_tile_tokens = ops.prompt_attention_tile_tokens(self.heads, self.kv_heads)
@@ -88,6 +91,11 @@ class GQAttention(Mixer):
     def kernel_libraries(self):
         return [ops.attention_library(self.head_dim)]
 
+    def parts(self):
+        yield self
+        if self.position is not None:
+            yield from self.position.parts()
+
     def weight_specs(self):
         specs = {
             "q_proj.weight": WeightSpec((self.q_width, self.hidden)),
@@ -96,9 +104,9 @@ class GQAttention(Mixer):
             "o_proj.weight": WeightSpec((self.hidden, self.q_width)),
         }
         if self.qkv_bias:
-            specs["q_proj.bias"] = WeightSpec((self.q_width,), role="vector")
-            specs["k_proj.bias"] = WeightSpec((self.kv_width,), role="vector")
-            specs["v_proj.bias"] = WeightSpec((self.kv_width,), role="vector")
+            specs["q_proj.bias"] = WeightSpec((self.q_width,), keep=KEEP_STORED)
+            specs["k_proj.bias"] = WeightSpec((self.kv_width,), keep=KEEP_STORED)
+            specs["v_proj.bias"] = WeightSpec((self.kv_width,), keep=KEEP_STORED)
         return specs
 
     def load_weights(self, tensors):
@@ -111,13 +119,13 @@ class GQAttention(Mixer):
                             and self.position.fused_inv_freq() is not None and self.transform_qk is None)
         rows = {"q": ops.pair_layout_rows(self.heads, self.head_dim), "k": ops.pair_layout_rows(self.kv_heads, self.head_dim)}
         order = lambda n, t: t[rows[n]] if self.pair_layout and n in rows else t
-        self.w_qkv = self._place(torch.cat([order(n, tensors[f"{n}_proj.weight"]) for n in "qkv"], dim=0), "matrix")
+        self.w_qkv = self._place(torch.cat([order(n, tensors[f"{n}_proj.weight"]) for n in "qkv"], dim=0), KEEP_COMPUTE)
         if self.qkv_bias:
             biases = [order(n, tensors[f"{n}_proj.bias"]) for n in "qkv"]
             if len({b.dtype for b in biases}) > 1:
                 biases = [b.to(torch.float32) for b in biases]
-            self.b_qkv = self._place(torch.cat(biases), "vector")
-        self.w_o = self._place(tensors["o_proj.weight"], "matrix")
+            self.b_qkv = self._place(torch.cat(biases), KEEP_STORED)
+        self.w_o = self._place(tensors["o_proj.weight"], KEEP_COMPUTE)
 
     # -- the step -----------------------------------------------------------------
     def _splits(self, ctx, tiles: int, longest: int | None = None) -> tuple[int, int]:
@@ -127,8 +135,9 @@ class GQAttention(Mixer):
         group = self.heads // self.kv_heads
         chunks = -(-group // ops.ATTENTION_ROWS)
         base = max(1, tiles * self.kv_heads * chunks)
-        waves = 8 if base <= _COMPUTE_UNITS else 4
-        by_fill = -(-(_COMPUTE_UNITS if waves == 8 else _TARGET_WORKGROUPS) // base)
+        units = self.compute_units
+        waves = 8 if base <= units else 4
+        by_fill = -(-(units if waves == 8 else 2 * units) // base)      # four waves: enough work-groups to fill the units twice
         longest = ctx.max_total_len if longest is None else longest
         longest = longest if self.window is None else min(longest, self.window + ctx.max_new_tokens)
         by_keys = max(1, longest // _MIN_KEYS_PER_SPLIT)
@@ -174,9 +183,10 @@ class GQAttention(Mixer):
         plain = self.transform_qk is not None               # nothing fused: the hook sits between projection and rotation
         fused = False
         if lazy is not None:
-            if self.pair_layout and not plain:
+            rms = lazy.rmsnorm()          # the fused kernel makes a root-mean-square norm and no other
+            if self.pair_layout and not plain and rms is not None:
                 residual_out = torch.empty_like(lazy.residual)
-                fused = ops.linear_rope_cache_write_normed(lazy.residual, lazy.pending, lazy.norm.weight, lazy.norm.eps,
+                fused = ops.linear_rope_cache_write_normed(lazy.residual, lazy.pending, rms[0], rms[1],
                                                            residual_out, w, b, qkv, self.heads, self.kv_heads, self.head_dim,
                                                            ctx.positions, inv_freq, *cache_args)
                 if fused:
@@ -228,7 +238,7 @@ class GQAttention(Mixer):
                 # each tile's keys are dealt to several work-groups, so that the compute units have work
                 groups = long[2] * self.kv_heads * -(-(self.heads // self.kv_heads) // ops.PROMPT_ATTENTION_ROWS)
                 keys = ctx.max_total_len if self.window is None else min(ctx.max_total_len, self.window + tq)
-                splits = _prompt_splits(groups, keys, uniform=long[5] >= 2 * ctx.max_new_tokens)
+                splits = _prompt_splits(groups, keys, uniform=long[5] >= 2 * ctx.max_new_tokens, units=self.compute_units)
                 extra = dict(max_total_len=ctx.max_total_len, splits=splits, merge_tokens=(long[3], long[4]))
             kernel(q, out, k_plane, v_plane, table, ctx.req_indptr, ctx.ctx_lens, long[0], long[1], long[2], tq, *common, **extra)
             if short[2]:     # split over their keys; the merge of the parts is kept to the rows of these requests

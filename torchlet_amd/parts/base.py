@@ -28,26 +28,92 @@ from ..config.base import ConfigError, PartSpec
 
 # ------------------------------------------------------------------ weights of a part
 
+# How a tensor is kept on the GPU, whatever its shape: a dtype policy.
+KEEP_COMPUTE = "compute"     # the engine's compute dtype (matrix-product operands)
+KEEP_STORED = "stored"       # as stored: bfloat16 stays bfloat16, 32-bit stays 32-bit; a 32-bit engine widens
+KEEP_FLOAT32 = "float32"     # always 32-bit, also under a bfloat16 engine (a router, a gate, a decay)
+KEEP_INT32 = "int32"         # integer tables
+DTYPE_POLICIES = (KEEP_COMPUTE, KEEP_STORED, KEEP_FLOAT32, KEEP_INT32)
+
+# The laws of the random-weights mode: name -> f(shape, generator, device, std) -> float32 (or int32) tensor.
+# A part that needs another law (a log-decay, a positive-only scale) adds it here by name and declares it.
+INIT_LAWS: dict[str, Callable] = {}
+
+
+def register_init_law(name: str) -> Callable[[Callable], Callable]:
+    def add(fn: Callable) -> Callable:
+        INIT_LAWS[name] = fn
+        return fn
+    return add
+
+
+@register_init_law("normal")
+def _init_normal(shape, gen, device, std):
+    return torch.randn(shape, generator=gen, device=device, dtype=torch.float32) * std
+
+
+@register_init_law("one_plus_normal")
+def _init_one_plus_normal(shape, gen, device, std):
+    return torch.randn(shape, generator=gen, device=device, dtype=torch.float32) * std + 1.0
+
+
+@register_init_law("random_table")
+def _init_random_table(shape, gen, device, std):
+    return torch.randint(0, 2 ** 15, shape, generator=gen, device=device, dtype=torch.int32)
+
+
 @dataclass(frozen=True)
 class WeightSpec:
     """One tensor a part wants from the checkpoint.
 
-    ``role``: ``matrix`` tensors are matrix-product operands and take the engine's
-    compute dtype; ``vector`` tensors keep the dtype they are stored in (bfloat16 stays
-    bfloat16, 32-bit stays 32-bit; a 32-bit engine widens them); ``table`` tensors are
-    integer tables kept as int32.
-    ``init``: law of the random-weights mode, ``normal`` = N(0, std),
-    ``one_plus_normal`` = 1 + N(0, std).
+    ``keep``: the dtype policy, one of :data:`DTYPE_POLICIES`, independent of the tensor's shape:
+    ``compute`` tensors take the engine's compute dtype (matrix-product operands), ``stored``
+    tensors keep the dtype they are stored in (bfloat16 stays bfloat16, 32-bit stays 32-bit; a 32-bit
+    engine widens them: norm weights, biases), ``float32`` tensors are 32-bit under every engine,
+    ``int32`` tensors are integer tables.
+    ``init``: the name of a law in :data:`INIT_LAWS` for the random-weights mode (``normal`` =
+    N(0, std), ``one_plus_normal`` = 1 + N(0, std), ``random_table`` = integers).
     ``optional``: the checkpoint may leave it out (a tied head).
     """
     shape: tuple[int, ...]
-    role: str = "matrix"
+    keep: str = KEEP_COMPUTE
     init: str = "normal"
     optional: bool = False
 
+    def __post_init__(self):
+        if self.keep not in DTYPE_POLICIES:
+            raise ConfigError(f"a tensor's dtype policy is one of {', '.join(DTYPE_POLICIES)}, not {self.keep!r}")
+        if self.init not in INIT_LAWS:
+            raise ConfigError(f"no initialisation law {self.init!r}; known: {', '.join(sorted(INIT_LAWS))}")
+
+    @property
+    def integer(self) -> bool:
+        return self.keep == KEEP_INT32
+
+
+def place(t: torch.Tensor, keep: str, dtype: torch.dtype, device) -> torch.Tensor:
+    """``t`` on ``device`` in the dtype that the policy ``keep`` gives it under an engine of ``dtype``."""
+    if keep not in DTYPE_POLICIES:
+        raise ConfigError(f"a tensor's dtype policy is one of {', '.join(DTYPE_POLICIES)}, not {keep!r}")
+    if keep == KEEP_COMPUTE:
+        return t.to(device=device, dtype=dtype).contiguous()
+    if keep == KEEP_INT32:
+        return t.to(device=device, dtype=torch.int32).contiguous()
+    if keep == KEEP_FLOAT32 or dtype == torch.float32 or t.dtype not in (torch.bfloat16, torch.float32):
+        t = t.to(torch.float32)
+    return t.to(device).contiguous()
+
 
 class Part:
-    """Common protocol: declare tensors, receive them."""
+    """Common protocol: declare tensors, receive them, say whether a step may be recorded.
+
+    ``graph_safe``: nothing in the part's ``forward`` depends on host-side values of the step (no
+    ``.item()``, ``.nonzero()``, shapes that follow the tokens), so a decode step through it can be
+    captured once as a HIP graph and replayed.  ``False`` unless a part says otherwise; a model runs
+    under graphs only if every part of every block says ``True``.  A subclass that overrides a stage or
+    adds a hook that reads host values must set it back to ``False``."""
+
+    graph_safe = False
 
     def __init__(self, spec: PartSpec, dtype: torch.dtype, device: torch.device):
         self.spec = spec
@@ -60,15 +126,13 @@ class Part:
     def load_weights(self, tensors: dict[str, torch.Tensor]) -> None:
         """``tensors``: the declared names (those present) -> CPU tensors as stored."""
 
+    def parts(self):
+        """This part and every part inside it (a block's four, a mixer's position encoding)."""
+        yield self
+
     # helpers ---------------------------------------------------------------------
-    def _place(self, t: torch.Tensor, role: str) -> torch.Tensor:
-        if role == "matrix":
-            return t.to(device=self.device, dtype=self.dtype).contiguous()
-        if role == "table":
-            return t.to(device=self.device, dtype=torch.int32).contiguous()
-        if self.dtype == torch.float32 or t.dtype not in (torch.bfloat16, torch.float32):
-            t = t.to(torch.float32)
-        return t.to(self.device).contiguous()
+    def _place(self, t: torch.Tensor, keep: str) -> torch.Tensor:
+        return place(t, keep, self.dtype, self.device)
 
 
 # ------------------------------------------------------------------------ cache needs
@@ -120,15 +184,24 @@ class Stream:
 
 class LazyNorm:
     """A norm that has not run yet, handed to the part that reads its output: ``norm(residual + pending)`` of
-    the stream, described by what a kernel needs to make it itself (``residual``, ``pending``, ``weight``,
-    ``eps``).  A consumer whose kernel did so calls :meth:`done` with the new residual it wrote; any other
-    calls :meth:`value`, which runs the norm the usual way (once).  The norm's own kernel is a launch and a
-    trip to memory that a step of one token can do without."""
+    the stream.  It states which norm it is (``kind``, the norm's registry name) and carries that kind's
+    constants (``rmsnorm``: ``weight`` and ``eps``), so that a consumer whose kernel can make a norm of that
+    kind itself does so and calls :meth:`done` with the new residual it wrote; a consumer that does not know the
+    kind, or whose shapes do not fit, calls :meth:`value`, which runs the norm the usual way (once).  The norm's
+    own kernel is a launch and a trip to memory that a step of one token can do without."""
 
-    def __init__(self, norm, stream: "Stream"):
+    def __init__(self, norm, stream: "Stream", kind: str, **constants):
         self.norm = norm
         self.stream = stream
+        self.kind = kind
+        self.constants = constants
         self._value = None
+
+    def rmsnorm(self):
+        """``(weight, eps)`` if this is a root-mean-square norm with one weight vector, else ``None``."""
+        if self.kind != "rmsnorm":
+            return None
+        return self.constants["weight"], self.constants["eps"]
 
     @property
     def residual(self):
@@ -160,7 +233,9 @@ class Norm(Part):
 
     def lazy(self, stream: Stream) -> "LazyNorm | None":
         """A :class:`LazyNorm` of the stream where a consumer's kernel could make this norm itself (the
-        norm says for which steps that is worth offering), else ``None``."""
+        norm says for which steps that is worth offering), else ``None``.  The :class:`LazyNorm` must name
+        its kind and carry that kind's constants: consumers fuse only the kinds they know and run every
+        other through :meth:`LazyNorm.value`."""
         return None
 
 

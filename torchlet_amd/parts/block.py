@@ -12,6 +12,8 @@ from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, Stream
 
 @BLOCKS.register("prenorm_residual")
 class PreNormBlock(Block):
+    graph_safe = True       # the arrangement itself; its four parts answer for themselves
+
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         self.mixer_norm = NORMS.build(spec.mixer_norm, dtype, device)
@@ -24,6 +26,11 @@ class PreNormBlock(Block):
             spec.ffn_norm_name: self.ffn_norm,
             spec.ffn_name: self.ffn,
         }
+
+    def parts(self):
+        yield self
+        for part in self._children.values():
+            yield from part.parts()
 
     def weight_specs(self):
         return {f"{name}.{k}": v for name, part in self._children.items() for k, v in part.weight_specs().items()}

@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import FEED_FORWARDS, FeedForward, LazyNorm, WeightSpec
+from .base import FEED_FORWARDS, KEEP_COMPUTE, FeedForward, LazyNorm, WeightSpec
 
 
 # The down product returns partial sums over slices of K where the kernel library finds that it
@@ -23,6 +23,8 @@ from .base import FEED_FORWARDS, FeedForward, LazyNorm, WeightSpec
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         self.hidden = spec.hidden
@@ -40,12 +42,12 @@ class SwiGLU(FeedForward):
     def load_weights(self, tensors):
         self.fused_gate = self.dtype == torch.bfloat16 and self.hidden % 8 == 0
         if self.fused_gate:
-            gate = self._place(tensors["gate_proj.weight"], "matrix")
-            up = self._place(tensors["up_proj.weight"], "matrix")
+            gate = self._place(tensors["gate_proj.weight"], KEEP_COMPUTE)
+            up = self._place(tensors["up_proj.weight"], KEEP_COMPUTE)
             self.gate_up = ops.interleave_gate_up(gate, up)
         else:
-            self.gate_up = self._place(torch.cat((tensors["gate_proj.weight"], tensors["up_proj.weight"]), dim=0), "matrix")
-        self.down = self._place(tensors["down_proj.weight"], "matrix")
+            self.gate_up = self._place(torch.cat((tensors["gate_proj.weight"], tensors["up_proj.weight"]), dim=0), KEEP_COMPUTE)
+        self.down = self._place(tensors["down_proj.weight"], KEEP_COMPUTE)
 
     takes_lazy_norm = True
 
@@ -53,10 +55,11 @@ class SwiGLU(FeedForward):
         lazy = h if isinstance(h, LazyNorm) else None
         if lazy is not None:
             # one row: the gate/up kernel makes the norm itself while its first weights arrive
-            if self.fused_gate:
+            rms = lazy.rmsnorm()          # the fused kernel makes a root-mean-square norm and no other
+            if self.fused_gate and rms is not None:
                 z = torch.empty((1, self.inter), dtype=self.dtype, device=lazy.residual.device)
                 residual_out = torch.empty_like(lazy.residual)
-                if ops.linear_swiglu_normed(lazy.residual, lazy.pending, lazy.norm.weight, lazy.norm.eps, residual_out,
+                if ops.linear_swiglu_normed(lazy.residual, lazy.pending, rms[0], rms[1], residual_out,
                                             self.gate_up, z):
                     lazy.done(residual_out)
                     return self._down(z, 1)

@@ -10,11 +10,13 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import NORMS, LazyNorm, Norm, Stream, WeightSpec
+from .base import KEEP_STORED, NORMS, LazyNorm, Norm, Stream, WeightSpec
 
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         self.dim = spec.dim
@@ -22,10 +24,10 @@ class RMSNorm(Norm):
         self.weight: torch.Tensor | None = None
 
     def weight_specs(self):
-        return {"weight": WeightSpec((self.dim,), role="vector", init="one_plus_normal")}
+        return {"weight": WeightSpec((self.dim,), keep=KEEP_STORED, init="one_plus_normal")}
 
     def load_weights(self, tensors):
-        self.weight = self._place(tensors["weight"], "vector")
+        self.weight = self._place(tensors["weight"], KEEP_STORED)
 
     def forward(self, stream: Stream, rows: torch.Tensor | None = None, gain: float = 1.0) -> torch.Tensor:
         n = stream.residual.shape[0] if rows is None else rows.numel()
@@ -38,5 +40,5 @@ class RMSNorm(Norm):
     def lazy(self, stream: Stream) -> LazyNorm | None:
         # one row in bfloat16: the kernels that read the norm's output can make it while their weights arrive
         if self.dtype == torch.bfloat16 and stream.residual.shape[0] == 1 and stream.residual.is_cuda:
-            return LazyNorm(self, stream)
+            return LazyNorm(self, stream, "rmsnorm", weight=self.weight, eps=self.eps)
         return None

@@ -17,6 +17,8 @@ from .base import POSITION_ENCODINGS, PositionEncoding
 
 @POSITION_ENCODINGS.register("rope_split_half")
 class RotaryEncoding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, spec, dtype, device):
         super().__init__(spec, dtype, device)
         if spec.head_dim % 2:

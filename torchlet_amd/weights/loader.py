@@ -10,7 +10,10 @@ tensor, every unexpected one and every wrong shape; the reference only logs thes
 
 Tensors are handed to the parts as stored: bfloat16 stays bfloat16 and a tensor stored in
 32-bit stays so, except that matrix-product operands take the engine's compute dtype and
-a 32-bit engine widens everything (see :class:`~torchlet_amd.parts.base.WeightSpec`).
+a 32-bit engine widens everything (the dtype policy of :class:`~torchlet_amd.parts.base.WeightSpec`).
+The engine's compute dtype itself follows the folder unless the caller names one
+(:func:`folder_dtype`): the reference types every parameter after its checkpoint tensor
+(/root/reference/src/torchlet/utils.py:18-38), so a folder stored in 32-bit runs in 32-bit.
 """
 from __future__ import annotations
 
@@ -90,9 +93,9 @@ def check_against(specs: dict[str, WeightSpec], source) -> None:
     def kind_ok(name, spec):
         if hasattr(source, "stored_dtype"):
             tag = source.stored_dtype(name)
-            return tag in (_INT_TAGS if spec.role == "table" else _FLOAT_TAGS)
+            return tag in (_INT_TAGS if spec.integer else _FLOAT_TAGS)
         t = source[name]
-        return (not t.is_floating_point()) if spec.role == "table" else t.is_floating_point()
+        return (not t.is_floating_point()) if spec.integer else t.is_floating_point()
 
     missing = [n for n, s in specs.items() if n not in source and not s.optional]
     unexpected = [n for n in source if n not in specs]
@@ -103,7 +106,7 @@ def check_against(specs: dict[str, WeightSpec], source) -> None:
             if got != tuple(s.shape):
                 wrong.append(f"{n}: stored {list(got)}, model wants {list(s.shape)}")
             elif not kind_ok(n, s):
-                wrong.append(f"{n}: stored element type does not fit a {s.role}")
+                wrong.append(f"{n}: stored element type does not fit {'an integer table' if s.integer else 'a floating-point tensor'}")
     if missing or unexpected or wrong:
         parts = []
         if missing:
@@ -125,3 +128,27 @@ def load_into(model, source) -> None:
 
 def load_folder(model, folder: str | Path) -> None:
     load_into(model, SafetensorsFolder(folder))
+
+
+_TAG_DTYPES = {"BF16": "bfloat16", "F32": "float32", "F16": "float16", "F64": "float64"}
+
+
+def folder_dtype(folder: str | Path, declared: str | None = None, probe: str | None = None) -> str:
+    """The compute dtype a model folder asks for: ``declared`` (its ``config.json``'s ``torch_dtype``) if
+    the folder says one, else the element type in which it stores ``probe`` (a tensor name; default: its
+    first floating-point tensor), as the reference types its parameters and its cache after the checkpoint's
+    tensors (/root/reference/src/torchlet/utils.py:18-38, v10_triton_paged_gqa/engine.py:58).  Only
+    ``bfloat16`` and ``float32`` engines are built; any other answer is refused by name."""
+    name = str(declared).replace("torch.", "").lower() if declared else None
+    if name is None:
+        source = SafetensorsFolder(folder)
+        names = [probe] if probe is not None and probe in source else list(source)
+        tags = [source.stored_dtype(n) for n in names if source.stored_dtype(n) in _FLOAT_TAGS]
+        if not tags:
+            raise WeightError(f"{folder} stores no floating-point tensor to take the compute dtype from")
+        name = _TAG_DTYPES[tags[0]]
+    name = {"bf16": "bfloat16", "fp32": "float32", "f32": "float32", "float": "float32"}.get(name, name)
+    if name not in ("bfloat16", "float32"):
+        raise ValueError(f"{folder} asks for a {name} engine; only bfloat16 and float32 are built "
+                         f"(name one of them as dtype= to convert the weights at load)")
+    return name

@@ -1,8 +1,9 @@
 """Random weights from a configuration and a seed.
 
-Law: matrices and biases ``N(0, 0.02)``, norm weights ``1 + N(0, 0.02)``, drawn in 32-bit
+Laws: matrices and biases ``N(0, 0.02)``, norm weights ``1 + N(0, 0.02)``; every tensor names its law
+(:data:`~torchlet_amd.parts.base.INIT_LAWS`, to which a part may add one), drawn in 32-bit
 from one ``torch.Generator(seed)`` in the order of the model's tensor declarations, then
-rounded to the storage dtype.  :func:`write_model_folder` writes ``config.json`` and
+rounded to the storage dtype (a tensor whose policy is 32-bit is stored in 32-bit).  :func:`write_model_folder` writes ``config.json`` and
 ``model.safetensors`` so that the engine and any other reader load identical values;
 :func:`random_tensors` makes the same kind of tensors directly on a device (for
 benchmark-size models, where a detour over a file would take minutes).
@@ -16,17 +17,14 @@ from safetensors.torch import save_file
 
 from ..config.base import ModelConfig
 from ..models.decoder import DecoderModel
+from ..parts.base import INIT_LAWS, KEEP_FLOAT32
 
 STD = 0.02
 
 
 def _draw(spec, gen: torch.Generator, device) -> torch.Tensor:
-    if spec.role == "table":
-        return torch.randint(0, 2 ** 15, spec.shape, generator=gen, device=device, dtype=torch.int32)
-    t = torch.randn(spec.shape, generator=gen, device=device, dtype=torch.float32) * STD
-    if spec.init == "one_plus_normal":
-        t = t + 1.0
-    return t
+    law = "random_table" if spec.integer and spec.init == "normal" else spec.init
+    return INIT_LAWS[law](spec.shape, gen, device, STD)
 
 
 def random_tensors(config: ModelConfig, seed: int, dtype: torch.dtype = torch.bfloat16, device="cpu") -> dict[str, torch.Tensor]:
@@ -39,7 +37,7 @@ def random_tensors(config: ModelConfig, seed: int, dtype: torch.dtype = torch.bf
         if spec.optional:
             continue
         t = _draw(spec, gen, device)
-        out[name] = t if spec.role == "table" else t.to(dtype)
+        out[name] = t if spec.integer else t.to(torch.float32 if spec.keep == KEEP_FLOAT32 else dtype)
     return out
 
 

@@ -18,14 +18,19 @@ recomputed from its own fields.  The same line carries
   steps) / its time, against the 8 TB/s of HBM3E (``frac``) and against the rate at which this GPU
   delivers memory to a kernel that only reads (``frac_measured``; ``measured`` holds that yardstick);
 * ``step_function``: the same decode step driven directly (no scheduler): what the scheduler costs;
-* ``prefill``: one 2048-token prompt in one step (tokens/s, ms, flops, ``frac`` of the dense matrix-core
-  peak of the dtype, ``frac_measured`` of the rate this repository's own large matrix product reaches);
+* ``prefill``: one 2048-token prompt in one step (tokens/s and ms as the mean of the timed runs, ``ms_best`` the
+  fastest of them, flops, ``frac`` of the dense matrix-core peak of the dtype, ``frac_measured`` of the rate this
+  repository's own large matrix product reaches);
 * ``points``: decode tokens/s at batch 1 and batch 64 through the engine; ``points_detail`` gives each
   point's ms per step, bytes per step and fractions.
 
-``--all`` adds the secondary workloads as ``extra``: Qwen2.5-14B sizes served through the scheduler
-(32 requests, prompts 128-4096, 128 new tokens, 512 tokens a step), and Qwen2.5-32B sizes (prefill of
-16384 tokens, decode at batch 1 on that context and at batch 16 on 4096-token contexts).
+``--all`` adds the secondary workloads as ``extra`` (``--extra 14b,32b,fp32`` picks among them): Qwen2.5-14B sizes
+served through the scheduler (32 requests, prompts 128-4096, 128 new tokens, 512 tokens a step); Qwen2.5-32B sizes
+through the engine: one request whose 16384-token prompt the scheduler prefills in portions of 2048 tokens and that
+then decodes 512 tokens greedily (``decode_32b_b1_ctx16384``, with the time of its prefill phase), and 16 requests
+with 4096-token prompts (``decode_32b_b16_ctx4096``), each with the bare step function on synthetic caches as a
+second figure (``step_function``), and the prefill of 16384 tokens as steps of the step function alone; and the same
+32B sizes in true 32-bit, all 64 layers (``fp32_32b``: decode at batch 1 through the engine, prefill of 2048 tokens).
 ``--workload serve`` prints the serving run alone as a line of its own.
 """
 from __future__ import annotations
@@ -79,7 +84,8 @@ def parse_args(argv=None):
     p.add_argument("--only", choices=["decode", "step", "prefill"], default=None,
                    help="run one part only (for profiling): the engine's decode steps at --batch, the bare step function's, "
                         "or the prefill")
-    p.add_argument("--all", action="store_true", help="add the secondary workloads (14B served, 32B prefill and decode)")
+    p.add_argument("--all", action="store_true", help="add the secondary workloads (14B served, 32B prefill and decode, 32B in 32-bit)")
+    p.add_argument("--extra", default=None, help="which secondary workloads, comma-separated: 14b, 32b, fp32 (implies --all)")
     return p.parse_args(argv)
 
 
@@ -87,14 +93,14 @@ def build(shape: str, layers: int, dtype: str):
     import torch
     from torchlet_amd.engine.loading import build_model
     from torchlet_amd.registry import config_class
-    from torchlet_amd.weights.random_init import random_tensors
+    from torchlet_amd.weights.random_init import RandomTensors
 
     d = dict(SHAPES[shape][1], num_hidden_layers=layers)
     cfg = config_class(d["architectures"][0]).from_dict(d)
     store = torch.bfloat16 if dtype == "bfloat16" else torch.float32
-    tensors = random_tensors(cfg, seed=2, dtype=store, device="cuda")
-    model = build_model(cfg, dtype, tensors=tensors)
-    del tensors
+    # every tensor drawn on the GPU as the model takes it: no second copy of the weights stands by
+    # (the 32B sizes in 32-bit are 131 GB of the 288)
+    model = build_model(cfg, dtype, tensors=RandomTensors(cfg, seed=2, dtype=store, device="cuda"))
     torch.cuda.empty_cache()
     return cfg, model
 
@@ -125,26 +131,32 @@ def random_prompts(vocab: int, count: int, length: int, seed: int = 0):
     return [torch.randint(0, vocab, (length,), generator=g).tolist() for _ in range(count)]
 
 
-def engine_decode(cfg, model, batch: int, steps: int, warmup: int, context: int, new_tokens: int) -> dict:
+def engine_decode(cfg, model, batch: int, steps: int, warmup: int, context: int, new_tokens: int, budget: int = PREFILL_BUDGET) -> dict:
     """``batch`` requests with ``context``-token random prompts through the whole engine: the prompts are
-    prefilled by the scheduler (portions under its token budget), then every step decodes one token for each
-    request.  ``warmup`` decode steps are left untimed (they capture the graphs), ``steps`` are timed.
-    No stop token; nobody may finish before the timed steps are over."""
+    prefilled by the scheduler (portions under its token budget ``budget``), then every step decodes one token for
+    each request.  The graphs of the decode steps are captured before the requests arrive; ``warmup`` decode steps
+    are left untimed, ``steps`` are timed.  No stop token; nobody may finish before the timed steps are over."""
     import torch
     from torchlet_amd.engine.config import EngineConfig
     from torchlet_amd.engine.loading import make_engine
     from torchlet_amd.engine.request import Request
 
     pages = batch * (-(-(context + new_tokens) // PAGE)) + 1
-    engine = make_engine(model, EngineConfig(page_size=PAGE, num_pages=pages, max_slots=batch, max_tokens_per_step=max(PREFILL_BUDGET, batch),
-                                             dtype="float32" if model.dtype == torch.float32 else "bfloat16", use_graphs=True,
-                                             lookahead=True, seed=0))
+    engine = make_engine(model, EngineConfig(page_size=PAGE, num_pages=pages, max_slots=batch, max_tokens_per_step=max(budget, batch),
+                                             use_graphs=True, lookahead=True, seed=0))
+    captured = engine.runner.warm_up(widths=[batch], max_len=context + new_tokens)     # ahead of need, as the Python entry point does
     reqs = [Request(prompt_tokens=p, max_new_tokens=new_tokens, temperature=0.0, stop_token_ids=frozenset())
             for p in random_prompts(cfg.vocab_size, batch, context)]
     engine.add_requests(reqs)
     finished = []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    prefill_steps = engine.steps
     while any(not r.output_tokens for r in reqs):          # the prefill phase (with decode tokens of those already through)
         finished += engine.step()
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    prefill_steps = engine.steps - prefill_steps
     ahead = max(len(r.output_tokens) for r in reqs)
     if ahead + warmup + steps >= new_tokens:
         raise SystemExit(f"bench.py: {warmup} + {steps} decode steps after a prefill phase in which a request already generated "
@@ -170,7 +182,9 @@ def engine_decode(cfg, model, batch: int, steps: int, warmup: int, context: int,
     mean_ctx = (ctx0 + ctx1) / 2.0 + 0.5      # keys a request's token attends to (its own included), averaged over the timed steps
     nbytes = decode_bytes(cfg, model, batch, mean_ctx)
     return {"batch": batch, "steps": steps, "ms_per_step": round(ms, 4), "tokens_per_s": round(batch * 1e3 / ms, 2),
-            "mean_context": round(mean_ctx, 1), "bytes_per_step": int(nbytes), "graph_replays": replays, "steps_ahead": ahead_steps}
+            "mean_context": round(mean_ctx, 1), "bytes_per_step": int(nbytes), "graph_replays": replays, "steps_ahead": ahead_steps,
+            "graphs_captured_ahead": captured, "prefill_phase_ms": round(prefill_s * 1e3, 2), "prefill_phase_steps": prefill_steps,
+            "prefill_phase_tokens": batch * context}
 
 
 def fill_context(runner, req_ids, context: int):
@@ -229,15 +243,16 @@ def step_function_decode(cfg, model, batch: int, steps: int, warmup: int, contex
             "mean_context": round(mean_ctx, 1), "bytes_per_step": int(decode_bytes(cfg, model, batch, mean_ctx))}
 
 
-def time_prefill(model, tokens: int, repeats: int = 3, context: int = 0):
-    """ms of one step that brings ``tokens`` prompt tokens (after ``context`` tokens fed in 2048-token steps)."""
+def time_prefill(model, tokens: int, repeats: int = 5, context: int = 0):
+    """(mean, best) ms of one step that brings ``tokens`` prompt tokens (after ``context`` tokens fed in 2048-token
+    steps) over ``repeats`` runs after one that warms up."""
     import torch
     from torchlet_amd.engine.batch import StepEntry
     from torchlet_amd.engine.loading import make_runner
 
     runner = make_runner(model, page_size=PAGE, num_pages=-(-(context + tokens) // PAGE) + 2, max_requests=1)
     prompt = random_prompts(model.spec.vocab_size, 1, context + tokens)[0]
-    best = float("inf")
+    times = []
     for i in range(repeats + 1):
         for a in range(0, context, 2048):
             runner.step([StepEntry("p", prompt[a:min(a + 2048, context)], [])])
@@ -248,10 +263,10 @@ def time_prefill(model, tokens: int, repeats: int = 3, context: int = 0):
         dt = (time.perf_counter() - t0) * 1e3
         runner.release("p")
         if i:                      # the first run warms up
-            best = min(best, dt)
+            times.append(dt)
     del runner
     torch.cuda.empty_cache()
-    return best
+    return sum(times) / len(times), min(times)
 
 
 def _best_ms(launch, rounds: int = 5, calls: int = 10) -> float:
@@ -341,27 +356,39 @@ def serve(cfg, model, args) -> dict:
     }
 
 
-def secondary(args) -> dict:
-    """The secondary workloads, each at its full layer count: 14B sizes served, 32B sizes prefilled and decoded."""
+def _with_roofline(r: dict) -> dict:
+    gbs = r["bytes_per_step"] / (r["ms_per_step"] * 1e-3) / 1e9
+    return dict(r, achieved_gbs=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 4))
+
+
+def secondary_14b(args) -> dict:
+    """14B sizes, all 48 layers, served: 32 requests, prompts 128-4096, 128 new tokens, 512 tokens a step."""
     import torch
-    out = {}
     cfg, model = build("14b", SHAPES["14b"][1]["num_hidden_layers"], args.dtype)
     a = argparse.Namespace(**vars(args))
     a.shape, a.requests, a.prompt_min, a.prompt_max, a.serve_new_tokens, a.portion = "14b", 32, 128, 4096, 128, 512
     s = serve(cfg, model, a)
-    out["serve_14b"] = {k: s[k] for k in ("value", "unit", "generated_tokens_per_s", "prompt_tokens", "generated_tokens", "seconds",
-                                           "engine_steps", "ms_per_step", "layers")}
     del model
     torch.cuda.empty_cache()
-    cfg, model = build("32b", SHAPES["32b"][1]["num_hidden_layers"], args.dtype)
-    tokens = 16384
-    # the long prompt in 2048-token steps, as the engine's budget would cut it: the sum of the steps' times
+    return {"serve_14b": {k: s[k] for k in ("value", "unit", "generated_tokens_per_s", "prompt_tokens", "generated_tokens", "seconds",
+                                            "engine_steps", "ms_per_step", "layers")}}
+
+
+def secondary_32b(args) -> dict:
+    """32B sizes, all 64 layers, through the engine: one request with a 16384-token prompt (prefilled by the
+    scheduler in portions of 2048 tokens) that decodes 512 tokens greedily, and 16 requests with 4096-token
+    prompts; beside each the bare step function on synthetic caches, and the long prefill as steps of the step
+    function alone."""
+    import torch
     from torchlet_amd.engine.batch import StepEntry
     from torchlet_amd.engine.loading import make_runner
+    out = {}
+    cfg, model = build("32b", SHAPES["32b"][1]["num_hidden_layers"], args.dtype)
+    tokens = 16384
     runner = make_runner(model, page_size=PAGE, num_pages=-(-tokens // PAGE) + 2, max_requests=1)
     prompt = random_prompts(cfg.vocab_size, 1, tokens)[0]
-    best = float("inf")
-    for rep in range(2):
+    times = []
+    for rep in range(3):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for a0 in range(0, tokens, 2048):
@@ -370,19 +397,55 @@ def secondary(args) -> dict:
         total = time.perf_counter() - t0
         runner.release("p")
         if rep:
-            best = min(best, total)
+            times.append(total)
     del runner
     torch.cuda.empty_cache()
+    mean, best = sum(times) / len(times), min(times)
     flops = sum(prefill_flops_step(cfg, 2048, a0) for a0 in range(0, tokens, 2048))
-    out["prefill_32b_16384"] = {"tokens": tokens, "steps_of": 2048, "ms": round(best * 1e3, 2), "value": round(tokens / best, 1),
-                                "flops": flops, "frac": round(flops / best / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12), 4),
-                                "layers": cfg.num_hidden_layers}
-    for name, batch, context, steps in (("decode_32b_b1_ctx16384", 1, 16384, 32), ("decode_32b_b16_ctx4096", 16, 4096, 32)):
-        r = step_function_decode(cfg, model, batch, steps, 4, context)
-        gbs = r["bytes_per_step"] / (r["ms_per_step"] * 1e-3) / 1e9
-        out[name] = dict(r, achieved_gbs=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 4), layers=cfg.num_hidden_layers)
+    out["prefill_32b_16384"] = {"tokens": tokens, "steps_of": 2048, "ms": round(mean * 1e3, 2), "ms_best": round(best * 1e3, 2), "runs": len(times),
+                                "value": round(tokens / mean, 1), "flops": flops,
+                                "frac": round(flops / mean / (MFMA_PEAK_TFLOPS[args.dtype] * 1e12), 4), "layers": cfg.num_hidden_layers}
+    # (name, requests, prompt tokens, new tokens, timed decode steps, token budget of a step)
+    for name, batch, context, new_tokens, steps, budget in (("decode_32b_b1_ctx16384", 1, 16384, 512, 480, 2048),
+                                                           ("decode_32b_b16_ctx4096", 16, 4096, 128, 96, 8192)):
+        r = _with_roofline(engine_decode(cfg, model, batch, steps, 8, context, new_tokens, budget=budget))
+        r["prefill_phase_flops"] = batch * sum(prefill_flops_step(cfg, min(2048, context - a0), a0) for a0 in range(0, context, 2048))
+        r["prefill_phase_tokens_per_s"] = round(r["prefill_phase_tokens"] / (r["prefill_phase_ms"] * 1e-3), 1)
+        r["step_function"] = _with_roofline(step_function_decode(cfg, model, batch, 32, 4, context))
+        r["layers"], r["new_tokens"], r["token_budget"] = cfg.num_hidden_layers, new_tokens, budget
+        out[name] = r
     del model
     torch.cuda.empty_cache()
+    return out
+
+
+def secondary_fp32_32b(args) -> dict:
+    """32B sizes in true 32-bit, all 64 layers (131 GB of weights): decode at batch 1 through the engine after a
+    2048-token prompt, and the prefill of 2048 tokens as one step."""
+    import torch
+    cfg, model = build("32b", SHAPES["32b"][1]["num_hidden_layers"], "float32")
+    r = _with_roofline(engine_decode(cfg, model, 1, 32, 4, 2048, 64, budget=2048))
+    pms, pbest = time_prefill(model, 2048, repeats=2)
+    flops = prefill_flops(cfg, 2048)
+    out = {"dtype": "fp32", "layers": cfg.num_hidden_layers, "weight_bytes": int(decode_bytes(cfg, model, 1, 0)),
+           "decode_b1": r,
+           "prefill": {"value": round(2048 * 1e3 / pms, 1), "tokens": 2048, "ms": round(pms, 2), "ms_best": round(pbest, 2), "runs": 2,
+                       "flops": flops, "frac": round(flops / (pms * 1e-3) / (MFMA_PEAK_TFLOPS["float32"] * 1e12), 4)}}
+    del model
+    torch.cuda.empty_cache()
+    return {"fp32_32b": out}
+
+
+def secondary(args) -> dict:
+    """The secondary workloads, each at its full layer count."""
+    which = [w.strip() for w in (args.extra or "14b,32b,fp32").split(",") if w.strip()]
+    parts = {"14b": secondary_14b, "32b": secondary_32b, "fp32": secondary_fp32_32b}
+    unknown = [w for w in which if w not in parts]
+    if unknown:
+        raise SystemExit(f"bench.py: --extra knows 14b, 32b and fp32, not {', '.join(unknown)}")
+    out = {}
+    for w in which:
+        out.update(parts[w](args))
     return out
 
 
@@ -415,10 +478,10 @@ def main(argv=None) -> int:
     peak_tflops = MFMA_PEAK_TFLOPS[args.dtype]
 
     def prefill_point(gemm_tflops=None):
-        pms = time_prefill(model, ptokens)
+        pms, pbest = time_prefill(model, ptokens)
         flops = prefill_flops(cfg, ptokens)
-        point = {"value": round(ptokens * 1e3 / pms, 1), "tokens": ptokens, "ms": round(pms, 3), "flops": flops,
-                 "frac": round(flops / (pms * 1e-3) / (peak_tflops * 1e12), 4)}
+        point = {"value": round(ptokens * 1e3 / pms, 1), "tokens": ptokens, "ms": round(pms, 3), "ms_best": round(pbest, 3), "runs": 5,
+                 "flops": flops, "frac": round(flops / (pms * 1e-3) / (peak_tflops * 1e12), 4)}
         if gemm_tflops:
             point["frac_measured"] = round(flops / (pms * 1e-3) / (gemm_tflops * 1e12), 4)
         return point
@@ -486,7 +549,7 @@ def main(argv=None) -> int:
                                       "frac": round(gbs / HBM_PEAK_GBS, 4), "frac_measured": round(gbs / stream_gbs, 4)}
         result["points"] = points
         result["points_detail"] = detail
-    if args.all:
+    if args.all or args.extra:
         del model
         torch.cuda.empty_cache()
         result["extra"] = secondary(args)

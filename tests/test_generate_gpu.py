@@ -50,6 +50,60 @@ def test_greedy_generation_through_the_entry_point(model_folders, dtype):
     assert llm.runner.cache.live_requests() == []
 
 
+def test_a_folder_stored_in_32_bit_gives_a_32_bit_engine(tmp_path):
+    """No dtype named: the engine runs in the dtype the folder is stored in, as the reference types its parameters
+    and its cache after the checkpoint (/root/reference/src/torchlet/utils.py:18-38,
+    v10_triton_paged_gqa/engine.py:58).  The folder's config.json has no ``torch_dtype``: what it stores decides."""
+    from torchlet_amd import LLM
+    from torchlet_amd.engine.batch import StepEntry
+    folder = tiny_models.write("B", tmp_path, dtype=torch.float32)
+    assert "torch_dtype" not in json.loads((folder / "config.json").read_text())
+    cfg, w = plain_qwen2.load_folder(folder)
+    llm = LLM(str(folder), max_decode_slots=2, kv_block_size=8, use_graphs=False)
+    assert llm.engine_config.dtype == "float32" and llm.model.dtype == torch.float32
+    assert llm.model.blocks[0].mixer.w_qkv.dtype == torch.float32 and llm.model.embed.dtype == torch.float32
+    assert {t.dtype for g in llm.runner.cache.groups for t in g.tensors} == {torch.float32}
+    prompt = list(scenarios.make_requests(cfg.vocab, [29], seed=3).values())[0]
+    assert llm.generate([prompt], max_new_tokens=8)[0] == plain_qwen2.greedy(cfg, w, prompt, 8)
+    logits = llm.runner.step([StepEntry("x", prompt, list(range(len(prompt))))]).cpu()
+    llm.runner.release("x")
+    torch.testing.assert_close(logits.double(), plain_qwen2.forward(cfg, w, prompt), **scenarios.FP32_TOL)
+    # the same folder with bfloat16 named: converted at load
+    llm16 = LLM(str(folder), max_decode_slots=2, kv_block_size=8, dtype="bfloat16", use_graphs=False)
+    assert llm16.model.dtype == torch.bfloat16 and llm16.model.embed.dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graphs_are_captured_before_the_first_request(model_folders, dtype):
+    """``LLM`` captures the graph of every (batch width, context bucket) its configuration can reach when it is built
+    (the reference captures its one shape inside its first decode step,
+    /root/reference/src/torchlet/v10_triton_paged_gqa/engine.py:137-176): every decode step, the first one
+    included, is a replay; no step stops to capture; what is generated is what the eager engine generates."""
+    from torchlet_amd import LLM
+    cfg, w = plain_qwen2.load_folder(model_folders["B"])            # 256 positions in pages of 8: one bucket of 32 pages
+    llm = LLM(str(model_folders["B"]), max_decode_slots=4, kv_block_size=8, dtype=dtype, use_graphs=True)
+    assert llm.runner.use_graphs and llm.graphs_captured == 3 and sorted(llm.runner._graphs) == [(1, 32), (2, 32), (4, 32)]
+    assert llm.runner.graph_replays == 0
+    prompts = list(scenarios.make_requests(cfg.vocab, [21, 6, 40], seed=5).values())
+    one = llm.generate([prompts[0]], max_new_tokens=9)[0]
+    assert llm.runner.graph_replays >= 8                               # eight decode steps, the first of them too
+    replays = llm.runner.graph_replays
+    three = llm.generate(prompts, max_new_tokens=12)
+    assert llm.runner.graph_replays >= replays + 11
+    assert len(llm.runner._graphs) == 3 and all(g.graph is not None for g in llm.runner._graphs.values())   # nothing captured later
+    eager = LLM(str(model_folders["B"]), max_decode_slots=4, kv_block_size=8, dtype=dtype, use_graphs=False)
+    assert eager.graphs_captured == 0
+    assert eager.generate([prompts[0]], max_new_tokens=9)[0] == one and eager.generate(prompts, max_new_tokens=12) == three
+    if dtype == "float32":
+        assert one == plain_qwen2.greedy(cfg, w, prompts[0], 9)
+    # a longer model in more buckets, sized by max_model_len
+    cfgd = json.loads((model_folders["D"] / "config.json").read_text())         # 400 positions, pages of 8
+    llm = LLM(str(model_folders["D"]), max_decode_slots=2, kv_block_size=8, dtype=dtype, use_graphs=True)
+    assert sorted(llm.runner._graphs) == [(w_, b) for w_ in (1, 2) for b in (32, 50)] and cfgd["max_position_embeddings"] == 400
+    llm = LLM(str(model_folders["D"]), max_decode_slots=2, kv_block_size=8, dtype=dtype, use_graphs=True, max_model_len=200)
+    assert sorted(llm.runner._graphs) == [(1, 25), (2, 25)]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("graphs", [False, True])
 def test_decode_steps_enqueued_ahead_of_their_tokens_generate_the_same(model_folders, dtype, graphs):

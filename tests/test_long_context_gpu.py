@@ -189,6 +189,31 @@ def test_prompt_attention_at_benchmark_lengths(ops, nh, nkv, hd, page, window, n
     _check_rows(out.double().view(new, nh, hd), ref, cache.v[0], f"{new} tokens on {ctx}")
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page,window,new,ctx", [
+    (28, 4, 128, 8, 0, 512, 20000),            # 2564 pages: more than the 128-row kernel keeps in shared memory
+    (8, 2, 96, 16, 0, 512, 5000),              # a head size the 128-row kernel is not built for
+    (6, 3, 112, 4, 3000, 300, 9000),           # pages of 4 tokens, a window
+])
+def test_prompt_attention_in_tiles_of_64_rows_at_real_lengths(ops, nh, nkv, hd, page, window, new, ctx):
+    """The 64-row kernel for prompt portions is what serves sequences of more than 2048 pages and head sizes other
+    than 64 and 128 from contexts of 4096 tokens on (``parts/attention.py``): here at those lengths, against the
+    float64 formula, with NaN in every place of the cache that holds no key."""
+    assert not ops.prompt_attention_fits(torch.bfloat16, hd, page, -(-(ctx + new) // page))      # the case the mixer sends here
+    total = ctx + new
+    cache = _Paged([total], nkv, hd, page, seed=new + ctx)
+    g = torch.Generator(device="cuda").manual_seed(10)
+    q = torch.randn((new, nh * hd), generator=g, device="cuda").to(torch.bfloat16)
+    tq = ops.prefill_attention_tile_tokens(nh, nkv)
+    tok0 = list(range(0, new, tq))
+    out = torch.full((new, nh * hd), float("nan"), dtype=torch.bfloat16, device="cuda")
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")
+    print(f"{new} new tokens on {ctx}: {len(tok0)} tiles of {tq} tokens, {cache.table.shape[1]} pages", flush=True)
+    ops.paged_attention_prefill(q, out, cache.kp, cache.vp, cache.table, i32([0, new]), i32([ctx]), i32([0] * len(tok0)), i32(tok0),
+                                len(tok0), tq, nh, nkv, hd, page, window, 1.0 / math.sqrt(hd))
+    ref = _reference(q.view(new, nh, hd), cache.k[0], cache.v[0], window)
+    _check_rows(out.double().view(new, nh, hd), ref, cache.v[0], f"{new} tokens on {ctx}")
+
+
 # ------------------------------------------------------------------------ engine level
 
 LONG = {
@@ -306,4 +331,58 @@ def test_every_split_at_long_contexts(long_model, dtype):
             assert err <= 1.25 * rms16
         del runner
     del model
+    torch.cuda.empty_cache()
+
+
+# A sequence of more pages than the 128-row prompt kernel holds: with pages of 8 tokens its 2048 pages are 16 384 tokens.
+BEYOND = dict(architectures=["Qwen2ForCausalLM"], vocab_size=170, hidden_size=128, num_hidden_layers=2,
+              num_attention_heads=4, num_key_value_heads=2, head_dim=64, intermediate_size=176,
+              max_position_embeddings=40960, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=True)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_portions_that_cross_the_edge_of_2048_pages(dtype):
+    """One request of 16 884 tokens in pages of 8: portions of 2048 tokens while the sequence has at most 2048 pages
+    (the 128-row kernel in bfloat16), then portions of 1500, 1000 and 32 tokens, the second of which takes the
+    sequence past 16 384 tokens (from there on the 64-row kernel), then 16 tokens one by one.  Logits of the last 64
+    tokens of every early portion and of every token from position 14 336 on, against the plain implementation."""
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import build_model, make_runner
+    from torchlet_amd.kernels import ops
+    from torchlet_amd.registry import ARCHITECTURES
+    from torchlet_amd.weights.random_init import random_tensors
+    page, sizes = 8, [2048] * 7 + [1500, 1000, 32] + [1] * 16
+    config = ARCHITECTURES["Qwen2ForCausalLM"].from_dict(BEYOND)
+    tensors = random_tensors(config, seed=23, dtype=torch.bfloat16, device="cuda")
+    for k in tensors:
+        if "q_proj" in k or "k_proj" in k:
+            tensors[k] = (tensors[k].float() * SHARPEN).to(torch.bfloat16)
+    requests = scenarios.make_requests(BEYOND["vocab_size"], [sum(sizes)], seed=8)
+    tokens = requests["r0"]
+    expected, noise, noise16, rms16 = scenarios.bounds_from_plain(plain.PlainConfig(BEYOND), tensors, requests)
+    print(f"32-bit noise {noise:.3e}; bfloat16 roundings move the logits by {noise16:.3e} at most, {rms16:.3e} rms", flush=True)
+    tol = dict(atol=8.0 * noise, rtol=2e-5) if dtype == "float32" else dict(atol=2 * noise16, rtol=0.0)
+    steps, done, kernels = [], 0, []
+    for n in sizes:
+        want = list(range(n)) if done >= 14336 else list(range(n - 64, n))
+        steps.append(dict(entries=[dict(id="r0", tokens=tokens[done:done + n], want=want)], end=["r0"] if done + n == len(tokens) else []))
+        done += n
+        kernels.append(ops.prompt_attention_fits(torch.bfloat16, 64, page, -(-done // page)))
+    assert kernels[:8] == [True] * 8 and not any(kernels[8:])          # the step of 1000 tokens is the first past the edge
+    steps = scenarios.number(steps)
+    model = build_model(config, dtype, tensors=tensors)
+    runner = make_runner(model, page_size=page, num_pages=-(-len(tokens) // page) + 2, max_requests=1)
+    for g in runner.cache.groups:
+        for plane in g.tensors:
+            plane.fill_(float("nan"))
+            plane[:, 0] = 0
+    out = {}
+    for s in steps:
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        out[s["step"]] = logits.cpu().numpy()
+        for r in s["end"]:
+            runner.release(r)
+    runner.cache.check()
+    scenarios.check(steps, out, expected, tol, what=f"{dtype}, past 2048 pages")
+    del runner, model, tensors
     torch.cuda.empty_cache()

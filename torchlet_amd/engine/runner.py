@@ -169,25 +169,25 @@ class ModelRunner:
         dg.graph = graph
 
     def warm_up(self, widths=None, max_len: int | None = None) -> int:
-        """Capture, ahead of need, the graph of every (batch width, context bucket) that decode steps of up to
-        ``max(widths)`` requests (default: as many as the cache has slots) and sequences of up to ``max_len``
-        tokens (default: the engine's limit) can ask for, so that no serving step stops to capture one
-        (the reference captures its one shape inside its first decode step,
-        /root/reference/src/torchlet/v10_triton_paged_gqa/engine.py:137-176).  Each shape runs once eagerly
-        on padding rows alone, which write to no page and to no request's state, and is then recorded.
-        Returns the number of graphs captured; nothing happens without ``use_graphs``."""
+        """Capture, ahead of need, the graphs that decode steps can ask for, so that no serving step stops to
+        capture one (the reference captures its one shape inside its first decode step,
+        /root/reference/src/torchlet/v10_triton_paged_gqa/engine.py:137-176): for every batch width (``widths``:
+        numbers of requests, each rounded up to the width its steps run at; default: every width up to the cache's
+        slots) every context bucket of sequences of up to ``max_len`` tokens (default: the engine's limit).  Each
+        shape runs once eagerly on padding rows alone, which write to no page and to no request's state, and is
+        then recorded.  Returns the number of graphs captured; nothing happens without ``use_graphs``."""
         if not self.use_graphs:
             return 0
         cache = self.cache
         if widths is None:
-            widths = [cache.max_requests]
-        top = min(_next_pow2(max(widths)), _next_pow2(self.max_graph_width))
+            top = min(_next_pow2(cache.max_requests), _next_pow2(self.max_graph_width))
+            widths = [1 << i for i in range(top.bit_length())]
+        widths = sorted({_next_pow2(int(w)) for w in widths if 0 < int(w) <= self.max_graph_width})
         max_len = self.max_positions if max_len is None else min(max_len, self.max_positions)
         most_blocks = _next_pow2(-(-max_len // cache.page_size))
         buckets = sorted({self._bucket(1 << i) for i in range(most_blocks.bit_length())})   # of 1, 2, 4, ... pages
         captured = 0
-        width = 1
-        while width <= top:
+        for width in widths:
             for bucket in buckets:
                 dg = self._decode_graph((width, bucket))
                 if dg.graph is None:
@@ -196,7 +196,6 @@ class ModelRunner:
                     self.model.forward(dg.ctx, self.caches)       # eager once: kernels loaded, buffers of this shape known
                     self._capture(dg)
                     captured += 1
-            width *= 2
         torch.cuda.synchronize()
         return captured
 

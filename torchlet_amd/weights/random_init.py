@@ -10,6 +10,7 @@ benchmark-size models, where a detour over a file would take minutes).
 """
 from __future__ import annotations
 
+from collections.abc import Mapping
 from pathlib import Path
 
 import torch
@@ -39,6 +40,40 @@ def random_tensors(config: ModelConfig, seed: int, dtype: torch.dtype = torch.bf
         t = _draw(spec, gen, device)
         out[name] = t if spec.integer else t.to(torch.float32 if spec.keep == KEEP_FLOAT32 else dtype)
     return out
+
+
+class RandomTensors(Mapping):
+    """``name -> tensor`` like :func:`random_tensors`, but every tensor is drawn when it is asked for and not kept,
+    from a generator of its own (seeded by ``seed`` and the tensor's place in the declarations), so that a model far
+    larger than half the GPU's memory can be filled without a second copy of its weights standing by.  Shapes and
+    element types can be asked for without drawing (``shape``, ``stored_dtype``, as of a folder of safetensors)."""
+
+    def __init__(self, config: ModelConfig, seed: int, dtype: torch.dtype = torch.bfloat16, device="cpu"):
+        model = DecoderModel(config.to_spec(), torch.float32, "cpu")
+        self._specs = {n: s for n, s in model.weight_specs().items() if not s.optional}
+        self._index = {n: i for i, n in enumerate(self._specs)}
+        self.seed, self.dtype, self.device = int(seed), dtype, device
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        spec = self._specs[name]
+        gen = torch.Generator(device=self.device).manual_seed(self.seed * 1_000_003 + self._index[name])
+        t = _draw(spec, gen, self.device)
+        return t if spec.integer else t.to(torch.float32 if spec.keep == KEEP_FLOAT32 else self.dtype)
+
+    def __iter__(self):
+        return iter(self._specs)
+
+    def __len__(self):
+        return len(self._specs)
+
+    def shape(self, name: str) -> tuple[int, ...]:
+        return tuple(self._specs[name].shape)
+
+    def stored_dtype(self, name: str) -> str:
+        if self._specs[name].integer:
+            return "I32"
+        kept32 = self._specs[name].keep == KEEP_FLOAT32 or self.dtype == torch.float32
+        return "F32" if kept32 else {torch.bfloat16: "BF16", torch.float16: "F16"}[self.dtype]
 
 
 def write_model_folder(config: ModelConfig, seed: int, folder: str | Path, dtype: torch.dtype = torch.bfloat16) -> Path:

@@ -18,6 +18,7 @@
 // treats the dimensions from hd up to TL_HEAD_DIM as zeros that are neither read nor written; the
 // matrix-core kernels are for hd == TL_HEAD_DIM.
 #include "common.h"
+#include <type_traits>
 
 #ifndef TL_HEAD_DIM
 #error "compile with -DTL_HEAD_DIM=<head size>"
@@ -834,6 +835,7 @@ static void launch_merge(const void* part_o, const void* part_ml, void* out, int
 #define ATQ_KBYTES (ATQ_KEYS * AT_HD * 2)
 #define ATQ_STAGE (2 * ATQ_KBYTES)                 // keys, then values
 #define ATQ_SMEM (ATQ_STAGES * ATQ_STAGE + ATM_BT_MAX * 4)
+#define ATQ_SLACK 8.f               // powers of two a row's scores may rise above its reference before it is moved
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 // 16 bytes per lane from memory straight into shared memory at lds_addr + 16 * lane.  Issued as
@@ -935,35 +937,56 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     constexpr int K_INSTR = ATQ_KBYTES / 1024 / 4;          // per wave
     constexpr int VDI = 1024 / ATQ_VROW;                    // value rows (d) per load instruction (8 or 16)
     static_assert(K_INSTR >= 1 && 2 * K_INSTR * (ATQ_STAGES - 2) < 64, "loads per wave and step");
-    // what does not change from step to step, per load instruction of this lane
-    int k_local[K_INSTR], k_piece[K_INSTR], v_key[K_INSTR], v_row[K_INSTR];
+    // What does not change from step to step is worked out here, per load instruction of this lane: a step's first key
+    // is a multiple of ATQ_KEYS, and pages are powers of two, so key kbase + x (x < ATQ_KEYS) lies in block
+    // (kbase >> shift) + (x >> shift) at place (kbase & pmask) + (x & pmask) of its page (of the two uniform parts the
+    // second is zero for pages of up to ATQ_KEYS keys, of the two lane parts the first is zero for longer ones).  A
+    // step then costs a lane one look-up of a page and one multiply-add per address.  (With all of it computed in the
+    // step, the addresses were a quarter of the loop's vector instructions.)
+    const bf16_t* k_src[K_INSTR];              // K row of key x, this lane's piece, in page 0
+    const bf16_t* v_src[K_INSTR];              // V^T row d, this lane's eight keys, in page 0
+    int k_blk[K_INSTR];                        // x >> shift
     unsigned k_dst[K_INSTR];
+    int v_blk;                                 // the same for every value load of a lane (its piece's slot depends on d / 2 mod 8 only)
 #pragma unroll
     for (int j = 0; j < K_INSTR; ++j) {
         const int ii = wave + 4 * j;
-        k_local[j] = KPI * ii + lane / KPP;
-        k_piece[j] = atq_key_slot(lane % KPP, k_local[j]) * 8;       // exclusive-or is its own inverse
+        const int kx = KPI * ii + lane / KPP;
+        k_blk[j] = kx >> shift;
+        k_src[j] = kp + kvh_off + (kx & pmask) * AT_HD + atq_key_slot(lane % KPP, kx) * 8;       // exclusive-or is its own inverse
         const int d = VDI * ii + lane / ATQ_VPP;
-        v_key[j] = 8 * atq_value_slot(lane % ATQ_VPP, d);            // first of the piece's eight keys
-        v_row[j] = kvh_off + d * page;
+        const int vx = 8 * atq_value_slot(lane % ATQ_VPP, d);           // first of the piece's eight keys
+        if (j == 0) v_blk = vx >> shift;
+        v_src[j] = vp + kvh_off + d * page + (vx & pmask);
         k_dst[j] = __builtin_amdgcn_readfirstlane(ii * 1024);
     }
-    const int key_last8 = (key_hi - 1) & ~7;
-    auto request_step = [&](int st, int buf) {
+    const int blk_last = blk_n - 1;
+    // (a block beyond the sequence's last is read as the last: the step that holds the sequence's end may reach past
+    // its last page; those keys' scores are masked and their values cleared below)
+    auto request = [&](int st, int buf, auto long_pages) {
         const int kbase = st * ATQ_KEYS;
         const unsigned sb = lds_base + buf * ATQ_STAGE;
+        const int ub = (kbase >> shift) - blk0;                          // uniform: the step's first block in bt_s
+        const int uin = long_pages ? kbase & pmask : 0;                  // uniform: its first key's place in that block's page
 #pragma unroll
         for (int j = 0; j < K_INSTR; ++j) {
-            const int key = min(kbase + k_local[j], key_hi - 1);
-            const int pg = bt_s[(key >> shift) - blk0];
-            attn_load_to_lds(kp + ((size_t)pg * kv_stride + kvh_off + (key & pmask) * AT_HD + k_piece[j]), sb + k_dst[j]);
+            const int pg = bt_s[min(ub + k_blk[j], blk_last)];
+            const bf16_t* src = k_src[j] + (size_t)(unsigned)pg * kv_stride;
+            if (long_pages) src += uin * AT_HD;
+            attn_load_to_lds(src, sb + k_dst[j]);
         }
+        const int pg = bt_s[min(ub + v_blk, blk_last)];
 #pragma unroll
         for (int j = 0; j < K_INSTR; ++j) {
-            const int key = min(kbase + v_key[j], key_last8);
-            const int pg = bt_s[(key >> shift) - blk0];
-            attn_load_to_lds(vp + ((size_t)pg * kv_stride + v_row[j] + (key & pmask)), sb + ATQ_KBYTES + k_dst[j]);
+            const bf16_t* src = v_src[j] + (size_t)(unsigned)pg * kv_stride;
+            if (long_pages) src += uin;
+            attn_load_to_lds(src, sb + ATQ_KBYTES + k_dst[j]);
         }
+    };
+    const bool long_pages = page > ATQ_KEYS;                              // (uniform)
+    auto request_step = [&](int st, int buf) {
+        if (long_pages) request(st, buf, std::true_type{});
+        else request(st, buf, std::false_type{});
     };
 
     const float scale2 = a.scale * 1.44269504088896341f;
@@ -1025,16 +1048,15 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
                 }
             }
             // ---- mask, maximum, probabilities.  Element (kb, 4 q + v) of this lane is key
-            // kbase + 32 kb + 16 (q / 2) + 8 h + 4 (q % 2) + v of row lr.
+            // kbase + 32 kb + 16 (q / 2) + 8 h + 4 (q % 2) + v of row lr.  The maximum is taken of the scores as
+            // they come out of the product; the factor on them (positive: the host checks) goes into the
+            // exponent's argument, one multiply-add per score.
             float mloc = -INFINITY;
             if (kbase + ATQ_KEYS - 1 <= w_pos_min && kbase >= w_lo_max) {
 #pragma unroll
                 for (int kb = 0; kb < ATQ_KB; ++kb)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        sc[kb][v] *= scale2;
-                        mloc = fmaxf(mloc, sc[kb][v]);
-                    }
+                    for (int v = 0; v < 16; ++v) mloc = fmaxf(mloc, sc[kb][v]);
             } else {
 #pragma unroll
                 for (int kb = 0; kb < ATQ_KB; ++kb)
@@ -1043,31 +1065,35 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
                         const int q = e >> 2, v = e & 3;
                         const int key = kbase + 32 * kb + 16 * (q >> 1) + 8 * h + 4 * (q & 1) + v;
                         const bool seen = row_ok && key <= r_pos && key >= r_lo;
-                        sc[kb][e] = seen ? sc[kb][e] * scale2 : -INFINITY;
+                        sc[kb][e] = seen ? sc[kb][e] : -INFINITY;
                         mloc = fmaxf(mloc, sc[kb][e]);
                     }
             }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TL_WAVE));
-            const float m_new = fmaxf(m, mloc);
-            const float alpha = (m == -INFINITY) ? 0.f : fast_exp2(m - m_new);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;     // nothing seen yet: every score is -inf
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TL_WAVE)) * scale2;
+            // m is the row's reference for the exponents, not its running maximum: it moves only when some row of
+            // the wave has a score more than ATQ_SLACK (in powers of two) above its reference, so most steps rescale
+            // nothing; until then probabilities are up to 2^ATQ_SLACK instead of up to 1, which 32-bit sums and the
+            // bfloat16 operand of the second product hold as exactly as before, and the quotient at the end is the same.
+            if (__any(mloc > m + ATQ_SLACK)) {
+                const float m_new = fmaxf(m, mloc);
+                const float alpha = (m == -INFINITY) ? 0.f : fast_exp2(m - m_new);      // 1 for a row that stays
+                m = m_new;
+                l *= alpha;
+#pragma unroll
+                for (int b = 0; b < AT_HD / 32; ++b) acc[b] *= alpha;
+            }
+            const float m_use = (m == -INFINITY) ? 0.f : -m;           // nothing seen yet: every score is -inf
             FragK pf[2 * ATQ_KB];
             float psum = 0.f;
 #pragma unroll
             for (int kb = 0; kb < ATQ_KB; ++kb)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const float p = fast_exp2(sc[kb][e] - m_use);
+                    const float p = fast_exp2(__builtin_fmaf(sc[kb][e], scale2, m_use));
                     psum += p;
                     pf[2 * kb + (e >> 3)].v[e & 7] = (__bf16)p;
                 }
-            l = l * alpha + psum;
-            const bool moved = __any(m_new != m);
-            m = m_new;
-            if (moved) {
-#pragma unroll
-                for (int b = 0; b < AT_HD / 32; ++b) acc[b] *= alpha;
-            }
+            l += psum;
             // ---- values
 #pragma unroll
             for (int c4 = 0; c4 < 2 * ATQ_KB; ++c4)
@@ -1143,6 +1169,7 @@ extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out,
 #if AT_HD == 64 || AT_HD == 128
     TL_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: heads %d not a multiple of kv heads %d", heads, kv_heads);
     TL_REQUIRE(page >= 8 && (page & (page - 1)) == 0 && tq > 0 && window >= 0, "attention_prompt: pages of 8, 16, 32, ... tokens, not %d", page);
+    TL_REQUIRE(scale > 0.f, "attention_prompt: the factor on the scores must be positive (the maximum is taken before it is applied), not %g", (double)scale);
     // used_blocks: the most block-table entries any request of the step uses (its length in pages)
     TL_REQUIRE(bt_stride > 0 && used_blocks > 0 && used_blocks <= ATM_BT_MAX,
                "attention_prompt: sequences of up to %d pages, not %d", ATM_BT_MAX, used_blocks);

@@ -619,12 +619,12 @@ PROMPT_ATTENTION_HEAD_DIMS = (64, 128)
 PROMPT_ATTENTION_MAX_BLOCKS = 2048     # pages of a sequence whose block-table entries a work-group keeps in shared memory
 
 
-def prompt_attention_fits(dtype: torch.dtype, head_dim: int, page_size: int, max_blocks: int = 0) -> bool:
+def prompt_attention_fits(dtype: torch.dtype, head_dim: int, page_size: int, max_blocks: int = 0, scale: float = 1.0) -> bool:
     """Whether :func:`paged_attention_prompt` is built for this case: bfloat16, head size 64 or
     128, pages of 8, 16, 32, ... tokens, sequences of up to 2048 pages (``max_blocks``: the
-    longest sequence of the step in pages)."""
+    longest sequence of the step in pages), a positive factor on the scores."""
     return (dtype == torch.bfloat16 and head_dim in PROMPT_ATTENTION_HEAD_DIMS and page_size >= 8
-            and page_size & (page_size - 1) == 0 and max_blocks <= PROMPT_ATTENTION_MAX_BLOCKS)
+            and page_size & (page_size - 1) == 0 and max_blocks <= PROMPT_ATTENTION_MAX_BLOCKS and scale > 0)
 
 
 def prompt_attention_tile_tokens(num_heads: int, num_kv_heads: int) -> int:

@@ -221,7 +221,7 @@ class GQAttention(Mixer):
         k_plane, v_plane, table = self._cache_views(ctx, cache)
         out = torch.empty((T, self.q_width), dtype=self.dtype, device=q.device)
         common = (self.heads, self.kv_heads, self.head_dim, cache.page_size, self.window or 0, self.scale)
-        rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size, -(-ctx.max_total_len // cache.page_size))
+        rows128 = (ops.prompt_attention_fits(self.dtype, self.head_dim, cache.page_size, -(-ctx.max_total_len // cache.page_size), self.scale)
                    and ctx.max_new_tokens >= _PORTION_MIN_TOKENS)
         portions = (self.dtype == torch.bfloat16 and self.head_dim <= ops.PREFILL_ATTENTION_MAX_HEAD_DIM
                     and self.head_dim % 16 == 0 and cache.page_size % 4 == 0 and ctx.max_new_tokens >= _PORTION_MIN_TOKENS

@@ -123,7 +123,7 @@ template <int MR>
 __global__ __launch_bounds__(256) void gemv_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                        const void* __restrict__ bias, int bias_f32,
                                                        float* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
-    constexpr int KC = MR > 8 ? 512 : 1024;        // 32 KB of x at most
+    constexpr int KC = MR >= 8 ? 512 : 1024;       // 32 KB of x at most; at eight rows the shorter chunk keeps the kernel to 128 registers
     __shared__ float4 xs[MR][KC / 4];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int n0 = blockIdx.x * GV_ROWS + wave * 2;
@@ -133,6 +133,21 @@ __global__ __launch_bounds__(256) void gemv_f32_kernel(const float* __restrict__
 #pragma unroll
     for (int m = 0; m < MR; ++m) acc[m][0] = acc[m][1] = 0.f;
 
+    // A lane's pieces of its two rows are lane, lane + 64, ...: IPC of them per chunk of x.  The pieces of the next
+    // chunk are requested while this chunk's are multiplied, so the stream of weights does not stop at the barriers
+    // around the copy of x (with the requests made inside a chunk only, every chunk began with an empty pipe: the
+    // 7B's decode step in 32-bit 9.5 -> see the measurements).  A piece beyond the row's end is fetched from the
+    // row's last piece and cleared.
+    constexpr int IPC = KC / 4 / 64;
+    const int all = K / 4;
+    float4 ra[IPC], rb[IPC];
+    auto fetch = [&](int j, int c) {
+        const int cc = min(c, all - 1);
+        ra[j] = *(const float4*)(wa + 4 * cc);
+        rb[j] = *(const float4*)(wb + 4 * cc);
+    };
+#pragma unroll
+    for (int j = 0; j < IPC; ++j) fetch(j, lane + 64 * j);
     for (int k0 = 0; k0 < K; k0 += KC) {
         const int pieces = min(KC, K - k0) / 4;
         __syncthreads();
@@ -143,16 +158,21 @@ __global__ __launch_bounds__(256) void gemv_f32_kernel(const float* __restrict__
             xs[m][c] = v;
         }
         __syncthreads();
-#pragma unroll 4
-        for (int c = lane; c < pieces; c += 64) {
-            const float4 a = *(const float4*)(wa + k0 + 4 * c);
-            const float4 b = *(const float4*)(wb + k0 + 4 * c);
+#pragma unroll
+        for (int j = 0; j < IPC; ++j) {
+            const int c = lane + 64 * j;
+            float4 a = ra[j], b = rb[j];
+            if (k0 + KC < K) fetch(j, (k0 + KC) / 4 + c);
+            if (c >= pieces) a = b = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
             for (int m = 0; m < MR; ++m) {
                 const float4 xv = xs[m][c];
                 acc[m][0] = fmaf(a.w, xv.w, fmaf(a.z, xv.z, fmaf(a.y, xv.y, fmaf(a.x, xv.x, acc[m][0]))));
                 acc[m][1] = fmaf(b.w, xv.w, fmaf(b.z, xv.z, fmaf(b.y, xv.y, fmaf(b.x, xv.x, acc[m][1]))));
             }
+            // (one piece's reads of x at a time: moved up across the pieces they take the kernel from 112 to 192
+            // registers at eight rows, and half the waves fit a compute unit)
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 #pragma unroll

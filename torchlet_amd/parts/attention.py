@@ -22,6 +22,7 @@ from .base import KEEP_COMPUTE, KEEP_STORED, MIXERS, POSITION_ENCODINGS, LazyNor
 # The plans below deal work-groups to the GPU's compute units; their number comes from the device
 # (``ops.compute_units()``), the thresholds in keys and tokens were measured on an MI355X (256 units).
 _MIN_KEYS_PER_SPLIT = 256
+_MIN_KEYS_PER_SPLIT_32BIT = 64
 _PORTION_MIN_TOKENS = 16     # requests that bring at least this many tokens go to a prompt-portion kernel: the
                              # 128-row one where it is built (head size 64 or 128, pages of 8, 16, 32, ...
                              # tokens; measured on MI355X at 28/4 heads of 128: 2048 new tokens 222 -> 110 us,
@@ -136,11 +137,13 @@ class GQAttention(Mixer):
         chunks = -(-group // ops.ATTENTION_ROWS)
         base = max(1, tiles * self.kv_heads * chunks)
         units = self.compute_units
-        waves = 8 if base <= units else 4
+        waves = 8 if base <= units and self.dtype == torch.bfloat16 else 4      # (the 32-bit kernel has work-groups of four)
         by_fill = -(-(units if waves == 8 else 2 * units) // base)      # four waves: enough work-groups to fill the units twice
         longest = ctx.max_total_len if longest is None else longest
         longest = longest if self.window is None else min(longest, self.window + ctx.max_new_tokens)
-        by_keys = max(1, longest // _MIN_KEYS_PER_SPLIT)
+        # (the 32-bit engine's kernel walks its keys 32 at a time through shared memory, one work-group of four waves
+        # on a part: parts of 64 keys keep the compute units busy where 256 left most of them idle)
+        by_keys = max(1, longest // (_MIN_KEYS_PER_SPLIT if self.dtype == torch.bfloat16 else _MIN_KEYS_PER_SPLIT_32BIT))
         return max(1, min(by_fill, by_keys, 64)), waves
 
     takes_lazy_norm = True

@@ -89,8 +89,14 @@ def parse_args(argv=None):
     return p.parse_args(argv)
 
 
+def say(msg: str) -> None:
+    """A line of progress on standard error (standard output carries the one JSON line)."""
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
 def build(shape: str, layers: int, dtype: str):
     import torch
+    say(f"building {SHAPES[shape][0]} sizes, {layers} layers, {dtype}, random weights")
     from torchlet_amd.engine.loading import build_model
     from torchlet_amd.registry import config_class
     from torchlet_amd.weights.random_init import RandomTensors
@@ -141,6 +147,7 @@ def engine_decode(cfg, model, batch: int, steps: int, warmup: int, context: int,
     from torchlet_amd.engine.loading import make_engine
     from torchlet_amd.engine.request import Request
 
+    say(f"engine: {batch} requests, {context}-token prompts, {warmup} + {steps} decode steps")
     pages = batch * (-(-(context + new_tokens) // PAGE)) + 1
     engine = make_engine(model, EngineConfig(page_size=PAGE, num_pages=pages, max_slots=batch, max_tokens_per_step=max(budget, batch),
                                              use_graphs=True, lookahead=True, seed=0))
@@ -209,6 +216,7 @@ def step_function_decode(cfg, model, batch: int, steps: int, warmup: int, contex
     from torchlet_amd.engine.loading import make_runner
     from torchlet_amd.sampling.sampler import Sampler
 
+    say(f"step function: {batch} requests on {context}-token caches, {warmup} + {steps} decode steps")
     pages = batch * (-(-(context + steps + warmup + 2) // PAGE)) + 1
     runner = make_runner(model, page_size=PAGE, num_pages=pages, max_requests=batch, use_graphs=True)
     ids = [f"b{i}" for i in range(batch)]
@@ -250,6 +258,7 @@ def time_prefill(model, tokens: int, repeats: int = 5, context: int = 0):
     from torchlet_amd.engine.batch import StepEntry
     from torchlet_amd.engine.loading import make_runner
 
+    say(f"prefill: {tokens} tokens on {context} cached, {repeats} runs")
     runner = make_runner(model, page_size=PAGE, num_pages=-(-(context + tokens) // PAGE) + 2, max_requests=1)
     prompt = random_prompts(model.spec.vocab_size, 1, context + tokens)[0]
     times = []
@@ -330,6 +339,7 @@ def serve(cfg, model, args) -> dict:
                                              dtype=args.dtype, use_graphs=True, seed=0))
 
     def run():
+        say(f"serving {len(prompts)} requests, {sum(lengths)} prompt tokens, {new_tokens} new tokens each")
         engine.add_requests([Request(prompt_tokens=list(p), max_new_tokens=new_tokens) for p in prompts])
         steps0 = engine.steps
         torch.cuda.synchronize()

@@ -18,7 +18,7 @@ recomputed from its own fields.  The same line carries
   steps) / its time, against the 8 TB/s of HBM3E (``frac``) and against the rate at which this GPU
   delivers memory to a kernel that only reads (``frac_measured``; ``measured`` holds that yardstick);
 * ``step_function``: the same decode step driven directly (no scheduler): what the scheduler costs;
-* ``prefill``: one 2048-token prompt in one step (tokens/s and ms as the mean of the timed runs, ``ms_best`` the
+* ``prefill``: one 2048-token prompt in one step (tokens/s and ms as the mean of three timed runs, ``ms_best`` the
   fastest of them, flops, ``frac`` of the dense matrix-core peak of the dtype, ``frac_measured`` of the rate this
   repository's own large matrix product reaches);
 * ``points``: decode tokens/s at batch 1 and batch 64 through the engine; ``points_detail`` gives each
@@ -251,7 +251,7 @@ def step_function_decode(cfg, model, batch: int, steps: int, warmup: int, contex
             "mean_context": round(mean_ctx, 1), "bytes_per_step": int(decode_bytes(cfg, model, batch, mean_ctx))}
 
 
-def time_prefill(model, tokens: int, repeats: int = 5, context: int = 0):
+def time_prefill(model, tokens: int, repeats: int = 3, context: int = 0):
     """(mean, best) ms of one step that brings ``tokens`` prompt tokens (after ``context`` tokens fed in 2048-token
     steps) over ``repeats`` runs after one that warms up."""
     import torch
@@ -490,7 +490,7 @@ def main(argv=None) -> int:
     def prefill_point(gemm_tflops=None):
         pms, pbest = time_prefill(model, ptokens)
         flops = prefill_flops(cfg, ptokens)
-        point = {"value": round(ptokens * 1e3 / pms, 1), "tokens": ptokens, "ms": round(pms, 3), "ms_best": round(pbest, 3), "runs": 5,
+        point = {"value": round(ptokens * 1e3 / pms, 1), "tokens": ptokens, "ms": round(pms, 3), "ms_best": round(pbest, 3), "runs": 3,
                  "flops": flops, "frac": round(flops / (pms * 1e-3) / (peak_tflops * 1e12), 4)}
         if gemm_tflops:
             point["frac_measured"] = round(flops / (pms * 1e-3) / (gemm_tflops * 1e12), 4)

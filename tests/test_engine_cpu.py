@@ -268,6 +268,11 @@ def test_toy_attention_that_differs_in_one_stage_on_the_host(cpu_ops):
     toy_parts.run_toy_qk_norm(torch.float32, torch.device("cpu"), lambda dtype, ref: dict(atol=2e-5, rtol=1e-4))
 
 
+def test_toy_norm_of_another_kind_is_run_not_fused_on_the_host(cpu_ops):
+    import toy_parts
+    toy_parts.run_toy_norm(torch.float32, torch.device("cpu"))
+
+
 def test_toy_mixer_whose_cache_planes_differ_on_the_host(cpu_ops):
     import toy_parts
     toy_parts.run_toy_latent(torch.float32, torch.device("cpu"))

@@ -314,3 +314,9 @@ def test_toy_attention_that_differs_in_one_stage(dtype):
 def test_toy_mixer_whose_cache_planes_differ_in_width_and_element_type(dtype):
     import toy_parts
     toy_parts.run_toy_latent(dtype, torch.device("cuda"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_norm_of_another_kind_is_run_and_never_taken_for_the_frameworks_own(dtype):
+    import toy_parts
+    toy_parts.run_toy_norm(dtype, torch.device("cuda"))

@@ -444,3 +444,121 @@ def run_toy_latent(dtype, device):
     finally:
         unregister_architecture("ToyLatentForCausalLM")
         MIXERS.unregister("toy_latent")
+
+
+def run_toy_norm(dtype, device):
+    """A norm of another kind than the framework's (it centres the row before it scales it, and has a bias) in every
+    place a norm stands, beside the framework's attention and feed-forward.  For a step of one token it offers itself
+    unrun, as the framework's norm does (``Norm.lazy``), naming its kind: the attention and the feed-forward, whose
+    kernels can make a root-mean-square norm inside and no other, must run it the usual way.  Requests token by
+    token, in portions and whole agree with each other and with the library's layer norm."""
+    from torchlet_amd.config import AttentionSpec, BlockSpec, ModelConfig, ModelSpec, PartSpec, RotarySpec, RunEntry, SwiGLUSpec
+    from torchlet_amd.engine.batch import StepEntry
+    from torchlet_amd.engine.loading import build_model, make_runner
+    from torchlet_amd.parts import NORMS, Norm, WeightSpec
+    from torchlet_amd.parts.base import LazyNorm
+    from torchlet_amd.registry import config_class, register_architecture, unregister_architecture
+    from torchlet_amd.weights.random_init import random_tensors
+
+    H, HEADS, KVH, HD, INTER, VOCAB, EPS = 64, 4, 2, 16, 96, 70, 1e-5
+    counts = {"offered": 0, "run_from_offer": 0}
+
+    @dataclass(frozen=True)
+    class CentredNormSpec(PartSpec):
+        kind: ClassVar[str] = "toy_centred_norm"
+        dim: int = 0
+
+    @NORMS.register("toy_centred_norm")
+    class CentredNorm(Norm):
+        graph_safe = True
+
+        def weight_specs(self):
+            return {"weight": WeightSpec((self.spec.dim,), keep="stored", init="one_plus_normal"),
+                    "bias": WeightSpec((self.spec.dim,), keep="stored")}
+
+        def load_weights(self, tensors):
+            self.weight = self._place(tensors["weight"], "stored").float()
+            self.bias = self._place(tensors["bias"], "stored").float()
+
+        def forward(self, stream, rows=None, gain=1.0):
+            r = stream.residual
+            if stream.pending is not None:
+                add = stream.pending.float()
+                r = r + (add.sum(0) if add.dim() == 3 else add)         # slabs of partial sums, or one tensor
+            if rows is None:
+                stream.residual.copy_(r)
+                stream.pending = None
+            else:
+                r = r[rows.long()]
+            y = torch.nn.functional.layer_norm(r, (self.spec.dim,), self.weight, self.bias, EPS) * gain
+            return y.to(self.dtype)
+
+        def lazy(self, stream):
+            if stream.residual.shape[0] == 1:
+                counts["offered"] += 1
+                return _Counted(self, stream, "toy_centred_norm", weight=self.weight, bias=self.bias, eps=EPS)
+            return None
+
+    class _Counted(LazyNorm):
+        def value(self):
+            if self._value is None:
+                counts["run_from_offer"] += 1
+            return super().value()
+
+    @dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyCentredNormForCausalLM"
+        vocab_size: int
+
+        def to_spec(self):
+            norm = CentredNormSpec(dim=H)
+            block = BlockSpec(mixer=AttentionSpec(hidden=H, num_heads=HEADS, num_kv_heads=KVH, head_dim=HD, qkv_bias=True,
+                                                  position=RotarySpec(head_dim=HD, theta=10000.0, max_positions=256)),
+                              mixer_norm=norm, ffn_norm=norm, ffn=SwiGLUSpec(hidden=H, intermediate=INTER))
+            return ModelSpec(vocab_size=self.vocab_size, hidden=H, layers=(block, block), order=(RunEntry(0), RunEntry(1)),
+                             final_norm=norm, tie_head=False, max_positions=256)
+
+    def plain_forward(w, ids):
+        sub = lambda p: {k[len(p):]: v for k, v in w.items() if k.startswith(p)}
+        T = len(ids)
+        x = w["model.embed_tokens.weight"][torch.tensor(ids)]
+        norm = lambda t, n: torch.nn.functional.layer_norm(t, (H,), n["weight"], n["bias"], EPS)
+        for layer in range(2):
+            lw = sub(f"model.layers.{layer}.")
+            x = x + plain.gqa_attention(norm(x, sub(f"model.layers.{layer}.input_layernorm.")), sub(f"model.layers.{layer}.self_attn."),
+                                        num_heads=HEADS, num_kv_heads=KVH, head_dim=HD, theta=10000.0, positions=torch.arange(T))
+            x = x + plain.swiglu_ffn(norm(x, sub(f"model.layers.{layer}.post_attention_layernorm.")), sub(f"model.layers.{layer}.mlp."))
+        return plain.linear(norm(x, sub("model.norm.")), w["lm_head.weight"])
+
+    register_architecture(ToyConfig)
+    try:
+        cfg = config_class("ToyCentredNormForCausalLM").from_dict(dict(vocab_size=VOCAB))
+        tensors = {k: (v * 4 if "proj" in k else v) for k, v in random_tensors(cfg, seed=15, dtype=torch.bfloat16).items()}
+        assert tensors["model.layers.1.post_attention_layernorm.bias"].shape == (H,)
+        model = build_model(cfg, dtype, device=device, tensors=tensors)
+        assert model.graph_safe()
+        runner = make_runner(model, page_size=8, num_pages=20, max_requests=2)
+        g = torch.Generator().manual_seed(4)
+        seqs = {"a": torch.randint(0, VOCAB, (37,), generator=g).tolist(), "b": torch.randint(0, VOCAB, (18,), generator=g).tolist()}
+        refs = {k: plain_forward({n: t.double() for n, t in tensors.items()}, v) for k, v in seqs.items()}
+        whole = {k: runner.step([StepEntry(k, v, list(range(len(v))))]).cpu() for k, v in seqs.items()}
+        for k in seqs:
+            runner.release(k)
+        assert counts["offered"] == 0                     # steps of many rows: nothing offered
+        singles = {k: [] for k in seqs}
+        singles["a"].append(runner.step([StepEntry("a", seqs["a"][:20], list(range(20)))]).cpu())
+        for t in seqs["a"][20:]:                          # one request, one token a step: the norms offer themselves
+            singles["a"].append(runner.step([StepEntry("a", [t], [0])]).cpu())
+        assert counts["offered"] == 2 * 2 * 17 and counts["run_from_offer"] == counts["offered"], counts
+        singles["b"].append(runner.step([StepEntry("b", seqs["b"][:9], list(range(9)))]).cpu())
+        for i in range(9, 18):                            # two requests a step: rows of two, nothing offered
+            out = runner.step([StepEntry("b", [seqs["b"][i]], [0])]).cpu()
+            singles["b"].append(out)
+        tol = dict(atol=3e-5, rtol=1e-4) if dtype == torch.float32 else dict(atol=6e-2, rtol=5e-2)
+        for k in seqs:
+            torch.testing.assert_close(whole[k].double(), refs[k], **tol)
+            torch.testing.assert_close(torch.cat(singles[k]).double(), refs[k], **tol)
+        assert float(refs["a"].std()) > 0.05
+    finally:
+        unregister_architecture("ToyCentredNormForCausalLM")
+        NORMS.unregister("toy_centred_norm")

@@ -293,6 +293,14 @@ def test_command_line(model_folders, tmp_path):
     cfg, w = plain_qwen2.load_folder(tmp_path / "m")
     assert [l["output"] for l in lines] == [plain_qwen2.greedy(cfg, w, [5, 6, 7], 4), plain_qwen2.greedy(cfg, w, [9], 4)]
     assert len(set(lines[0]["output"])) >= 3
+    # the replay program as a sub-command: the same options and files as bin/trace_run
+    step = json.dumps({"step": 0, "entries": [{"id": "a", "tokens": [5, 6, 7, 72, 73], "want": [0, 4]}], "end": ["a"]})
+    rep = subprocess.run([sys.executable, "-m", "torchlet_amd", "replay", "--model", str(tmp_path / "m"), "--dtype", "float32",
+                          "--out", str(tmp_path / "logits"), "--max-tokens", "64"], input=step + "\n", cwd=ROOT, capture_output=True, text=True, timeout=120)
+    assert rep.returncode == 0 and rep.stdout.strip() == "done 0", rep.stderr
+    import numpy as np
+    got = torch.from_numpy(np.fromfile(tmp_path / "logits" / "0.f32", dtype="<f4").reshape(2, cfg.vocab))
+    torch.testing.assert_close(got.double(), plain_qwen2.forward(cfg, w, [5, 6, 7, 72, 73])[[0, 4]], **scenarios.FP32_TOL)
 
 
 def _write_tokenizer(folder, vocab_size):

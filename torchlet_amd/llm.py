@@ -23,6 +23,7 @@ The tokenizer is read from the folder's ``tokenizer.json`` with the ``tokenizers
     python -m torchlet_amd --model DIR --prompt "hello" --max-new-tokens 64
     python -m torchlet_amd --model DIR --prompt-ids 1,2,3 --temperature 0.8 --seed 1
     python -m torchlet_amd init --config config.json --seed 0 --out DIR     # random weights
+    python -m torchlet_amd replay --model DIR --dtype float32 --out DIR --max-tokens N < steps.jsonl    # = bin/trace_run
 """
 from __future__ import annotations
 
@@ -216,6 +217,7 @@ def _parser():
         q.add_argument("--max-num-batched-tokens", type=int, default=2048)
         q.add_argument("--max-model-len", type=int, default=None, help="sequences no longer than this (default: the model's limit)")
         q.add_argument("--verbose", action="store_true", help="report the backend, the folder's tensors and the engine's sizes at start-up")
+    sub.add_parser("replay", add_help=False, help="feed given token ids step by step and write logits (the options of bin/trace_run)")
     i = sub.add_parser("init", help="write a model folder with random weights from a configuration and a seed")
     i.add_argument("--config", required=True, help="a config.json")
     i.add_argument("--seed", type=int, default=0)
@@ -225,6 +227,10 @@ def _parser():
 
 
 def main(argv=None) -> int:
+    argv = list(sys.argv[1:] if argv is None else argv)
+    if argv and argv[0] == "replay":              # the trace replay program's own options (bin/trace_run is the same program)
+        from .engine import trace
+        return trace.main(argv[1:])
     args = _parser().parse_args(argv)
     if args.command == "init":
         from .engine.loading import parse_dtype

@@ -193,9 +193,17 @@ def test_linear_few_rows_in_32_bit(ops, M, N, K):
     out = torch.full((M, N), float("nan"), device="cuda")
     ops.linear(x, w, b, out)
     torch.testing.assert_close(out.double(), ref, **tol32)
-    alone = torch.empty(1, N, device="cuda")
-    ops.linear(x[M - 1:], w, b, alone)
-    assert torch.equal(alone[0], out[M - 1])
+    # two kernels serve these row counts (multiply-adds up to 8 rows, the matrix cores' true 32-bit instruction from 9
+    # on): each agrees with float64, and in each a row's sum runs in one order whatever stands beside it (bitwise)
+    for variant in (2, 3):
+        got = torch.full((M, N), float("nan"), device="cuda")
+        ops.linear_f32_variant(x, w, b, got, variant)
+        torch.testing.assert_close(got.double(), ref, **tol32)
+        alone = torch.empty(1, N, device="cuda")
+        ops.linear_f32_variant(x[M - 1:], w, b, alone, variant)
+        assert torch.equal(alone[0], got[M - 1]), f"variant {variant}"
+        if variant == (3 if M > 8 else 2):
+            assert torch.equal(got, out)                   # the dispatch's choice
     wide = torch.zeros(M, K + 24, device="cuda")          # a strided input view, a wider output
     wide[:, 8:8 + K] = x
     out2 = torch.full((M, N + 5), 3.0, device="cuda")

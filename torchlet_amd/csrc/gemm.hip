@@ -188,12 +188,95 @@ __global__ __launch_bounds__(256) void gemv_f32_kernel(const float* __restrict__
     }
 }
 
+// The same on the matrix cores, 2 to 16 rows: v_mfma_f32_16x16x4_f32 multiplies and adds in true 32-bit (as
+// v_mfma_f32_32x32x2_f32 below), and a step of several rows costs the stream of weights and little else, where the
+// kernel above spends a multiply-add per row and weight (the dispatch takes this kernel from 9 rows on).  A work-group of eight waves owns 16 weight rows; chunks of GM_KC columns of x wait in shared
+// memory (rows beyond M as zeros); within a chunk the waves take its pieces of 16 columns in turn.  A lane fetches
+// four neighbouring k of its weight row and of its x row at once: lane group g = lane / 16 takes k = 4 g .. 4 g + 3
+// of the piece, so instruction e of a piece multiplies k = 4 g + e of the four groups: which k meet in one instruction
+// is free as long as both operands agree.  The pieces of the next chunk are requested while this chunk's are
+// multiplied.  Each wave's sum over its pieces runs in one fixed order and the eight partial tiles are added in wave
+// order, whatever M is: a row's result does not depend on the batch (it differs from the other 32-bit kernels' by
+// rounding).  Needs K % 4 == 0 and 16-byte aligned rows.
+typedef float gm_f32x4_t __attribute__((ext_vector_type(4)));
+#define GM_WAVES 8
+#define GM_KC 512                        // columns of x in shared memory at a time: 16 rows x 512 x 4 bytes = 32 KB
+#define GM_LD (GM_KC + 4)                // floats between rows of x: 16-byte reads of 16 rows fall on all banks
+__global__ __launch_bounds__(GM_WAVES * 64) void gemv_f32_mfma_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                      const void* __restrict__ bias, int bias_f32,
+                                                                      float* __restrict__ out, int M, int N, int K, int ldx, int ldo) {
+    __shared__ __attribute__((aligned(16))) float xs[16 * GM_LD];
+    __shared__ __attribute__((aligned(16))) float red[GM_WAVES * 256];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 15, lg = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const float* wrow = w + (size_t)min(n0 + li, N - 1) * K;       // rows past the end: the last row again, never stored
+    constexpr int PPW = GM_KC / 16 / GM_WAVES;                     // pieces of 16 columns a wave takes of a chunk
+    gm_f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    float4 ring[PPW];
+    // piece q of the chunk at k0 that is this wave's: columns k0 + 16 (wave + q GM_WAVES) + 4 lg .. + 3; beyond K the
+    // row's last whole four are fetched and cleared
+    auto fetch = [&](int q, int k0) {
+        const int k = k0 + 16 * (wave + q * GM_WAVES) + 4 * lg;
+        ring[q] = *(const float4*)(wrow + min(k, K - 4));
+        if (k >= K) ring[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+#pragma unroll
+    for (int q = 0; q < PPW; ++q) fetch(q, 0);
+    for (int k0 = 0; k0 < K; k0 += GM_KC) {
+        const int cols = min(GM_KC, K - k0);
+        __syncthreads();                                           // the chunk before is read
+        for (int i = tid; i < 16 * (GM_KC / 4); i += GM_WAVES * 64) {
+            const int m = i / (GM_KC / 4), c = i % (GM_KC / 4);
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m < M && 4 * c < cols) v = *(const float4*)(x + (size_t)m * ldx + k0 + 4 * c);
+            *(float4*)(&xs[m * GM_LD + 4 * c]) = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < PPW; ++q) {
+            const float4 a = ring[q];
+            if (k0 + GM_KC < K) fetch(q, k0 + GM_KC);
+            const float4 b = *(const float4*)(&xs[li * GM_LD + 16 * (wave + q * GM_WAVES) + 4 * lg]);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, acc, 0, 0, 0);
+        }
+    }
+    // a lane holds weight rows i = 4 (lane / 16) + v and x row j = lane % 16 of its wave's partial tile
+    *(gm_f32x4_t*)(&red[(wave * 64 + lane) * 4]) = acc;
+    __syncthreads();
+    if (wave == 0) {
+        gm_f32x4_t sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int wv = 0; wv < GM_WAVES; ++wv) sum += *(const gm_f32x4_t*)(&red[(wv * 64 + lane) * 4]);
+        const int m = li;
+        if (m < M) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int n = n0 + 4 * lg + v;
+                if (n < N) out[(size_t)m * ldo + n] = sum[v] + (bias ? load_vec(bias, bias_f32, n) : 0.f);
+            }
+        }
+    }
+}
+
 static bool gemv_f32_fits(const void* x, const void* w, int M, int K, int ldx) {
     return M <= 16 && K % 4 == 0 && ldx % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0;
 }
 
+// mfma: 0 the multiply-add kernel, 1 the matrix-core kernel, -1 the one that is faster for M.  Measured on the four
+// products of a 7B layer (us, multiply-adds / matrix cores): 1 row 174 / 237, 4 rows 216 / 241, 8 rows 274 / 265,
+// 16 rows 425 / 300: the matrix-core kernel's time hardly grows with the rows, but its work-groups of 16 weight rows
+// are too few on the narrow matrices (224 for 3584 rows) to stream as fast as the other's 448 of 8.
 static void launch_gemv_f32(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
-                            int ldx, int ldo, hipStream_t stream) {
+                            int ldx, int ldo, hipStream_t stream, int mfma = -1) {
+    if (mfma == 1 || (mfma < 0 && M > 8)) {
+        gemv_f32_mfma_kernel<<<dim3((N + 15) / 16), dim3(GM_WAVES * 64), 0, stream>>>((const float*)x, (const float*)w, bias, bias_f32,
+                                                                                     (float*)out, M, N, K, ldx, ldo);
+        return;
+    }
     dim3 grid((N + GV_ROWS - 1) / GV_ROWS), block(256);
 #define GV_LAUNCH(MR) gemv_f32_kernel<MR><<<grid, block, 0, stream>>>((const float*)x, (const float*)w, bias, bias_f32, (float*)out, M, N, K, ldx, ldo)
     if (M <= 1) GV_LAUNCH(1);
@@ -342,11 +425,15 @@ static void launch_gemm_f32_mfma(const void* x, const void* w, const void* bias,
     }
 }
 
-// One named kernel of the 32-bit products (for tests and tuning): 0 the general tile kernel (v_fma_f32), 1 the matrix-core kernel.
+// One named kernel of the 32-bit products (for tests and tuning): 0 the general tile kernel (v_fma_f32), 1 the matrix-core
+// tile kernel, 2 and 3 the kernels for up to 16 rows on multiply-adds and on the matrix cores.
 extern "C" int tl_gemm_f32_variant(const void* x, const void* w, const void* bias, int bias_f32, void* out,
                                    int M, int N, int K, int ldx, int ldo, int matrix_cores, hipStream_t stream) {
     TL_REQUIRE(M > 0 && N > 0 && K > 0 && ldx >= K && ldo >= N, "gemm_f32: bad sizes M=%d N=%d K=%d ldx=%d ldo=%d", M, N, K, ldx, ldo);
-    if (matrix_cores) {
+    if (matrix_cores == 2 || matrix_cores == 3) {      // the two kernels for up to 16 rows: 2 multiply-adds, 3 matrix cores
+        TL_REQUIRE(gemv_f32_fits(x, w, M, K, ldx), "gemm_f32: the few-rows kernels need M <= 16, K %% 4 == 0 and 16-byte aligned rows");
+        launch_gemv_f32(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream, matrix_cores - 2);
+    } else if (matrix_cores) {
         TL_REQUIRE(gemm_f32_mfma_fits(x, w, 17, K, ldx), "gemm_f32: the matrix-core kernel needs K %% 4 == 0 and 16-byte aligned rows");
         launch_gemm_f32_mfma(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, stream);
     } else {

@@ -207,9 +207,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out
                                     c_int(1 if out.dtype == torch.float32 else 0), _stream()))
 
 
-def linear_f32_variant(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, matrix_cores: bool) -> None:
-    """One named kernel of the 32-bit products (for tests and tuning): the general tile kernel (``v_fma_f32``)
-    or the matrix-core kernel (``v_mfma_f32_32x32x2_f32``, K a multiple of 4); both multiply and add in true 32-bit."""
+def linear_f32_variant(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out: torch.Tensor, matrix_cores) -> None:
+    """One named kernel of the 32-bit products (for tests and tuning): 0 / False the general tile kernel (``v_fma_f32``),
+    1 / True the matrix-core tile kernel (``v_mfma_f32_32x32x2_f32``, K a multiple of 4), 2 and 3 the kernels for up to 16
+    rows on multiply-adds and on the matrix cores (``v_mfma_f32_16x16x4_f32``); all multiply and add in true 32-bit."""
     M, K = x.shape
     N = weight.shape[0]
     if x.dtype != torch.float32 or weight.dtype != torch.float32 or out.dtype != torch.float32 or out.shape != (M, N) \
@@ -218,7 +219,7 @@ def linear_f32_variant(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
     bf = _vec(bias, N, "linear bias")
     lib = _lib("gemm")
     _check(lib, lib.tl_gemm_f32_variant(_ptr(x), _ptr(weight), _ptr(bias), c_int(bf), _ptr(out), c_int(M), c_int(N), c_int(K),
-                                        c_int(x.stride(0)), c_int(out.stride(0)), c_int(1 if matrix_cores else 0), _stream()))
+                                        c_int(x.stride(0)), c_int(out.stride(0)), c_int(int(matrix_cores)), _stream()))
 
 
 def linear_few_rows_variant(x, weight, bias, out, strips_per_wave: int, waves_along_k: int, rows_per_strip: int = 0) -> None:

@@ -101,6 +101,23 @@ def test_linear_partials_and_their_sum_in_the_norm(ops, M, N, K):
     torch.testing.assert_close(out2.double(), refn[rows.long()], **_tol(torch.bfloat16))
 
 
+def test_a_portion_of_2048_rows_against_a_narrow_down_projection_is_split_in_two(ops):
+    """2048 rows against a 5120 x 27648 matrix: 160 tiles of 256 x 256 leave three compute units in eight idle, and
+    128 tiles of 256 x 320 with K in two halves are one round of 256 work-groups.  The plan is that one, and its sum
+    is the product."""
+    M, N, K = 2048, 5120, 27648
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    assert ops.linear_partials_pay(M, N, K)
+    parts = ops.linear_partials(x, w)
+    if ops.compute_units() == ops.MEASURED_COMPUTE_UNITS:
+        assert parts.shape[0] == 2
+    ref = x.double() @ w.double().T
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    torch.testing.assert_close(parts.double().sum(0), ref, **tol32)
+
+
 def test_rmsnorm_zero_row_is_zero_not_nan(ops):
     res = torch.zeros(2, 64, device="cuda")
     w = torch.ones(64, device="cuda")
@@ -307,7 +324,7 @@ def test_linear_many_rows_fetched_straight_into_shared_memory(ops, out_dtype, ti
     assert bool((out2[:, N:] == 5.0).all())
 
 
-@pytest.mark.parametrize("tile", [(64, 64, 0), (64, 192, 0), (64, 320, 0), (128, 192, 0), (128, 128, 0), (128, 128, 4), (128, 256, 0), (256, 128, 0), (192, 256, 0), (256, 192, 0), (256, 256, 0)])
+@pytest.mark.parametrize("tile", [(64, 64, 0), (64, 192, 0), (64, 320, 0), (128, 192, 0), (128, 128, 0), (128, 128, 4), (128, 256, 0), (256, 128, 0), (192, 256, 0), (256, 192, 0), (256, 256, 0), (256, 320, 0)])
 @pytest.mark.parametrize("M,N,K,parts", [(65, 129, 128, 2), (128, 520, 1024, 4), (100, 3584, 2048, 8), (300, 257, 1088, 3), (7, 48, 3584, 7)])
 def test_linear_split_over_k_on_every_tile_shape(ops, tile, M, N, K, parts):
     """Slabs of partial sums from every tile shape of the direct-load kernel (the four-slab 128 x 128

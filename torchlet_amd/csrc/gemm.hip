@@ -1312,21 +1312,18 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
 #undef DL_SWZ
 
     // The loop is a hand-laid pipeline; scheduling fences keep the compiler from undoing it.  A step
-    // of TK columns has TK / 16 phases of FM * FN products.  Each phase first issues the operand reads
-    // of the next phase into the other register set, then its products, so a read has a whole
-    // phase to arrive.  The last phase of a step waits for the next slab, meets the other waves at
-    // the barrier (they have all read their last operands of this slab by then), requests the slab
-    // STAGES - 1 ahead into the buffer just given up, and reads the first operands of the next slab,
-    // all before its own products.  Past the end the last slab is requested again (nobody reads
-    // it), so the count of requests in flight is the same in every step, which the wait relies on.
+    // of TK columns has TK / 16 phases of FM * FN products.  A phase's memory instructions go between
+    // its products, one product first: the operand reads of the next phase into the other register set,
+    // so a read has a whole phase to arrive, and the wait before a phase's first product is for operands
+    // asked for a phase ago with nothing younger outstanding.  (All reads first and then all products,
+    // the wait at the loop's head came out as one for every read, the ones just issued too, and the 7B's fused
+    // gate/up product at 2048 rows took 537 us instead of 487.)  The last phase of a step first waits for the
+    // next slab and meets the other waves at the barrier (they have all read their last operands of this
+    // slab by then); between its products go the requests for the slab STAGES - 1 ahead, into the buffer
+    // just given up, and then the reads of the first operands of the next slab.  Past the end the last slab
+    // is requested again (nobody reads it), so the count of requests in flight is the same in every step,
+    // which the wait relies on.
     Frag16 af[2][FM], bfr[2][FN];
-    auto read_operands = [&](int set, const bf16_t* cb, int kk) {
-        const int c = 2 * kk + fh;
-#pragma unroll
-        for (int i = 0; i < FM; ++i) af[set][i].u = *(const uint4*)(cb + arow[i] * TK + ((c ^ akey[i]) * 8));
-#pragma unroll
-        for (int j = 0; j < FN; ++j) bfr[set][j].u = *(const uint4*)(cb + brow[j] * TK + ((c ^ bkey[j]) * 8));
-    };
     auto request_slab = [&](int slab) {
         const int k0 = min(slab, slabs - 1) * TK;
         const unsigned nb = lds_base + (slab % STAGES) * LROWS * TK * 2;
@@ -1338,30 +1335,46 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
     wait_direct_loads<(STAGES - 2) * LOADS>();
     __syncthreads();
     request_slab(STAGES - 1);
-    read_operands(0, lds_raw, 0);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) af[0][i].u = *(const uint4*)(lds_raw + arow[i] * TK + ((fh ^ akey[i]) * 8));
+#pragma unroll
+    for (int j = 0; j < FN; ++j) bfr[0][j].u = *(const uint4*)(lds_raw + brow[j] * TK + ((fh ^ bkey[j]) * 8));
     __builtin_amdgcn_sched_barrier(0);
 
     constexpr int PHASES = TK / 16;
+    constexpr int NM = FM * FN, NR = FM + FN;               // products and operand reads of a phase
     for (int sl = 0; sl < slabs; ++sl) {
         const bf16_t* cb = lds_raw + (sl % STAGES) * LROWS * TK;
 #pragma unroll
         for (int kk = 0; kk < PHASES; ++kk) {
             const int cur = kk & 1, nxt = cur ^ 1;
-            if (kk + 1 < PHASES) {
-                read_operands(nxt, cb, kk + 1);
-            } else {
+            const bool last = kk + 1 == PHASES;
+            const bf16_t* nb = last ? lds_raw + ((sl + 1) % STAGES) * LROWS * TK : cb;      // where the next phase's operands lie
+            const int c = (last ? 0 : 2 * (kk + 1)) + fh;
+            const int k0 = min(sl + STAGES, slabs - 1) * TK;
+            const unsigned qb = lds_base + (sl % STAGES) * LROWS * TK * 2;                   // the buffer given up: slab sl + STAGES goes there
+            const int ops = last ? LOADS + NR : NR;                                          // memory instructions of this phase ...
+            const int per = (ops + NM - 1) / NM;                                             // ... and how many follow each product
+            if (last) {
                 wait_direct_loads<(STAGES - 2) * LOADS>();
                 __syncthreads();
-                request_slab(sl + STAGES);
-                read_operands(nxt, lds_raw + ((sl + 1) % STAGES) * LROWS * TK, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
+            int op = 0;
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+            for (int q = 0; q < NM; ++q) {
+                acc[q / FN][q % FN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][q % FN].v, af[cur][q / FN].v, acc[q / FN][q % FN], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][j].v, af[cur][i].v, acc[i][j], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+                for (int e = 0; e < per; ++e, ++op) {
+                    if (op >= ops) break;
+                    const int r = last ? op - LOADS : op;
+                    if (r < 0) load_to_lds(src[op] + k0, qb + ldst[op]);
+                    else if (r < FM) af[nxt][r].u = *(const uint4*)(nb + arow[r] * TK + ((c ^ akey[r]) * 8));
+                    else bfr[nxt][r - FM].u = *(const uint4*)(nb + brow[r - FM] * TK + ((c ^ bkey[r - FM]) * 8));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     }
     wait_direct_loads<0>();

@@ -1212,12 +1212,13 @@ static int launch_mfma_tile(const void* x, const void* w, const void* bias, int 
 // that the sixteen rows a quarter-wave reads for one MFMA operand fall on all 64 banks (measured:
 // no bank conflicts).  The lane that fills slot s of row r therefore fetches piece s ^ ((r >> 1) & 7)
 // of that row from memory.  STAGES slabs are in flight or in use: the slab STAGES - 1 ahead is
-// requested at the top of a step into the buffer that the previous step has finished with, and a
-// step ends with a wait for this wave's requests of the next slab and one barrier.
+// requested into the buffer that a step has just finished with, and a step ends with a wait for
+// this wave's requests of the next slab and one barrier.
 // The requests are issued as assembly: the compiler orders every later shared-memory read behind
-// a direct load it knows of (a full wait per slab), so the kernel keeps that order itself.
-__device__ __forceinline__ void load_to_lds(const void* gptr, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
+// a direct load it knows of (a full wait per slab), so the kernel keeps that order itself.  The
+// address is a base that the wave shares and a 32-bit offset per lane.
+__device__ __forceinline__ void load_to_lds_at(const void* base, unsigned offset, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(offset), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
@@ -1280,18 +1281,28 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
     }
     const int m0 = tm * BM, n0 = tn * BN;
 
-    // instruction j of this wave fills rows RPL (wave + j NW) .. + RPL of the stacked [x rows; w rows] slab
-    const bf16_t* src[LOADS];
+    // Instruction j of this wave fills rows RPL (wave + j NW) .. + RPL of the stacked [x rows; w rows] slab.  Its
+    // eight rows are all of x or all of w (BM is a multiple of RPL), so its address is a base the wave shares (the
+    // tile's first row of x or of w, moved along K from step to step by scalar instructions) and a 32-bit offset per
+    // lane that never changes: half the address registers of a 64-bit address per lane, and no vector addition per
+    // request (2048 x 37888 x 3584: 500 -> 478 us).
+    static_assert(BM % RPL == 0, "the rows of one request lie in one operand");
     int ldst[LOADS];
+    unsigned soff[LOADS];
+    unsigned of_x = 0;                                      // bit j: request j fetches rows of x
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
         const int base_row = RPL * (wave + j * NW);
         const int row = min(base_row + lane / PPR, ROWS - 1);      // (rows of the rounding: copies of the last row, never read)
         const int c = (lane % PPR) ^ DL_SWZ(row);
-        if (row < BM) src[j] = x + (size_t)min(m0 + row, M - 1) * ldx + c * 8;
-        else src[j] = w + (size_t)min(n0 + row - BM, N - 1) * ldw + c * 8;
+        if (row < BM) soff[j] = (unsigned)((min(m0 + row, M - 1) - m0) * ldx + c * 8) * 2;
+        else soff[j] = (unsigned)((min(n0 + row - BM, N - 1) - n0) * ldw + c * 8) * 2;
         ldst[j] = __builtin_amdgcn_readfirstlane(base_row * TK * 2);
+        of_x |= (unsigned)(base_row < BM) << j;
     }
+    of_x = __builtin_amdgcn_readfirstlane(of_x);
+    const bf16_t* xt = x + (size_t)m0 * ldx;
+    const bf16_t* wt = w + (size_t)n0 * ldw;
     const unsigned lds_base = (unsigned)(uintptr_t)((void __attribute__((address_space(3)))*)lds_raw);
 
     f32x16_t acc[FM][FN];
@@ -1319,22 +1330,27 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
     // the wait at the loop's head came out as one for every read, the ones just issued too, and the 7B's fused
     // gate/up product at 2048 rows took 537 us instead of 487.)  The last phase of a step first waits for the
     // next slab and meets the other waves at the barrier (they have all read their last operands of this
-    // slab by then); between its products go the requests for the slab STAGES - 1 ahead, into the buffer
-    // just given up, and then the reads of the first operands of the next slab.  Past the end the last slab
-    // is requested again (nobody reads it), so the count of requests in flight is the same in every step,
-    // which the wait relies on.
+    // slab by then); between its products go the first half of the requests for the slab STAGES - 1 ahead, into
+    // the buffer just given up, and then the reads of the first operands of the next slab.  The other half of
+    // the requests goes into the first phase of the next step: a compute unit's 64 requests in one phase hold
+    // its waves up, whatever they fetch (requests of 4 bytes a lane cost the same; without any the loop ran a
+    // sixth faster), and in two phases less so (2048 x 3584 x 18944: 392 -> 353 us; spread over three phases the
+    // last ones arrive too late).  Past the end the last slab is requested again (nobody reads it), so the count
+    // of requests in flight is the same in every step, which the wait relies on.
     Frag16 af[2][FM], bfr[2][FN];
-    auto request_slab = [&](int slab) {
-        const int k0 = min(slab, slabs - 1) * TK;
-        const unsigned nb = lds_base + (slab % STAGES) * LROWS * TK * 2;
-#pragma unroll
-        for (int j = 0; j < LOADS; ++j) load_to_lds(src[j] + k0, nb + ldst[j]);
+    constexpr int L_LAST = (LOADS + 1) / 2;                 // requests of a slab issued in the last phase of a step; the rest in the next step's first
+    auto request = [&](int slab, int j) {
+        const bf16_t* from = ((of_x >> j) & 1 ? xt : wt) + min(slab, slabs - 1) * TK;
+        load_to_lds_at(from, soff[j], lds_base + (slab % STAGES) * LROWS * TK * 2 + ldst[j]);
     };
 #pragma unroll
-    for (int st = 0; st < STAGES - 1; ++st) request_slab(st);
+    for (int st = 0; st < STAGES - 1; ++st)
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j) request(st, j);
     wait_direct_loads<(STAGES - 2) * LOADS>();
     __syncthreads();
-    request_slab(STAGES - 1);
+#pragma unroll
+    for (int j = 0; j < L_LAST; ++j) request(STAGES - 1, j);
 #pragma unroll
     for (int i = 0; i < FM; ++i) af[0][i].u = *(const uint4*)(lds_raw + arow[i] * TK + ((fh ^ akey[i]) * 8));
 #pragma unroll
@@ -1351,9 +1367,12 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
             const bool last = kk + 1 == PHASES;
             const bf16_t* nb = last ? lds_raw + ((sl + 1) % STAGES) * LROWS * TK : cb;      // where the next phase's operands lie
             const int c = (last ? 0 : 2 * (kk + 1)) + fh;
-            const int k0 = min(sl + STAGES, slabs - 1) * TK;
-            const unsigned qb = lds_base + (sl % STAGES) * LROWS * TK * 2;                   // the buffer given up: slab sl + STAGES goes there
-            const int ops = last ? LOADS + NR : NR;                                          // memory instructions of this phase ...
+            // this phase's requests [lfirst, lend) and the slab they fetch: in the last phase the slab that gets the
+            // buffer given up now, in the first the rest of the slab that got the buffer given up a step ago
+            const int lfirst = last ? 0 : L_LAST, lend = last ? L_LAST : kk == 0 ? LOADS : L_LAST;
+            const int slab_of = last ? sl + STAGES : sl - 1 + STAGES;
+            const int nl = lend - lfirst;
+            const int ops = nl + NR;                                                         // memory instructions of this phase ...
             const int per = (ops + NM - 1) / NM;                                             // ... and how many follow each product
             if (last) {
                 wait_direct_loads<(STAGES - 2) * LOADS>();
@@ -1368,8 +1387,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
 #pragma unroll
                 for (int e = 0; e < per; ++e, ++op) {
                     if (op >= ops) break;
-                    const int r = last ? op - LOADS : op;
-                    if (r < 0) load_to_lds(src[op] + k0, qb + ldst[op]);
+                    const int r = op - nl;
+                    if (r < 0) request(slab_of, lfirst + op);
                     else if (r < FM) af[nxt][r].u = *(const uint4*)(nb + arow[r] * TK + ((c ^ akey[r]) * 8));
                     else bfr[nxt][r - FM].u = *(const uint4*)(nb + brow[r - FM] * TK + ((c ^ bkey[r - FM]) * 8));
                 }
@@ -1560,6 +1579,8 @@ template <int BM, int BN, int WGM, int WGN, int STAGES, typename TOut, bool SW, 
 static int launch_dl_tile_t(const void* x, const void* w, const void* bias, int bias_f32, void* out, int M, int N, int K,
                             int ldx, int ldo, int out_cols, hipStream_t stream, int parts = 1, int k_per = 0) {
     constexpr size_t lds = (size_t)STAGES * dl_slab_rows(BM, BN, WGM * WGN, TK) * TK * sizeof(bf16_t);
+    // (a lane's offset from its tile's first row is kept in 32 bits)
+    TL_REQUIRE((long)(BM > BN ? BM : BN) * (ldx > K ? ldx : K) * 2 < (1L << 31), "gemm_dl_tile: rows of %d elements are too long", ldx > K ? ldx : K);
     auto kernel = gemm_dl_tile_kernel<BM, BN, WGM, WGN, STAGES, TOut, SW, TK>;
     static hipError_t allowed = allow_lds(kernel, lds);
     if (allowed != hipSuccess) {

@@ -902,6 +902,12 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
         const bf16_t* q = (const bf16_t*)a.q + (size_t)r_token * a.q_stride + (size_t)r_head * AT_HD;
 #pragma unroll
         for (int c = 0; c < AT_HD / 16; ++c) qf[c].u = row_ok ? *(const uint4*)(q + 16 * c + 8 * h) : make_uint4(0, 0, 0, 0);
+        // The query is waited for here, once.  Left to the compiler, the wait would stand before the first product of
+        // every step (at the loop's head it must assume the fetch of before the loop still under way), and as a wait for
+        // all fetches it would also wait for the keys and values just requested for the next step: no step would
+        // overlap with the fetch of the next.
+#pragma unroll
+        for (int c = 0; c < AT_HD / 16; ++c) asm volatile("" : "+v"(qf[c].v));
     }
 
     const int key_hi = ctx + tok0 + ntok;
@@ -1034,19 +1040,33 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
         }
         if (wave_has_rows && kbase <= w_pos_max && kbase + ATQ_KEYS > w_lo_min) {
             // ---- scores of two blocks of 32 keys
+            // (the blocks take turns: a product that adds to the sums of the one before it waits for it to finish)
             f32x16_t sc[ATQ_KB];
 #pragma unroll
-            for (int kb = 0; kb < ATQ_KB; ++kb) {
+            for (int kb = 0; kb < ATQ_KB; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) sc[kb][v] = 0.f;
+            // and a block's keys are read two products of that block ahead
+            constexpr int KAHEAD = 2;
+            FragK kf[KAHEAD + 1][ATQ_KB];
+            auto read_keys = [&](int c, int kb) {
                 const int kl = 32 * kb + krow;
+                kf[c % (KAHEAD + 1)][kb].u = *(const uint4*)(kb_s + kl * (AT_HD * 2) + atq_key_slot(2 * c + h, kl) * 16);
+            };
 #pragma unroll
-                for (int c = 0; c < AT_HD / 16; ++c) {
-                    FragK kf;
-                    kf.u = *(const uint4*)(kb_s + kl * (AT_HD * 2) + atq_key_slot(2 * c + h, kl) * 16);
-                    sc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[c].v, sc[kb], 0, 0, 0);
+            for (int c = 0; c < KAHEAD; ++c)
+#pragma unroll
+                for (int kb = 0; kb < ATQ_KB; ++kb) read_keys(c, kb);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int c = 0; c < AT_HD / 16; ++c)
+#pragma unroll
+                for (int kb = 0; kb < ATQ_KB; ++kb) {
+                    sc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[c % (KAHEAD + 1)][kb].v, qf[c].v, sc[kb], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (c + KAHEAD < AT_HD / 16) read_keys(c + KAHEAD, kb);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-            }
             // ---- mask, maximum, probabilities.  Element (kb, 4 q + v) of this lane is key
             // kbase + 32 kb + 16 (q / 2) + 8 h + 4 (q % 2) + v of row lr.  The maximum is taken of the scores as
             // they come out of the product; the factor on them (positive: the host checks) goes into the

@@ -302,7 +302,7 @@ def test_linear_many_rows_on_matrix_cores(ops, out_dtype, tile, M, N, K):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("tile", [(64, 64), (64, 128), (64, 192), (64, 256), (64, 320), (128, 128), (128, 192), (128, 256), (256, 128), (192, 256), (256, 192), (256, 256)])
+@pytest.mark.parametrize("tile", [(64, 64), (64, 128), (64, 192), (64, 256), (64, 320), (128, 128), (128, 192), (128, 256), (256, 128), (192, 256), (256, 192), (256, 256), (256, 160)])
 @pytest.mark.parametrize("M,N,K", [(65, 129, 64), (300, 520, 192), (1000, 257, 1024), (33, 48, 3584), (40, 4608, 128), (513, 700, 320)])
 def test_linear_many_rows_fetched_straight_into_shared_memory(ops, out_dtype, tile, M, N, K):
     """Every tile shape of the direct-load matrix-core kernel, with tails in M and N, one slab to
@@ -324,7 +324,7 @@ def test_linear_many_rows_fetched_straight_into_shared_memory(ops, out_dtype, ti
     assert bool((out2[:, N:] == 5.0).all())
 
 
-@pytest.mark.parametrize("tile", [(64, 64, 0), (64, 192, 0), (64, 320, 0), (128, 192, 0), (128, 128, 0), (128, 128, 4), (128, 256, 0), (256, 128, 0), (192, 256, 0), (256, 192, 0), (256, 256, 0), (256, 320, 0)])
+@pytest.mark.parametrize("tile", [(64, 64, 0), (64, 192, 0), (64, 320, 0), (128, 192, 0), (128, 128, 0), (128, 128, 4), (128, 256, 0), (256, 128, 0), (192, 256, 0), (256, 192, 0), (256, 256, 0), (256, 320, 0), (256, 160, 0)])
 @pytest.mark.parametrize("M,N,K,parts", [(65, 129, 128, 2), (128, 520, 1024, 4), (100, 3584, 2048, 8), (300, 257, 1088, 3), (7, 48, 3584, 7)])
 def test_linear_split_over_k_on_every_tile_shape(ops, tile, M, N, K, parts):
     """Slabs of partial sums from every tile shape of the direct-load kernel (the four-slab 128 x 128

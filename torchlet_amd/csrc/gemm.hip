@@ -1496,11 +1496,17 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
 // two halves are one round of 256 work-groups.  Measured at 2048 rows, slabs written: 5120 x 27648 504 us against
 // 651 whole and 573 in three parts of 256 x 256; 5120 x 13824 263 against 324 and 306; 5120 x 5120 112 against 140
 // and 132.  Its rate here is the one it reaches with all compute units busy, lower than a tile's that runs on 160.)
-enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_64x128, DL_128x128_S4, DL_64x192, DL_128x192, DL_64x320, DL_256x320, DL_TILES };
-static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 192, 256, 256, 64, 128, 64, 128, 64, 256};
-static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256, 128, 128, 192, 192, 320, 320};
-static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12, 2.1e12, 4.2e12, 3.0e12, 4.4e12, 3.5e12, 5.5e12};   // FLOP/s of one compute unit
-static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6, 5e-6, 4.5e-6, 9e-6, 9e-6, 12e-6, 10e-6};       // seconds per tile
+// (DL_256x160: four waves of 64 x 160, for matrices 5120 wide as well: 2048 rows are 256 tiles, one to a compute
+// unit, and 4096 rows two rounds of them where tiles of 256 x 256 take one and a quarter.  A compute unit gets through
+// a slab of it hardly faster than through one of 256 x 256 (what a slab costs is mostly its requests, 52 against 64,
+// not its products, 40 against 64), so it wins only where it fills rounds that the square tile leaves part empty.
+// Measured, whole products: 2048 x 5120 x 13824 261 us against 274-296; 2048 x 5120 x 5120 97 against 106; at 4096
+// rows 499 against 585 and 202 against 239; 4096 x 4608 x 3584 130 against 158.  Eight waves of 32 x 160: 265, 99.)
+enum DlTile { DL_64x64, DL_64x256, DL_128x128, DL_128x256, DL_256x128, DL_192x256, DL_256x192, DL_256x256, DL_64x128, DL_128x128_S4, DL_64x192, DL_128x192, DL_64x320, DL_256x320, DL_256x160, DL_TILES };
+static const int DL_BM[DL_TILES] = {64, 64, 128, 128, 256, 192, 256, 256, 64, 128, 64, 128, 64, 256, 256};
+static const int DL_BN[DL_TILES] = {64, 256, 128, 256, 128, 256, 192, 256, 128, 128, 192, 192, 320, 320, 160};
+static const double DL_RATE[DL_TILES] = {2.45e12, 3.3e12, 4.2e12, 4.6e12, 4.8e12, 5.2e12, 5.2e12, 6.1e12, 2.1e12, 4.2e12, 3.0e12, 4.4e12, 3.5e12, 5.5e12, 4.3e12};   // FLOP/s of one compute unit
+static const double DL_FIXED[DL_TILES] = {2.7e-6, 11.5e-6, 5.5e-6, 11e-6, 15e-6, 6e-6, 8e-6, 14e-6, 5e-6, 4.5e-6, 9e-6, 9e-6, 12e-6, 10e-6, 10e-6};       // seconds per tile
 
 // Seconds for `groups` work-groups of tile t over k columns each.  The two smallest tiles run two
 // to a compute unit: each then works at half the unit's rate, and one that has a unit to itself
@@ -1532,7 +1538,7 @@ static DlTile pick_dl_tile(int M, int N, int K, bool sw, double* estimate = null
     DlTile best = DL_128x128;
     double best_t = 1e30;
     for (int t = 0; t < DL_TILES; ++t) {
-        if (sw && (t == DL_64x64 || t == DL_256x192 || t == DL_64x320)) continue;      // a wave of the fused gate needs whole 64-row blocks of weights
+        if (sw && (t == DL_64x64 || t == DL_256x192 || t == DL_64x320 || t == DL_256x160)) continue;      // a wave of the fused gate needs whole 64-row blocks of weights
         if (t == DL_256x320) continue;      // float slabs of partial sums only: a bfloat16 result tile of 160 KB does not fit its slab buffers
         const long tiles = (long)((M + DL_BM[t] - 1) / DL_BM[t]) * ((N + DL_BN[t] - 1) / DL_BN[t]);
         if (t == DL_128x128_S4 && (tiles > TL_COMPUTE_UNITS || M > 128)) continue;      // one round of work-groups, every weight drawn once
@@ -1616,6 +1622,9 @@ static int launch_dl_tile(DlTile tile, const void* x, const void* w, const void*
         if constexpr (!SW) return launch_dl_tile_t<256, 192, 4, 2, 2, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
         else break;
     case DL_256x256: return launch_dl_tile_t<256, 256, 4, 2, 2, TOut, SW>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+    case DL_256x160:
+        if constexpr (!SW) return launch_dl_tile_t<256, 160, 4, 1, 2, TOut, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
+        else break;
     case DL_256x320:
         if constexpr (!SW && sizeof(TOut) == 4) return launch_dl_tile_t<256, 320, 4, 2, 2, float, false>(x, w, bias, bias_f32, out, M, N, K, ldx, ldo, out_cols, stream, parts, k_per);
         else break;
@@ -1665,7 +1674,7 @@ extern "C" int tl_gemm_swiglu_direct_variant(const void* x, const void* w, void*
                "gemm_swiglu_direct: needs M > 0, K a multiple of 64 and 16-byte aligned rows");
     int tile = -1;
     for (int t = 0; t < DL_TILES; ++t)
-        if (DL_BM[t] == BM && DL_BN[t] == BN && t != DL_128x128_S4 && t != DL_64x64 && t != DL_256x192 && t != DL_64x320 && t != DL_256x320) tile = t;
+        if (DL_BM[t] == BM && DL_BN[t] == BN && t != DL_128x128_S4 && t != DL_64x64 && t != DL_256x192 && t != DL_64x320 && t != DL_256x320 && t != DL_256x160) tile = t;
     TL_REQUIRE(tile >= 0, "gemm_swiglu_direct: no tile of %d x %d with the fused gate", BM, BN);
     const int N = ((I + 31) / 32) * 64;
     const int rc = launch_dl_tile<bf16_t, true>((DlTile)tile, x, w, nullptr, 0, out, M, N, K, ldx, ldo, I, stream);

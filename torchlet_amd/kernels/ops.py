@@ -250,7 +250,7 @@ def linear_many_rows_variant(x, weight, bias, out, tile_m: int, tile_n: int, sla
                                          c_int(1 if out.dtype == torch.float32 else 0), c_int(tile_m), c_int(tile_n), c_int(slab), _stream()))
 
 
-DIRECT_TILES = ((64, 64), (64, 128), (64, 192), (64, 256), (64, 320), (128, 128), (128, 192), (128, 256), (256, 128), (192, 256), (256, 192), (256, 256))
+DIRECT_TILES = ((64, 64), (64, 128), (64, 192), (64, 256), (64, 320), (128, 128), (128, 192), (128, 256), (256, 128), (192, 256), (256, 192), (256, 256), (256, 160))
 
 
 def linear_direct_variant(x, weight, bias, out, tile_m: int, tile_n: int) -> None:

@@ -324,6 +324,20 @@ def test_linear_many_rows_fetched_straight_into_shared_memory(ops, out_dtype, ti
     assert bool((out2[:, N:] == 5.0).all())
 
 
+def test_the_tile_product_refuses_rows_too_far_apart_for_its_32_bit_offsets(ops):
+    """A lane of the direct-load kernel addresses its piece as a shared base plus a 32-bit offset from the tile's first
+    row: rows of x that lie 2^23 elements apart put a tile's last row beyond that, and the launcher says so."""
+    K, N = 64, 64
+    store = torch.zeros(2 * (1 << 23), dtype=torch.bfloat16, device="cuda")
+    x = store.view(2, 1 << 23)[:, :K]                       # two rows, 2^23 elements from one to the next
+    w = torch.zeros(N, K, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty(2, N, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ops.KernelError, match="too long"):
+        ops.linear_direct_variant(x, w, None, out, 256, 256)
+    ops.linear_direct_variant(x, w, None, out, 64, 64)      # a tile of 64 rows reaches a quarter as far
+    assert bool((out == 0).all())
+
+
 @pytest.mark.parametrize("tile", [(64, 64, 0), (64, 192, 0), (64, 320, 0), (128, 192, 0), (128, 128, 0), (128, 128, 4), (128, 256, 0), (256, 128, 0), (192, 256, 0), (256, 192, 0), (256, 256, 0), (256, 320, 0), (256, 160, 0)])
 @pytest.mark.parametrize("M,N,K,parts", [(65, 129, 128, 2), (128, 520, 1024, 4), (100, 3584, 2048, 8), (300, 257, 1088, 3), (7, 48, 3584, 7)])
 def test_linear_split_over_k_on_every_tile_shape(ops, tile, M, N, K, parts):

@@ -324,6 +324,24 @@ def test_linear_many_rows_fetched_straight_into_shared_memory(ops, out_dtype, ti
     assert bool((out2[:, N:] == 5.0).all())
 
 
+@pytest.mark.parametrize("M", [2048, 4096])
+@pytest.mark.parametrize("N,K", [(5120, 1024), (7168, 640), (4608, 1088)])
+def test_linear_of_thousands_of_rows_against_narrow_matrices_whatever_tile_it_picks(ops, M, N, K):
+    """Whole prompt portions against matrices for which the planner weighs its widest tiles against each other (256 x 256,
+    256 x 160, 192 x 256; one round of tiles or two): whichever it takes, the product is the product."""
+    g = torch.Generator(device="cuda").manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g, device="cuda").to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g, device="cuda") / math.sqrt(K)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g, device="cuda").to(torch.bfloat16)
+    ref = x.double() @ w.double().T + b.double()
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops.linear(x, w, b, out)
+    torch.testing.assert_close(out.double(), ref, **_tol(torch.bfloat16))
+    parts = ops.linear_partials(x, w)
+    tol32 = dict(rtol=2e-5, atol=8 * 2 ** -24 * math.sqrt(K) * float(ref.pow(2).mean().sqrt()))
+    torch.testing.assert_close(parts.double().sum(0), ref - b.double(), **tol32)
+
+
 def test_the_tile_product_refuses_rows_too_far_apart_for_its_32_bit_offsets(ops):
     """A lane of the direct-load kernel addresses its piece as a shared base plus a 32-bit offset from the tile's first
     row: rows of x that lie 2^23 elements apart put a tile's last row beyond that, and the launcher says so."""

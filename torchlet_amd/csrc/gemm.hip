@@ -1338,9 +1338,13 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
     // last ones arrive too late).  Past the end the last slab is requested again (nobody reads it), so the count
     // of requests in flight is the same in every step, which the wait relies on.
     Frag16 af[2][FM], bfr[2][FN];
-    constexpr int L_LAST = (LOADS + 1) / 2;                 // requests of a slab issued in the last phase of a step; the rest in the next step's first
+    // requests of a slab issued in the last phase of a step; the rest in the next step's first.  (Not for the smallest tile,
+    // four requests a wave and slab: split in two they made the decode step's products over K a fiftieth slower.)
+    constexpr int L_LAST = LOADS >= 6 ? (LOADS + 1) / 2 : LOADS;
     auto request = [&](int slab, int j) {
-        const bf16_t* from = ((of_x >> j) & 1 ? xt : wt) + min(slab, slabs - 1) * TK;
+        // (which operand request j fetches is known at compile time where the waves' requests cover whole multiples of x's rows)
+        const bool from_x = BM % (RPL * NW) == 0 ? j < BM / (RPL * NW) : (bool)((of_x >> j) & 1);
+        const bf16_t* from = (from_x ? xt : wt) + min(slab, slabs - 1) * TK;
         load_to_lds_at(from, soff[j], lds_base + (slab % STAGES) * LROWS * TK * 2 + ldst[j]);
     };
 #pragma unroll

@@ -1383,6 +1383,28 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dl_tile_kernel(const bf16
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if constexpr (NM == 1) {
+                // One product a phase (the smallest tile): a phase's memory instructions first, then its product, which
+                // covers them; but for the step's first phase, whose product comes first so that the wait at the loop's
+                // head is for that product's operands alone.
+                if (kk == 0) {
+                    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0].v, af[cur][0].v, acc[0][0], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int op = 0; op < ops; ++op) {
+                    const int r = op - nl;
+                    if (r < 0) request(slab_of, lfirst + op);
+                    else if (r < FM) af[nxt][r].u = *(const uint4*)(nb + arow[r] * TK + ((c ^ akey[r]) * 8));
+                    else bfr[nxt][r - FM].u = *(const uint4*)(nb + brow[r - FM] * TK + ((c ^ bkey[r - FM]) * 8));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (kk > 0) {
+                    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[cur][0].v, af[cur][0].v, acc[0][0], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                continue;
+            }
             int op = 0;
 #pragma unroll
             for (int q = 0; q < NM; ++q) {

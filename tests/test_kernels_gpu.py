@@ -863,6 +863,7 @@ def test_paged_attention_prompt_portions(ops, nh, nkv, hd, page, window):
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [
     (28, 4, 128, 16, 0), (20, 1, 64, 16, 0), (40, 8, 128, 8, 0), (4, 4, 64, 32, 0), (130, 1, 64, 16, 0),
     (14, 2, 128, 64, 40), (4, 4, 64, 32, 29), (6, 2, 128, 8, 100),
+    (28, 4, 128, 128, 0), (6, 2, 64, 256, 100),              # pages longer than a step: steps begin inside a page
 ])
 def test_paged_attention_prompt_tiles_of_128_rows(ops, nh, nkv, hd, page, window):
     """The 128-row kernel for prompt portions: whole prompts, portions on top of a cached context

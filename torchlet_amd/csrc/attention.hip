@@ -258,6 +258,16 @@ union FragK {
 #define ATM_BT_MAX 2048                    // block-table entries a work-group keeps in shared memory
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// The larger of a lane's value and that of lane ^ 32 (lane ^ 16): the halves (the rows of 16 lanes) change places in
+// the vector unit, where a shuffle would go through shared memory and the step would wait for the trip.
+__device__ __forceinline__ float max_across_halves(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_across_rows(float x) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
 
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void paged_attention_mfma_kernel(AttnArgs a) {
@@ -419,8 +429,7 @@ __global__ __launch_bounds__(64 * NW) void paged_attention_mfma_kernel(AttnArgs 
                     mloc = fmaxf(mloc, x);
                 }
         }
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, TL_WAVE));
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TL_WAVE));
+        mloc = max_across_halves(max_across_rows(mloc));
         const float m_new = fmaxf(m, mloc);
         const float alpha = (m == -INFINITY) ? 0.f : fast_exp2(m - m_new);
         FragK pf;
@@ -686,8 +695,7 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_kernel(AttnArgs a
                         mloc = fmaxf(mloc, x);
                     }
             }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, TL_WAVE));
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TL_WAVE));
+            mloc = max_across_halves(max_across_rows(mloc));
             const float m_new = fmaxf(m, mloc);
             const float alpha = (m == -INFINITY) ? 0.f : fast_exp2(m - m_new);
             FragK pf;
@@ -949,8 +957,10 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     // second is zero for pages of up to ATQ_KEYS keys, of the two lane parts the first is zero for longer ones).  A
     // step then costs a lane one look-up of a page and one multiply-add per address.  (With all of it computed in the
     // step, the addresses were a quarter of the loop's vector instructions.)
-    const bf16_t* k_src[K_INSTR];              // K row of key x, this lane's piece, in page 0
-    const bf16_t* v_src[K_INSTR];              // V^T row d, this lane's eight keys, in page 0
+    // A page's keys (values) of all heads are kv_stride elements; the host checked that twice that fits 32 bits, so an
+    // address is ONE 64-bit multiply-add of page number and stride on what was worked out here.
+    unsigned long long k_src[K_INSTR];         // address of: K row of key x, this lane's piece, in page 0
+    unsigned long long v_src[K_INSTR];         // V^T row d, this lane's eight keys, in page 0
     int k_blk[K_INSTR];                        // x >> shift
     unsigned k_dst[K_INSTR];
     int v_blk;                                 // the same for every value load of a lane (its piece's slot depends on d / 2 mod 8 only)
@@ -959,40 +969,46 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
         const int ii = wave + 4 * j;
         const int kx = KPI * ii + lane / KPP;
         k_blk[j] = kx >> shift;
-        k_src[j] = kp + kvh_off + (kx & pmask) * AT_HD + atq_key_slot(lane % KPP, kx) * 8;       // exclusive-or is its own inverse
+        k_src[j] = (unsigned long long)(uintptr_t)(kp + kvh_off + (kx & pmask) * AT_HD + atq_key_slot(lane % KPP, kx) * 8);   // exclusive-or is its own inverse
         const int d = VDI * ii + lane / ATQ_VPP;
         const int vx = 8 * atq_value_slot(lane % ATQ_VPP, d);           // first of the piece's eight keys
         if (j == 0) v_blk = vx >> shift;
-        v_src[j] = vp + kvh_off + d * page + (vx & pmask);
+        v_src[j] = (unsigned long long)(uintptr_t)(vp + kvh_off + d * page + (vx & pmask));
         k_dst[j] = __builtin_amdgcn_readfirstlane(ii * 1024);
     }
     const int blk_last = blk_n - 1;
+    const unsigned page_bytes = (unsigned)kv_stride * 2u;
+    // The pages of a step are looked up one request early and kept in registers: looked up where they are needed, each
+    // of the five look-ups stood between a request and the one before it, with the trip to shared memory in full.
     // (a block beyond the sequence's last is read as the last: the step that holds the sequence's end may reach past
     // its last page; those keys' scores are masked and their values cleared below)
-    auto request = [&](int st, int buf, auto long_pages) {
-        const int kbase = st * ATQ_KEYS;
+    // Look-ups and requests come one at a time (j: the step's K_INSTR key loads, then its value loads), for the loop
+    // to place them between its products.
+    int pg_k[K_INSTR], pg_v;
+    const bool long_pages = page > ATQ_KEYS;                              // (uniform)
+    auto look_up_one = [&](int st, int j) {
+        const int ub = ((st * ATQ_KEYS) >> shift) - blk0;                // uniform: the step's first block in bt_s
+        if (j < K_INSTR) pg_k[j] = bt_s[min(ub + k_blk[j], blk_last)];
+        else pg_v = bt_s[min(ub + v_blk, blk_last)];
+    };
+    auto look_up = [&](int st) {
+#pragma unroll
+        for (int j = 0; j <= K_INSTR; ++j) look_up_one(st, j);
+    };
+    auto request_one = [&](int st, int buf, int j) {                    // (after look_up(st))
         const unsigned sb = lds_base + buf * ATQ_STAGE;
-        const int ub = (kbase >> shift) - blk0;                          // uniform: the step's first block in bt_s
-        const int uin = long_pages ? kbase & pmask : 0;                  // uniform: its first key's place in that block's page
-#pragma unroll
-        for (int j = 0; j < K_INSTR; ++j) {
-            const int pg = bt_s[min(ub + k_blk[j], blk_last)];
-            const bf16_t* src = k_src[j] + (size_t)(unsigned)pg * kv_stride;
-            if (long_pages) src += uin * AT_HD;
-            attn_load_to_lds(src, sb + k_dst[j]);
-        }
-        const int pg = bt_s[min(ub + v_blk, blk_last)];
-#pragma unroll
-        for (int j = 0; j < K_INSTR; ++j) {
-            const bf16_t* src = v_src[j] + (size_t)(unsigned)pg * kv_stride;
-            if (long_pages) src += uin;
-            attn_load_to_lds(src, sb + ATQ_KBYTES + k_dst[j]);
+        const unsigned uin = long_pages ? (st * ATQ_KEYS) & pmask : 0;   // uniform: the step's first key's place in its page
+        if (j < K_INSTR) {
+            const unsigned long long src = k_src[j] + (unsigned long long)(unsigned)pg_k[j] * page_bytes + uin * (AT_HD * 2);
+            attn_load_to_lds((const void*)(uintptr_t)src, sb + k_dst[j]);
+        } else {
+            const unsigned long long v_page = (unsigned long long)(unsigned)pg_v * page_bytes + uin * 2;
+            attn_load_to_lds((const void*)(uintptr_t)(v_src[j - K_INSTR] + v_page), sb + ATQ_KBYTES + k_dst[j - K_INSTR]);
         }
     };
-    const bool long_pages = page > ATQ_KEYS;                              // (uniform)
     auto request_step = [&](int st, int buf) {
-        if (long_pages) request(st, buf, std::true_type{});
-        else request(st, buf, std::false_type{});
+#pragma unroll
+        for (int j = 0; j < 2 * K_INSTR; ++j) request_one(st, buf, j);
     };
 
     const float scale2 = a.scale * 1.44269504088896341f;
@@ -1010,13 +1026,18 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     // again (nobody reads it), so that the number of requests in flight is the same at every wait.
     if (any_step) {
 #pragma unroll
-        for (int i = 0; i < ATQ_STAGES - 1; ++i) request_step(min(st_first + i, st_last - 1), i);
+        for (int i = 0; i < ATQ_STAGES - 1; ++i) {
+            look_up(min(st_first + i, st_last - 1));
+            request_step(min(st_first + i, st_last - 1), i);
+        }
+        look_up(min(st_first + ATQ_STAGES - 1, st_last - 1));
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * K_INSTR * (ATQ_STAGES - 2)) : "memory");
         __syncthreads();
     }
     for (int st = st_first; st < st_last; ++st) {
         const int buf = (st - st_first) % ATQ_STAGES;
-        request_step(min(st + ATQ_STAGES - 1, st_last - 1), (st - st_first + ATQ_STAGES - 1) % ATQ_STAGES);
+        const int st_req = min(st + ATQ_STAGES - 1, st_last - 1), buf_req = (st - st_first + ATQ_STAGES - 1) % ATQ_STAGES;
+        const int st_look = min(st + ATQ_STAGES, st_last - 1);
         const int kbase = st * ATQ_KEYS;
         unsigned char* kb_s = atq_smem + buf * ATQ_STAGE;
         unsigned char* vb_s = kb_s + ATQ_KBYTES;
@@ -1058,6 +1079,8 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
 #pragma unroll
                 for (int kb = 0; kb < ATQ_KB; ++kb) read_keys(c, kb);
             __builtin_amdgcn_sched_barrier(0);
+            // (the requests of the step ahead go between the products, one beside every other product)
+            static_assert(AT_HD / 16 * ATQ_KB >= 4 * K_INSTR, "a request beside every other product");
 #pragma unroll
             for (int c = 0; c < AT_HD / 16; ++c)
 #pragma unroll
@@ -1065,6 +1088,8 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
                     sc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[c % (KAHEAD + 1)][kb].v, qf[c].v, sc[kb], 0, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
                     if (c + KAHEAD < AT_HD / 16) read_keys(c + KAHEAD, kb);
+                    const int slot = c * ATQ_KB + kb;
+                    if (slot % 2 == 0 && slot / 2 < 2 * K_INSTR) request_one(st_req, buf_req, slot / 2);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             // ---- mask, maximum, probabilities.  Element (kb, 4 q + v) of this lane is key
@@ -1089,7 +1114,7 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
                         mloc = fmaxf(mloc, sc[kb][e]);
                     }
             }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, TL_WAVE)) * scale2;
+            mloc = max_across_halves(mloc) * scale2;
             // m is the row's reference for the exponents, not its running maximum: it moves only when some row of
             // the wave has a score more than ATQ_SLACK (in powers of two) above its reference, so most steps rescale
             // nothing; until then probabilities are up to 2^ATQ_SLACK instead of up to 1, which 32-bit sums and the
@@ -1105,25 +1130,45 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
             const float m_use = (m == -INFINITY) ? 0.f : -m;           // nothing seen yet: every score is -inf
             FragK pf[2 * ATQ_KB];
             float psum = 0.f;
+            auto probabilities = [&](int kb, int e0, int n) {
 #pragma unroll
-            for (int kb = 0; kb < ATQ_KB; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
+                for (int e = e0; e < e0 + n; ++e) {
                     const float p = fast_exp2(__builtin_fmaf(sc[kb][e], scale2, m_use));
                     psum += p;
                     pf[2 * kb + (e >> 3)].v[e & 7] = (__bf16)p;
                 }
+            };
+            // ---- values.  Product i takes the values of d = 32 (i % NB) .. + 32 for the 16 keys of chunk i / NB; the
+            // values are read two products ahead.  Only the first block's probabilities are worked out before the
+            // products begin: those of each later block go beside the products of the block before it, and the
+            // look-ups of the pages that the next step requests beside the products of the last block, so that the
+            // vector unit works while the matrix unit does.
+            constexpr int NB = AT_HD / 32, NPV = 2 * ATQ_KB * NB, VAHEAD = 2;
+            constexpr int PER = 16 / (2 * NB);                     // probabilities beside one product
+            static_assert(2 * NB >= K_INSTR + 1, "a look-up beside each product of the last block");
+            FragK vfb[VAHEAD + 1];
+            auto read_values = [&](int i) {
+                const int d = 32 * (i % NB) + lr;
+                vfb[i % (VAHEAD + 1)].u = *(const uint4*)(vb_s + d * ATQ_VROW + atq_value_slot(2 * (i / NB) + h, d) * 16);
+            };
+#pragma unroll
+            for (int i = 0; i < VAHEAD; ++i) read_values(i);
+            probabilities(0, 0, 16);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < NPV; ++i) {
+                acc[i % NB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfb[i % (VAHEAD + 1)].v, pf[i / NB].v, acc[i % NB], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (i + VAHEAD < NPV) read_values(i + VAHEAD);
+                const int kb = i / (2 * NB), within = i % (2 * NB);
+                if (kb + 1 < ATQ_KB) probabilities(kb + 1, within * PER, PER);
+                else if (within <= K_INSTR) look_up_one(st_look, within);
+                __builtin_amdgcn_sched_barrier(0);
+            }
             l += psum;
-            // ---- values
-#pragma unroll
-            for (int c4 = 0; c4 < 2 * ATQ_KB; ++c4)
-#pragma unroll
-                for (int b = 0; b < AT_HD / 32; ++b) {
-                    const int d = 32 * b + lr;
-                    FragK vf;
-                    vf.u = *(const uint4*)(vb_s + d * ATQ_VROW + atq_value_slot(2 * c4 + h, d) * 16);
-                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[c4].v, acc[b], 0, 0, 0);
-                }
+        } else {
+            request_step(st_req, buf_req);
+            look_up(st_look);
         }
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * K_INSTR * (ATQ_STAGES - 2)) : "memory");
         __syncthreads();
@@ -1193,6 +1238,7 @@ extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out,
     // used_blocks: the most block-table entries any request of the step uses (its length in pages)
     TL_REQUIRE(bt_stride > 0 && used_blocks > 0 && used_blocks <= ATM_BT_MAX,
                "attention_prompt: sequences of up to %d pages, not %d", ATM_BT_MAX, used_blocks);
+    TL_REQUIRE((long)kv_heads * page * AT_HD * 2 < (1L << 32), "attention_prompt: a page of %d heads x %d tokens is too large", kv_heads, page);
     const int group = heads / kv_heads;
     const int gcap = group < ATQ_ROWS ? group : ATQ_ROWS;
     TL_REQUIRE(tq * gcap <= ATQ_ROWS, "attention_prompt: tile of %d tokens x %d heads exceeds %d rows", tq, gcap, ATQ_ROWS);

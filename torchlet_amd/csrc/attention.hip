@@ -45,6 +45,7 @@ struct AttnArgs {
     int q_stride, bt_stride, heads, kv_heads, page, window, tq, gcap, splits;
     int hd;                   // the true head size, <= HD: width of a head in q, out and the planes
     int page_shift;           // log2(page) when page is a power of two, else -1
+    int units;                // compute units of the GPU (the prompt kernel's order of work)
     float scale;
 };
 
@@ -873,7 +874,15 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     // a 2048-token prompt 83 -> 75 us, 4096 tokens 231 -> 180 us, 2048 tokens with 40 heads in 8 groups
     // 102 -> 81 us).
     const int per_tile = gridDim.y;
-    const int rank = blockIdx.y * gridDim.x + blockIdx.x;
+    // With more work-groups than compute units, but no more than fit at once (two a unit), nothing is handed out
+    // later to even things out: unit u runs the u-th work-group and the (units + u)-th, so the second batch
+    // runs from light to heavy and every unit gets a heavy tile and a light one (2048 tokens, 28 heads in 4
+    // groups, 256 units: 456 work-groups, 51 -> 49 us).
+    int rank = blockIdx.y * gridDim.x + blockIdx.x;
+    {
+        const int n = gridDim.x * gridDim.y;
+        if (gridDim.z == 1 && n <= 2 * a.units && rank >= a.units) rank = n - 1 - (rank - a.units);
+    }
     const int tile = gridDim.x - 1 - rank / per_tile;
     const int by = rank % per_tile;
     const int group = a.heads / a.kv_heads;
@@ -1255,6 +1264,14 @@ extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out,
     a.q_stride = q_stride; a.bt_stride = bt_stride; a.heads = heads; a.kv_heads = kv_heads; a.page = page;
     a.window = window; a.tq = tq; a.gcap = gcap; a.splits = splits; a.scale = scale; a.hd = AT_HD;
     a.page_shift = (page & (page - 1)) == 0 ? __builtin_ctz(page) : -1;
+    static int units = 0;                        // (of the device of the first call: one kind of GPU in a process)
+    if (units == 0) {
+        int dev = 0, n = 0;
+        TL_REQUIRE(hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0,
+                   "attention_prompt: cannot ask the device for its compute units");
+        units = n;
+    }
+    a.units = units;
     const int chunks = (group + gcap - 1) / gcap;
     static hipError_t allowed = hipFuncSetAttribute((const void*)paged_attention_prompt_kernel,
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, ATQ_SMEM);

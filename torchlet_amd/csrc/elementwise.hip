@@ -341,6 +341,16 @@ void rope_cache_write_rows_kernel(bf16_t* __restrict__ qkv, int row_stride, int 
     if (k_plane) page_base = (size_t)block_table[(size_t)token_req[t] * bt_stride + pos / page_size] * kv_heads * page_size * head_dim;
     const bool stores = k_plane && page_base != 0;                 // page 0 is the sentinel: never written
     const int off = pos % page_size;
+    // The token's cosines and sines are worked out once, not once a head: the same 32-bit angle and functions, read
+    // back from shared memory by every head's threads (28 query heads and 4 key heads of 128: 2048 tokens 17 -> 12 us).
+    __shared__ float2 turn[128];                                   // (head_dim <= 256: the host checks)
+    if (inv_freq) {
+        for (int j = threadIdx.x; j < head_dim / 2; j += 256) {
+            const float angle = (float)pos * inv_freq[j];
+            turn[j] = make_float2(cosf(angle), sinf(angle));
+        }
+        __syncthreads();
+    }
     for (int p = threadIdx.x; p < heads * pph; p += 256) {
         const int head = p / pph, d0 = (p % pph) * 8;
         union { uint4 u; uint16_t e[8]; } piece;
@@ -355,16 +365,14 @@ void rope_cache_write_rows_kernel(bf16_t* __restrict__ qkv, int row_stride, int 
         }
         const bool rotate = inv_freq && head < rot_heads;
         if (rotate) {
-            const float4 f = *(const float4*)(inv_freq + d0 / 2);
-            const float freq[4] = {f.x, f.y, f.z, f.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 bf16_t a, b;
                 a.bits = piece.e[2 * j];
                 b.bits = piece.e[2 * j + 1];
                 float x1 = to_float(a), x2 = to_float(b);
-                const float angle = (float)pos * freq[j];
-                rope_turn(x1, x2, cosf(angle), sinf(angle));
+                const float2 cs = turn[d0 / 2 + j];
+                rope_turn(x1, x2, cs.x, cs.y);
                 piece.e[2 * j] = from_float<bf16_t>(x1).bits;
                 piece.e[2 * j + 1] = from_float<bf16_t>(x2).bits;
             }

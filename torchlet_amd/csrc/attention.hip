@@ -854,6 +854,11 @@ __device__ __forceinline__ void attn_load_to_lds(const void* gptr, unsigned lds_
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
 
+// The same from a base that the wave shares plus 32 bits of each lane's own.
+__device__ __forceinline__ void attn_load_to_lds_at(const void* base, unsigned offset, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(offset), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
+
 __device__ __forceinline__ int atq_key_slot(int piece, int key) {        // slot of a 16-byte piece in its key row
     return AT_HD == 128 ? (piece ^ (key & 15)) : (piece ^ ((key >> 1) & 7));
 }
@@ -861,6 +866,9 @@ __device__ __forceinline__ int atq_value_slot(int piece, int d) {        // ... 
     return ATQ_KEYS == 64 ? (piece ^ ((d >> 1) & 7)) : (piece ^ ((d >> 2) & 3));
 }
 
+// LONG: pages of more than ATQ_KEYS keys, where a step begins inside a page (an addition per address that the usual
+// short pages are spared).
+template <bool LONG>
 __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char atq_smem[];
     int* bt_s = (int*)(atq_smem + ATQ_STAGES * ATQ_STAGE);
@@ -968,7 +976,9 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     // step, the addresses were a quarter of the loop's vector instructions.)
     // A page's keys (values) of all heads are kv_stride elements; the host checked that twice that fits 32 bits, so an
     // address is ONE 64-bit multiply-add of page number and stride on what was worked out here.
-    unsigned long long k_src[K_INSTR];         // address of: K row of key x, this lane's piece, in page 0
+    // The keys of one load instruction (1024 bytes: 4 or 8 rows) lie in one page, pages being of 8 keys or more: their
+    // page's address is the wave's, worked out by the scalar unit, and a lane adds 32 bits that never change.
+    unsigned k_off[K_INSTR];                   // K row of key x, this lane's piece: bytes from the start of its head's page
     unsigned long long v_src[K_INSTR];         // V^T row d, this lane's eight keys, in page 0
     int k_blk[K_INSTR];                        // x >> shift
     unsigned k_dst[K_INSTR];
@@ -978,7 +988,7 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
         const int ii = wave + 4 * j;
         const int kx = KPI * ii + lane / KPP;
         k_blk[j] = kx >> shift;
-        k_src[j] = (unsigned long long)(uintptr_t)(kp + kvh_off + (kx & pmask) * AT_HD + atq_key_slot(lane % KPP, kx) * 8);   // exclusive-or is its own inverse
+        k_off[j] = (unsigned)((kx & pmask) * AT_HD + atq_key_slot(lane % KPP, kx) * 8) * 2u;       // exclusive-or is its own inverse
         const int d = VDI * ii + lane / ATQ_VPP;
         const int vx = 8 * atq_value_slot(lane % ATQ_VPP, d);           // first of the piece's eight keys
         if (j == 0) v_blk = vx >> shift;
@@ -994,7 +1004,6 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     // Look-ups and requests come one at a time (j: the step's K_INSTR key loads, then its value loads), for the loop
     // to place them between its products.
     int pg_k[K_INSTR], pg_v;
-    const bool long_pages = page > ATQ_KEYS;                              // (uniform)
     auto look_up_one = [&](int st, int j) {
         const int ub = ((st * ATQ_KEYS) >> shift) - blk0;                // uniform: the step's first block in bt_s
         if (j < K_INSTR) pg_k[j] = bt_s[min(ub + k_blk[j], blk_last)];
@@ -1006,10 +1015,11 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     };
     auto request_one = [&](int st, int buf, int j) {                    // (after look_up(st))
         const unsigned sb = lds_base + buf * ATQ_STAGE;
-        const unsigned uin = long_pages ? (st * ATQ_KEYS) & pmask : 0;   // uniform: the step's first key's place in its page
+        const unsigned uin = LONG ? (st * ATQ_KEYS) & pmask : 0;         // uniform: the step's first key's place in its page
         if (j < K_INSTR) {
-            const unsigned long long src = k_src[j] + (unsigned long long)(unsigned)pg_k[j] * page_bytes + uin * (AT_HD * 2);
-            attn_load_to_lds((const void*)(uintptr_t)src, sb + k_dst[j]);
+            const unsigned pg = __builtin_amdgcn_readfirstlane(pg_k[j]);
+            const unsigned long long src = (unsigned long long)(uintptr_t)(kp + kvh_off) + (unsigned long long)pg * page_bytes + uin * (AT_HD * 2);
+            attn_load_to_lds_at((const void*)(uintptr_t)src, k_off[j], sb + k_dst[j]);
         } else {
             const unsigned long long v_page = (unsigned long long)(unsigned)pg_v * page_bytes + uin * 2;
             attn_load_to_lds((const void*)(uintptr_t)(v_src[j - K_INSTR] + v_page), sb + ATQ_KBYTES + k_dst[j - K_INSTR]);
@@ -1273,10 +1283,13 @@ extern "C" int tl_paged_attention_prompt(const void* q, int q_stride, void* out,
     }
     a.units = units;
     const int chunks = (group + gcap - 1) / gcap;
-    static hipError_t allowed = hipFuncSetAttribute((const void*)paged_attention_prompt_kernel,
+    static hipError_t allowed = hipFuncSetAttribute((const void*)paged_attention_prompt_kernel<false>,
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, ATQ_SMEM);
-    TL_REQUIRE(allowed == hipSuccess, "attention_prompt: cannot get %d bytes of shared memory", ATQ_SMEM);
-    paged_attention_prompt_kernel<<<dim3(tiles, kv_heads * chunks, splits), dim3(256), ATQ_SMEM, stream>>>(a);
+    static hipError_t allowed_long = hipFuncSetAttribute((const void*)paged_attention_prompt_kernel<true>,
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, ATQ_SMEM);
+    TL_REQUIRE(allowed == hipSuccess && allowed_long == hipSuccess, "attention_prompt: cannot get %d bytes of shared memory", ATQ_SMEM);
+    if (page > ATQ_KEYS) paged_attention_prompt_kernel<true><<<dim3(tiles, kv_heads * chunks, splits), dim3(256), ATQ_SMEM, stream>>>(a);
+    else paged_attention_prompt_kernel<false><<<dim3(tiles, kv_heads * chunks, splits), dim3(256), ATQ_SMEM, stream>>>(a);
     TL_CHECK_LAUNCH("paged_attention_prompt");
     if (splits > 1) {
         launch_merge(part_o, part_ml, out, splits, merge_tokens, heads, (long)merge_count * heads, false, stream);

@@ -76,7 +76,7 @@ def test_registry(tmp_path):
 
 
 def test_run_order_is_checked():
-    from torchlet_amd.config import ModelSpec, RunEntry
+    from torchlet_amd.config import RunEntry
     spec = Qwen2Config.from_dict(REF_TINY).to_spec()
     import dataclasses
     dataclasses.replace(spec, order=(RunEntry(0), RunEntry(0), RunEntry(0, cache_of=0)))   # a layer twice, a shared cache
@@ -305,7 +305,7 @@ def test_dtype_policy_of_a_tensor_is_apart_from_its_shape_and_laws_are_named():
 def test_every_part_is_asked_whether_a_step_may_be_recorded():
     """Not the mixers alone: a feed-forward, a norm or a position encoding that reads values of the step on the host
     keeps the whole model off graphs.  ``False`` is the default of a part; the built-in parts say ``True``."""
-    from torchlet_amd.parts import FEED_FORWARDS, FeedForward, Part
+    from torchlet_amd.parts import FeedForward, Part
     from torchlet_amd.parts.base import LazyNorm, Stream
     assert Part.graph_safe is False
     model = _model(REF_TINY)

@@ -1,7 +1,6 @@
 """The engine's own configuration (no GPU): defaults after the reference's rules, validation, and what
 the scheduler and the step function make of ``max_model_len``."""
 import pytest
-import torch
 
 from torchlet_amd.cache.manager import CacheManager
 from torchlet_amd.engine.config import EngineConfig

@@ -1,7 +1,5 @@
 """Each part alone on the GPU against its plain formula, at sizes of its own, and a toy
 mixer with fixed-size state registered from outside the framework."""
-import dataclasses
-import math
 from dataclasses import dataclass
 from typing import ClassVar
 

@@ -3,7 +3,6 @@ routines it must reduce to, invariants, and the vectors the reference's own file
 Each check is chosen so that a plausible mistake fails it."""
 import math
 
-import pytest
 import torch
 import torch.nn.functional as F
 

@@ -3,12 +3,10 @@ cutting the same requests into steps, in 32-bit and in bfloat16."""
 import json
 import os
 import subprocess
-import sys
 from pathlib import Path
 
 import numpy as np
 import pytest
-import torch
 
 import scenarios
 import tiny_models

@@ -23,8 +23,6 @@ import json
 import sys
 from pathlib import Path
 
-import numpy as np
-
 
 def parse_args(argv=None):
     p = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])

@@ -33,8 +33,6 @@ import json
 import sys
 from pathlib import Path
 
-import torch
-
 from .engine.config import EngineConfig
 from .engine.loading import load_model, make_engine, require_gpu
 from .engine.request import Request

@@ -871,9 +871,25 @@ def test_paged_attention_prompt_tiles_of_128_rows(ops, nh, nkv, hd, page, window
     1, 3, 5, 7, 20 and 130 heads.  Places of the pages that hold no key yet are filled with NaN:
     nothing of them may reach a result."""
     assert ops.prompt_attention_fits(torch.bfloat16, hd, page) and not ops.prompt_attention_fits(torch.bfloat16, hd, 24)
+    _prompt_tiles_case(ops, nh, nkv, hd, page, window, [150, 37, 70, 1, 64, 300], [0, 150, 43, 99, 64, 5])
+
+
+def test_paged_attention_prompt_with_more_tiles_than_compute_units_but_no_more_than_fit_at_once(ops):
+    """Between one and two work-groups a compute unit the kernel runs its second batch of tiles from light to
+    heavy: four requests of different lengths, 96 tiles of 18 tokens for each of 4 key/value heads, and the
+    same split over the keys (then the order is the plain one)."""
+    nh, nkv = 28, 4
+    lens = [700, 500, 300, 200]
+    tiles = sum(-(-n // ops.prompt_attention_tile_tokens(nh, nkv)) for n in lens) * nkv
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    if not units < tiles <= 2 * units:
+        pytest.skip(f"{tiles} work-groups on {units} compute units: not the case this test is for")
+    _prompt_tiles_case(ops, nh, nkv, 128, 16, 0, lens, [0, 37, 0, 64])
+
+
+def _prompt_tiles_case(ops, nh, nkv, hd, page, window, lens, ctxs):
     dtype = torch.bfloat16
     g = torch.Generator().manual_seed(15)
-    lens, ctxs = [150, 37, 70, 1, 64, 300], [0, 150, 43, 99, 64, 5]
     R, T = len(lens), sum(lens)
     totals = [a + b for a, b in zip(lens, ctxs)]
     max_blocks = (max(totals) + page - 1) // page + 1

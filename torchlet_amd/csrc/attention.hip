@@ -921,20 +921,6 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     const int w_lo_min = a.window > 0 ? max(0, w_pos_min - a.window + 1) : 0;
     const int w_lo_max = a.window > 0 ? max(0, w_pos_max - a.window + 1) : 0;
 
-    // my row's query, B operand of the first product: d = 16 c + 8 h .. + 8
-    FragK qf[AT_HD / 16];
-    {
-        const bf16_t* q = (const bf16_t*)a.q + (size_t)r_token * a.q_stride + (size_t)r_head * AT_HD;
-#pragma unroll
-        for (int c = 0; c < AT_HD / 16; ++c) qf[c].u = row_ok ? *(const uint4*)(q + 16 * c + 8 * h) : make_uint4(0, 0, 0, 0);
-        // The query is waited for here, once.  Left to the compiler, the wait would stand before the first product of
-        // every step (at the loop's head it must assume the fetch of before the loop still under way), and as a wait for
-        // all fetches it would also wait for the keys and values just requested for the next step: no step would
-        // overlap with the fetch of the next.
-#pragma unroll
-        for (int c = 0; c < AT_HD / 16; ++c) asm volatile("" : "+v"(qf[c].v));
-    }
-
     const int key_hi = ctx + tok0 + ntok;
     const int key_lo = a.window > 0 ? max(0, ctx + tok0 - a.window + 1) : 0;
     // the tile's steps of ATQ_KEYS keys; with a.splits > 1 work-group blockIdx.z takes its share of them
@@ -958,7 +944,19 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
     const int blk0 = (st_first * ATQ_KEYS) >> shift;
     const int blk_n = ((key_hi - 1) >> shift) - blk0 + 1;
     if (blk_n > ATM_BT_MAX) return;            // longer than the host promised: leave the rows unwritten rather than overrun
-    for (int i = threadIdx.x; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
+    // A tile begins with three trips to memory: the block table, which the first requests need, those requests, and
+    // the query.  The table is asked for first and the query right after it, so that the query is on its way while
+    // the table arrives and the first keys and values are requested.
+    const int bt_first = (int)threadIdx.x < blk_n ? bt_g[blk0 + threadIdx.x] : 0;
+    // my row's query, B operand of the first product: d = 16 c + 8 h .. + 8
+    FragK qf[AT_HD / 16];
+    {
+        const bf16_t* q = (const bf16_t*)a.q + (size_t)r_token * a.q_stride + (size_t)r_head * AT_HD;
+#pragma unroll
+        for (int c = 0; c < AT_HD / 16; ++c) qf[c].u = row_ok ? *(const uint4*)(q + 16 * c + 8 * h) : make_uint4(0, 0, 0, 0);
+    }
+    if ((int)threadIdx.x < blk_n) bt_s[threadIdx.x] = bt_first;
+    for (int i = threadIdx.x + 256; i < blk_n; i += 256) bt_s[i] = bt_g[blk0 + i];
     __syncthreads();
     const bool any_step = st_first < st_last;  // (a share of the steps can be empty)
 
@@ -1053,6 +1051,12 @@ __global__ __launch_bounds__(256, 2) void paged_attention_prompt_kernel(AttnArgs
         asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * K_INSTR * (ATQ_STAGES - 2)) : "memory");
         __syncthreads();
     }
+    // The query is waited for here, once.  Left to the compiler, the wait would stand before the first product of
+    // every step (at the loop's head it must assume the fetch of before the loop still under way), and as a wait for
+    // all fetches it would also wait for the keys and values just requested for the next step: no step would
+    // overlap with the fetch of the next.
+#pragma unroll
+    for (int c = 0; c < AT_HD / 16; ++c) asm volatile("" : "+v"(qf[c].v));
     for (int st = st_first; st < st_last; ++st) {
         const int buf = (st - st_first) % ATQ_STAGES;
         const int st_req = min(st + ATQ_STAGES - 1, st_last - 1), buf_req = (st - st_first + ATQ_STAGES - 1) % ATQ_STAGES;

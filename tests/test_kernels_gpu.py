@@ -585,6 +585,26 @@ def test_projection_with_rotation_and_cache_write_in_its_epilogue(ops, M, nh, nk
     assert torch.equal(q_only, got[:, : nh * hd])
 
 
+@pytest.mark.parametrize("rows,hidden", [(1, 96), (3, 3584), (5, 5120), (2, 1000), (2, 20000)])
+@pytest.mark.parametrize("slabs", [1, 2, 3, 4, 5, 6, 7, 9])
+def test_add_rmsnorm_adds_any_number_of_slabs_in_their_order(ops, rows, hidden, slabs):
+    """The pending branch as float slabs of partial sums: four are fetched at a time, the last one to three as a
+    group of their own; the new residual is the sum in the slabs' order, to the bit."""
+    g = torch.Generator().manual_seed(rows * hidden + slabs)
+    res = torch.randn(rows, hidden, generator=g)
+    parts = torch.randn(slabs, rows, hidden, generator=g)
+    w = (1 + 0.1 * torch.randn(hidden, generator=g)).to(torch.bfloat16)
+    total = res.clone()
+    for p in range(slabs):
+        total = total + parts[p]                      # 32-bit, in this order
+    r = res.clone().cuda()
+    out = torch.empty(rows, hidden, dtype=torch.bfloat16, device="cuda")
+    ops.add_rmsnorm(r, parts.cuda(), w.cuda(), 1e-6, out)
+    assert torch.equal(r.cpu(), total)
+    ref = total.double() * torch.rsqrt(total.double().pow(2).mean(-1, keepdim=True) + 1e-6) * w.double()
+    torch.testing.assert_close(out.cpu().double(), ref, **_tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("H,I", [(96, 200), (3584, 1000), (1032, 300), (5120, 512), (8192, 96)])
 @pytest.mark.parametrize("pending", ["none", "row", "slabs"])
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
@@ -618,16 +638,21 @@ def test_gate_up_product_of_one_row_that_makes_its_norm_itself(ops, H, I, pendin
 
 @pytest.mark.parametrize("nh,nkv,hd,page,hidden,bias", [(28, 4, 128, 16, 3584, True), (4, 2, 16, 8, 64, False), (14, 2, 64, 16, 896, True),
                                                         (40, 8, 128, 32, 5120, True), (5, 5, 48, 16, 240, True)])
-@pytest.mark.parametrize("pending", ["none", "row", "slabs"])
+@pytest.mark.parametrize("pending", ["none", "row", "slabs", "1 slab", "3 slabs", "7 slabs", "8 slabs"])
 def test_projection_of_one_row_that_makes_its_norm_itself(ops, nh, nkv, hd, page, hidden, bias, pending):
     """``linear_rope_cache_write_normed`` against the norm's own kernel followed by the fused projection:
-    the new residual, the rotated queries and what lands in the pages, to the bit."""
+    the new residual, the rotated queries and what lands in the pages, to the bit (slabs of partial sums are
+    fetched four at a time, the last one to three as a group of their own)."""
     g = torch.Generator().manual_seed(nh + hidden)
     width = (nh + 2 * nkv) * hd
     res = torch.randn(1, hidden, generator=g).cuda()
     nw = (1 + 0.1 * torch.randn(hidden, generator=g)).to(torch.bfloat16).cuda()
-    pend = {"none": None, "row": torch.randn(1, hidden, generator=g).to(torch.bfloat16).cuda(),
-            "slabs": torch.randn(4, 1, hidden, generator=g).cuda()}[pending]
+    if pending == "none":
+        pend = None
+    elif pending == "row":
+        pend = torch.randn(1, hidden, generator=g).to(torch.bfloat16).cuda()
+    else:
+        pend = torch.randn(4 if pending == "slabs" else int(pending.split()[0]), 1, hidden, generator=g).cuda()
     w = (torch.randn(width, hidden, generator=g) / math.sqrt(hidden)).to(torch.bfloat16).cuda()
     b = torch.randn(width, generator=g).to(torch.bfloat16).cuda() if bias else None
     inv_freq = (1.0 / (1e6 ** (torch.arange(0, hd, 2).float() / hd))).cuda()

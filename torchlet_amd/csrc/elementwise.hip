@@ -97,6 +97,18 @@ template <> struct Vec4<bf16_t> {
     }
 };
 
+// r += the N slabs' four elements at src, src + stride, ...: all requested, then added in their order.
+template <int N>
+__device__ __forceinline__ void add_slabs(const float* src, size_t stride, float (&r)[4]) {
+    float p[N][4];
+#pragma unroll
+    for (int u = 0; u < N; ++u) Vec4<float>::load(src + u * stride, p[u]);
+#pragma unroll
+    for (int u = 0; u < N; ++u)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) r[v] += p[u][v];
+}
+
 template <typename T, int IT>
 __global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const void* __restrict__ pending, int parts, size_t part_stride,
                                        const void* __restrict__ weight, int weight_f32, float eps, float gain,
@@ -124,23 +136,13 @@ __global__ void add_rmsnorm_reg_kernel(float* __restrict__ residual, const void*
             if (pparts) {
                 // four slabs at a time, all requested before the first is added (a loop over a count known
                 // only at run time fetches one slab after the other: a trip to memory each); the sums are
-                // added in the order of the slabs either way
+                // added in the order of the slabs either way.  The last two or three slabs are a group as well
+                // (three slabs, as for the matrices 5120 wide, were three trips).
                 int q = 0;
-                for (; q + 4 <= parts; q += 4) {
-                    float p[4][4];
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) Vec4<float>::load(pparts + (q + u) * part_stride + i, p[u]);
-#pragma unroll
-                    for (int u = 0; u < 4; ++u)
-#pragma unroll
-                        for (int v = 0; v < 4; ++v) r[it][v] += p[u][v];
-                }
-                for (; q < parts; ++q) {
-                    float p[4];
-                    Vec4<float>::load(pparts + q * part_stride + i, p);
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) r[it][v] += p[v];
-                }
+                for (; q + 4 <= parts; q += 4) add_slabs<4>(pparts + q * part_stride + i, part_stride, r[it]);
+                if (parts - q == 3) add_slabs<3>(pparts + q * part_stride + i, part_stride, r[it]);
+                else if (parts - q == 2) add_slabs<2>(pparts + q * part_stride + i, part_stride, r[it]);
+                else if (parts - q == 1) add_slabs<1>(pparts + q * part_stride + i, part_stride, r[it]);
             }
             if (weight_f32) Vec4<float>::load((const float*)weight + i, wv[it]);
             else Vec4<bf16_t>::load((const bf16_t*)weight + i, wv[it]);
@@ -275,7 +277,15 @@ void rope_cache_write_kernel(T* __restrict__ qkv, int row_stride, int q_heads, i
 #pragma unroll
             for (int u = 0; u < 4; ++u) sum += v[u];
         }
-        for (; p < num_parts; ++p) sum += src[(size_t)p * part_stride];
+        if (num_parts - p == 3) {                  // (and the last two or three)
+            const float v0 = src[(size_t)p * part_stride], v1 = src[(size_t)(p + 1) * part_stride], v2 = src[(size_t)(p + 2) * part_stride];
+            sum += v0; sum += v1; sum += v2;
+        } else if (num_parts - p == 2) {
+            const float v0 = src[(size_t)p * part_stride], v1 = src[(size_t)(p + 1) * part_stride];
+            sum += v0; sum += v1;
+        } else if (num_parts - p == 1) {
+            sum += src[(size_t)p * part_stride];
+        }
         return sum;
     };
     if (head >= q_heads + kv_heads) {      // value head: [head_dim, page] inside the page

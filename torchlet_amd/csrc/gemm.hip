@@ -544,6 +544,18 @@ __device__ __forceinline__ void store8(bf16_t* p, const float* v) {
     *(uint4*)p = t;
 }
 
+// r += the N slabs' eight elements at src, src + stride, ...: all requested, then added in their order.
+template <int N>
+__device__ __forceinline__ void add_slabs8(const float* src, size_t stride, float (&r)[8]) {
+    float p[N][8];
+#pragma unroll
+    for (int u = 0; u < N; ++u) load8(src + u * stride, p[u]);
+#pragma unroll
+    for (int u = 0; u < N; ++u)
+#pragma unroll
+        for (int v = 0; v < 8; ++v) r[v] += p[u][v];
+}
+
 // NF (one row, with XL): x is not read but made here, as the norm of the residual stream would make it:
 // r = residual + pending (bfloat16, or float slabs of partial sums), x = r * rsqrt(mean(r^2) + eps) * weight, all
 // in 32-bit and rounded once; the first work-group writes r out as the new residual (to another place than it
@@ -666,11 +678,26 @@ __global__ __launch_bounds__(KS * 64) void gemm_skinny_kernel(const bf16_t* __re
 #pragma unroll
                 for (int v = 0; v < 8; ++v) r[c][v] += p[v];
             }
-            for (int q = 0; q < na.parts; ++q) {
-                float p[8];
-                load8((const float*)na.pending + q * na.part_stride + i, p);
+            const float* slab = (const float*)na.pending + i;
+            if constexpr (RP) {
+                // The query/key/value projection follows the down projection, whose K is split many ways: four slabs
+                // at a time, all requested before the first is added, in their order (one after the other, the eight
+                // slabs of the 7B's down projection were eight trips to memory before the first weight was used); the
+                // last two or three are a group as well.
+                int q = 0;
+                for (; q + 4 <= na.parts; q += 4) add_slabs8<4>(slab + q * na.part_stride, na.part_stride, r[c]);
+                if (na.parts - q == 3) add_slabs8<3>(slab + q * na.part_stride, na.part_stride, r[c]);
+                else if (na.parts - q == 2) add_slabs8<2>(slab + q * na.part_stride, na.part_stride, r[c]);
+                else if (na.parts - q == 1) add_slabs8<1>(slab + q * na.part_stride, na.part_stride, r[c]);
+            } else {
+                // (the fused gate follows the output projection, one slab or few: the registers of a group would cost
+                // its work-groups of sixteen waves the second one on a compute unit)
+                for (int q = 0; q < na.parts; ++q) {
+                    float p[8];
+                    load8(slab + q * na.part_stride, p);
 #pragma unroll
-                for (int v = 0; v < 8; ++v) r[c][v] += p[v];
+                    for (int v = 0; v < 8; ++v) r[c][v] += p[v];
+                }
             }
             if ((int)threadIdx.x + c * KS * 64 < pieces) {
 #pragma unroll
